@@ -1,0 +1,153 @@
+/*
+ * rafhip_optim.h -- C ABI of the gfx950 (MI355X) fused optimizer-step kernels that stand in for
+ * awslabs/raf's `raf.op.sgd` and `raf.op.lans` backends.
+ *
+ * Plain C: raw device pointers, element counts, a HIP stream passed as void*.  No C++ or torch
+ * types cross this boundary.  Every function returns a rafhip_status (0 = success) unless noted;
+ * the text of the last failure on the calling thread is available from rafhip_last_error().
+ * No function throws, and none of the *step* functions allocates or frees device memory.
+ *
+ * Reference interfaces replaced (paths relative to the reference tree):
+ *   rafhip_sgd_f32          the TVM-built packed function behind `raf.op.tvm.sgd`:
+ *                           python/raf/_tvm_op/sgd.py:13-30, registered at
+ *                           src/op/dialect/tvm/optimizer.cc:44-45 and invoked with
+ *                           [x, dx, v, v1, x1] at src/op/dialect/tvm/tvm_utils.cc:92-133.
+ *   rafhip_lans_*           multi_tensor_lans_cuda<float>(...) declared at
+ *                           src/op/dialect/cuda/kernels/kernel_util.cuh:25-34 and called from
+ *                           LansImpl::Execute, src/op/dialect/cuda/lans.cc:124-130; the plan object
+ *                           takes the role of LansImpl's constructor state (lans.cc:27-83) and
+ *                           rafhip_lans_workspace_bytes that of its RequestWorkspace calls
+ *                           (lans.cc:66-77).
+ */
+#ifndef RAFHIP_OPTIM_H_
+#define RAFHIP_OPTIM_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RAFHIP_ABI_VERSION 1
+
+typedef enum rafhip_status {
+  RAFHIP_OK = 0,
+  RAFHIP_ERR_INVALID_ARG = 1, /* null pointer, negative size, bad enum, n % 4 != 0 ...        */
+  RAFHIP_ERR_UNSUPPORTED = 2, /* dtype or size the kernels do not handle                       */
+  RAFHIP_ERR_WORKSPACE = 3,   /* workspace missing, too small or misaligned                    */
+  RAFHIP_ERR_HIP = 4,         /* a HIP runtime call failed; message carries hipGetErrorString  */
+  RAFHIP_ERR_NO_DEVICE = 5    /* no usable gfx950 device in this process                       */
+} rafhip_status;
+
+typedef enum rafhip_dtype {
+  RAFHIP_F32 = 0,
+  RAFHIP_F16 = 1 /* IEEE binary16; accepted for LANS gradients only */
+} rafhip_dtype;
+
+/* ABI version of the loaded library (== RAFHIP_ABI_VERSION it was built with). */
+int rafhip_abi_version(void);
+
+/* Message of the last failing call on this thread ("" if none).  Never NULL. */
+const char* rafhip_last_error(void);
+
+/* Number of HIP devices visible (0 on a host without a GPU; never fails). */
+int rafhip_device_count(void);
+
+/* ------------------------------------------------------------------------------------------ SGD
+ * Momentum SGD step of `raf.op.sgd` (python/raf/_tvm_op/sgd.py:16-30):
+ *     v_out = fl32(fl32(mu32 * v) + dx)        x_out = fl32(x - fl32(lr32 * v_out))
+ * with mu32 = (float)mu, lr32 = (float)learning_rate: four separately rounded fp32 operations,
+ * never fused, so the result is bit-identical to the reference's CPU (LLVM) lowering.
+ * Out of place like the reference op (src/op/declare/optimizer.cc:22-44); v_out may alias v and
+ * x_out may alias x (element i is read before it is written by the same lane).
+ * n == 0 is a successful no-op.  All pointers are device pointers of n floats.
+ */
+int rafhip_sgd_f32(const float* x, const float* dx, const float* v, float* v_out, float* x_out,
+                   int64_t n, double learning_rate, double mu, void* stream);
+
+/* ----------------------------------------------------------------------------------------- LANS
+ * Hyper-parameters: the non-tensor schema fields of `raf.op.lans`
+ * (scripts/src_codegen/def_schema.py:685-693) in schema order, fp32 like the schema's `float`.
+ */
+typedef struct rafhip_lans_hparams {
+  float learning_rate;
+  float beta1;
+  float beta2;
+  float eps;
+  int32_t bias_correction; /* 1: bc_k = 1 - beta_k^step (lans.cc:102-105); else bc_k = 1      */
+  float weight_decay;
+  int32_t grad_averaging;  /* 1: beta3 = 1 - beta1 (lans.cc:107-109); else beta3 = 1          */
+  int32_t mode;            /* 1: decoupled weight decay; 0: L2 on the scaled gradient          */
+  int32_t normalize_grad;  /* bool: divide g by (||g|| + eps) when ||g|| != 0                  */
+  float grad_unscale;      /* extension: g is multiplied by this first (loss-scale undo); 1.0  */
+} rafhip_lans_hparams;
+
+/* Defaults of raf.optim.LANS (python/raf/optim/lans.py:44-55) with grad_unscale = 1. */
+void rafhip_lans_default_hparams(rafhip_lans_hparams* hp);
+
+/*
+ * A plan fixes what LansImpl's constructor fixes: the number of tensors and their element counts
+ * (lans.cc:51-72), plus the gradient dtype.  Creation builds the device-side chunk table (one
+ * hipMalloc + upload); the step calls then launch a fixed five-kernel sequence without touching
+ * the allocator.  A plan belongs to the device that was current at creation and is not
+ * thread-safe: one step at a time per plan.
+ */
+typedef struct rafhip_lans_plan rafhip_lans_plan;
+
+/* Pure host arithmetic, usable without a GPU: how many chunks a tensor list is cut into and how
+ * many workspace bytes a step over it needs (what LansImpl computes at lans.cc:66-77).  Either
+ * output pointer may be NULL. */
+int rafhip_lans_query_layout(int32_t n_tensors, const int64_t* numel, int64_t* n_chunks_out,
+                             int64_t* workspace_bytes_out);
+
+/* numel[i] >= 0 (zero-sized tensors are allowed and untouched); n_tensors >= 0. */
+int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t grad_dtype,
+                            rafhip_lans_plan** out_plan);
+int rafhip_lans_plan_destroy(rafhip_lans_plan* plan);
+
+/* Bytes of caller-provided scratch a step needs (partial sums + per-tensor norms); 256-byte
+ * alignment required.  Returns a negative value on a NULL plan. */
+int64_t rafhip_lans_workspace_bytes(const rafhip_lans_plan* plan);
+int32_t rafhip_lans_plan_num_tensors(const rafhip_lans_plan* plan);
+int64_t rafhip_lans_plan_num_chunks(const rafhip_lans_plan* plan);
+int64_t rafhip_lans_plan_total_elements(const rafhip_lans_plan* plan);
+
+/*
+ * One LANS step, in place on w/m/v; g is read-only (the reference overwrites it with an
+ * intermediate, multi_tensor_lans.cu:314, which no caller reads).
+ *
+ *   g, w, m, v   host arrays of n_tensors device pointers (the four quarters of the reference's
+ *                tensor_list, python/raf/optim/lans.py:89).  g[i] has the plan's gradient dtype.
+ *   step_dev     device pointer to the 0-d fp32 step tensor (lans.cc:92-99), read on the device
+ *                so the call never blocks the host; or NULL to use step_host.
+ *   workspace    device scratch of at least rafhip_lans_workspace_bytes(plan); contents need not
+ *                be preserved between calls and need no initialisation.
+ *   stream       hipStream_t (NULL = the default stream).  All work is enqueued on it.
+ *
+ * Arithmetic: scalars are the fp32 schema values; everything per element and every norm is
+ * evaluated in float64 and rounded once to fp32 on store.
+ */
+int rafhip_lans_step(rafhip_lans_plan* plan, const void* const* g, float* const* w,
+                     float* const* m, float* const* v, const float* step_dev, int32_t step_host,
+                     const rafhip_lans_hparams* hp, void* workspace, int64_t workspace_bytes,
+                     void* stream);
+
+/* Copies the per-tensor norms left in the workspace by the last step on `stream`
+ * (4 doubles per tensor: ||g||, ||w||, ||u_m||, ||u_g||) to host memory; synchronises `stream`. */
+int rafhip_lans_read_norms(const rafhip_lans_plan* plan, const void* workspace, double* host_out,
+                           void* stream);
+
+/*
+ * Optional per-kernel timing.  slots > 0 makes each following step record HIP events around its
+ * five kernels on the step's stream into slot (step_index % slots); slots == 0 turns it off.
+ * rafhip_lans_timing_read waits for that slot's last event and returns the five durations in
+ * milliseconds: [0] norms of g,w  [1] finish  [2] norms of u_m,u_g  [3] finish  [4] apply.
+ */
+int rafhip_lans_timing_enable(rafhip_lans_plan* plan, int32_t slots);
+int rafhip_lans_timing_read(rafhip_lans_plan* plan, int32_t slot, float* ms_out5);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RAFHIP_OPTIM_H_ */

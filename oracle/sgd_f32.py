@@ -1,0 +1,49 @@
+"""CPU oracle for ``raf.op.sgd`` -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+
+The reference computes the momentum-SGD step with a two-stage TVM tensor
+expression (python/raf/_tvm_op/sgd.py:13-30):
+
+    v1 = mu * v0 + dx            (:21-24)
+    x1 = x0 - learning_rate * v1 (:26-29)
+
+where ``mu`` and ``learning_rate`` are the schema's doubles
+(scripts/src_codegen/def_schema.py:675-676) turned into constants of the
+tensor dtype by ``tir.const(..., dtype=x0.dtype)`` (sgd.py:18-19), and the
+outputs come back as the tuple ``(v1, x1)`` (src/op/declare/optimizer.cc:34-42).
+The CPU build target is plain ``llvm`` with no ``-mcpu``
+(include/raf/device.h:97-104), i.e. generic x86-64 without FMA, so each of the
+four fp32 operations is rounded on its own:
+
+    t  = fl32(mu32 * v0)     v1 = fl32(t + dx)
+    s  = fl32(lr32 * v1)     x1 = fl32(x0 - s)
+
+The arithmetic itself lives in TVM (dmlc/tvm, an un-vendored submodule with no
+pinned revision), which is absent here, so the no-contraction property cannot
+be confirmed by running the reference; it is pinned instead
+(tests/test_oracle_sgd.py) by exact rational arithmetic with explicit
+roundings, vectors on which a fused multiply-add gives a different bit
+pattern, the reference's own float64 closed-form test
+(tests/python/op/tvm/test_tvm_loss.py:158-176) and ``torch.optim.SGD``.
+
+Only tests, the smoke check and the benchmark's CPU baseline leg may import
+this module.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+
+def sgd_step(x0, dx, v0, learning_rate: float, mu: float):
+    """Returns ``(v1, x1)`` as new fp32 arrays; inputs are not modified."""
+    x0 = np.asarray(x0, dtype=np.float32)
+    dx = np.asarray(dx, dtype=np.float32)
+    v0 = np.asarray(v0, dtype=np.float32)
+    assert x0.shape == dx.shape == v0.shape  # declare/optimizer.cc:29-33
+    lr32 = np.float32(learning_rate)
+    mu32 = np.float32(mu)
+    with np.errstate(all="ignore"):
+        t = np.multiply(mu32, v0, dtype=np.float32)
+        v1 = np.add(t, dx, dtype=np.float32)
+        s = np.multiply(lr32, v1, dtype=np.float32)
+        x1 = np.subtract(x0, s, dtype=np.float32)
+    return v1, x1

@@ -1,0 +1,109 @@
+"""ctypes bindings of the C ABI declared in include/rafhip_optim.h.
+
+The libraries are built in-tree by ``python -m raf_amd.build`` (hipcc, gfx950).  Loading fails
+loudly if they are missing: there is no CPU or eager fallback anywhere in this package.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import (POINTER, Structure, c_char_p, c_double, c_float, c_int, c_int32, c_int64,
+                    c_void_p)
+from pathlib import Path
+
+LIB_DIR = Path(__file__).resolve().parent / "lib"
+OPTIM_LIB = LIB_DIR / "libraf_hip_optim.so"
+DIALECT_LIB = LIB_DIR / "libraf_hip_dialect.so"
+
+RAFHIP_OK = 0
+RAFHIP_ERR_INVALID_ARG = 1
+RAFHIP_ERR_UNSUPPORTED = 2
+RAFHIP_ERR_WORKSPACE = 3
+RAFHIP_ERR_HIP = 4
+RAFHIP_ERR_NO_DEVICE = 5
+
+RAFHIP_F32 = 0
+RAFHIP_F16 = 1
+
+
+class RafHipError(RuntimeError):
+    """A C-ABI call returned a non-zero status."""
+
+    def __init__(self, status: int, message: str):
+        super().__init__(f"rafhip status {status}: {message}")
+        self.status = status
+        self.message = message
+
+
+class LansHParams(Structure):
+    """``rafhip_lans_hparams``: schema order of ``raf.op.lans``
+    (scripts/src_codegen/def_schema.py:685-693 in the reference) plus ``grad_unscale``."""
+
+    _fields_ = [
+        ("learning_rate", c_float),
+        ("beta1", c_float),
+        ("beta2", c_float),
+        ("eps", c_float),
+        ("bias_correction", c_int32),
+        ("weight_decay", c_float),
+        ("grad_averaging", c_int32),
+        ("mode", c_int32),
+        ("normalize_grad", c_int32),
+        ("grad_unscale", c_float),
+    ]
+
+
+# name -> (restype, argtypes); every symbol the header declares.
+OPTIM_SYMBOLS = {
+    "rafhip_abi_version": (c_int, []),
+    "rafhip_last_error": (c_char_p, []),
+    "rafhip_device_count": (c_int, []),
+    "rafhip_sgd_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_double,
+                               c_double, c_void_p]),
+    "rafhip_lans_default_hparams": (None, [POINTER(LansHParams)]),
+    "rafhip_lans_query_layout": (c_int, [c_int32, POINTER(c_int64), POINTER(c_int64),
+                                         POINTER(c_int64)]),
+    "rafhip_lans_plan_create": (c_int, [c_int32, POINTER(c_int64), c_int32, POINTER(c_void_p)]),
+    "rafhip_lans_plan_destroy": (c_int, [c_void_p]),
+    "rafhip_lans_workspace_bytes": (c_int64, [c_void_p]),
+    "rafhip_lans_plan_num_tensors": (c_int32, [c_void_p]),
+    "rafhip_lans_plan_num_chunks": (c_int64, [c_void_p]),
+    "rafhip_lans_plan_total_elements": (c_int64, [c_void_p]),
+    "rafhip_lans_step": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
+                                 POINTER(c_void_p), c_void_p, c_int32, POINTER(LansHParams),
+                                 c_void_p, c_int64, c_void_p]),
+    "rafhip_lans_read_norms": (c_int, [c_void_p, c_void_p, POINTER(c_double), c_void_p]),
+    "rafhip_lans_timing_enable": (c_int, [c_void_p, c_int32]),
+    "rafhip_lans_timing_read": (c_int, [c_void_p, c_int32, POINTER(c_float)]),
+}
+
+_optim = None
+
+
+def _bind(lib, table):
+    for name, (restype, argtypes) in table.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        fn.restype = restype
+        fn.argtypes = argtypes
+
+
+def optim():
+    """The kernel library, loaded once."""
+    global _optim
+    if _optim is None:
+        if not OPTIM_LIB.exists():
+            raise RuntimeError(
+                f"{OPTIM_LIB} is missing: build it with `python -m raf_amd.build` "
+                "(hipcc --offload-arch=gfx950); there is no fallback path")
+        lib = ctypes.CDLL(str(OPTIM_LIB), mode=ctypes.RTLD_GLOBAL)
+        _bind(lib, OPTIM_SYMBOLS)
+        _optim = lib
+    return _optim
+
+
+def last_error() -> str:
+    return optim().rafhip_last_error().decode("utf-8", "replace")
+
+
+def check(status: int) -> None:
+    if status != RAFHIP_OK:
+        raise RafHipError(status, last_error())

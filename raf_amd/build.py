@@ -1,0 +1,99 @@
+"""Builds the native libraries in-tree with hipcc for gfx950.
+
+    python -m raf_amd.build            # build everything
+    python -m raf_amd.build --check    # exit 1 if a library is missing or older than its sources
+
+Two shared objects land in raf_amd/lib/:
+  libraf_hip_optim.so    HIP kernels + the C ABI declared in include/rafhip_optim.h
+  libraf_hip_dialect.so  C++ host layer: OpEnv / dialect registry mirror + the `hip` dialect ops
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent.parent
+CSRC = ROOT / "raf_amd" / "csrc"
+LIB = ROOT / "raf_amd" / "lib"
+INCLUDE = ROOT / "include"
+
+ARCH = "gfx950"
+# -packed-fp32-ops is switched off on purpose: the compiler must not form v_pk_*_f32.
+HIP_FLAGS = [
+    f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-command-line-argument",
+]
+
+OPTIM_SOURCES = ["status.hip", "sgd.hip", "lans_kernels.hip", "lans_plan.hip"]
+DIALECT_SOURCES = ["dialect/registry.cc", "dialect/hip_dialect.cc", "dialect/c_api.cc"]
+
+
+def hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; the HIP libraries cannot be built")
+    return exe
+
+
+def _run(cmd):
+    print("+", " ".join(str(c) for c in cmd), flush=True)
+    subprocess.run([str(c) for c in cmd], check=True, cwd=ROOT)
+
+
+def optim_lib() -> Path:
+    return LIB / "libraf_hip_optim.so"
+
+
+def dialect_lib() -> Path:
+    return LIB / "libraf_hip_dialect.so"
+
+
+def build_optim() -> Path:
+    LIB.mkdir(parents=True, exist_ok=True)
+    out = optim_lib()
+    srcs = [CSRC / s for s in OPTIM_SOURCES]
+    _run([hipcc(), *HIP_FLAGS, "-shared", f"-I{INCLUDE}", f"-I{CSRC}", "-o", out, *srcs])
+    return out
+
+
+def build_dialect() -> Path:
+    LIB.mkdir(parents=True, exist_ok=True)
+    out = dialect_lib()
+    srcs = [CSRC / s for s in DIALECT_SOURCES]
+    # Host-only C++ that calls the C ABI; hipcc is used as the C++ driver so hip_runtime_api.h
+    # (stream type) resolves the same way as in the kernels' translation units.
+    _run([hipcc(), "-x", "c++", "-O2", "-std=c++17", "-fPIC", "-Wall", "-shared",
+          "-D__HIP_PLATFORM_AMD__", f"-I{INCLUDE}", f"-I{CSRC}", "-I/opt/rocm/include",
+          "-o", out, *srcs, f"-L{LIB}", "-lraf_hip_optim", "-Wl,-rpath,$ORIGIN"])
+    return out
+
+
+def build_all() -> None:
+    build_optim()
+    build_dialect()
+
+
+def stale() -> list:
+    """Libraries that are missing or older than any of their sources."""
+    bad = []
+    deps = {
+        optim_lib(): [CSRC / s for s in OPTIM_SOURCES] + list(CSRC.glob("*.h")) + list(INCLUDE.glob("*.h")),
+        dialect_lib(): [CSRC / s for s in DIALECT_SOURCES] + list((CSRC / "dialect").glob("*.h")) + list(INCLUDE.glob("*.h")),
+    }
+    for lib, srcs in deps.items():
+        if not lib.exists() or any(s.stat().st_mtime > lib.stat().st_mtime for s in srcs if s.exists()):
+            bad.append(lib)
+    return bad
+
+
+if __name__ == "__main__":
+    if "--check" in sys.argv:
+        bad = stale()
+        for b in bad:
+            print("stale or missing:", b)
+        sys.exit(1 if bad else 0)
+    build_all()

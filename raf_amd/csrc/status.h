@@ -1,0 +1,24 @@
+// Error reporting shared by the C-ABI entry points: a status code plus a thread-local message.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "rafhip_optim.h"
+
+namespace rafhip {
+
+// Stores a printf-style message for rafhip_last_error() and returns `code`.
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+void clear_error();
+
+}  // namespace rafhip
+
+#define RAFHIP_HIP_TRY(expr)                                                                \
+  do {                                                                                      \
+    hipError_t _e = (expr);                                                                 \
+    if (_e != hipSuccess)                                                                   \
+      return ::rafhip::fail(RAFHIP_ERR_HIP, "%s failed: %s (%s:%d)", #expr,                 \
+                            hipGetErrorString(_e), __FILE__, __LINE__);                     \
+  } while (0)

@@ -1,0 +1,148 @@
+"""Thin Python handles over the C ABI, operating on torch tensors that live on a ROCm device.
+
+torch is only the owner of device memory and of the current HIP stream here; every computation is
+done by the HIP kernels behind ``include/rafhip_optim.h``.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_double, c_float, c_int64, c_void_p
+from typing import List, Optional, Sequence
+
+import torch
+
+from . import _lib
+from ._lib import LansHParams, RAFHIP_F16, RAFHIP_F32, check
+
+
+def _current_stream(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _require_gpu_f32(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise ValueError(f"{name}: expected a tensor on the GPU, got device {t.device}")
+    if t.dtype != torch.float32:
+        raise TypeError(f"{name}: expected float32, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name}: expected a contiguous tensor")
+
+
+def sgd_f32(x: torch.Tensor, dx: torch.Tensor, v: torch.Tensor, learning_rate: float, mu: float,
+            v_out: Optional[torch.Tensor] = None, x_out: Optional[torch.Tensor] = None):
+    """``rafhip_sgd_f32`` on torch tensors; returns ``(v1, x1)`` (new tensors unless given)."""
+    for t, name in ((x, "x"), (dx, "dx"), (v, "v")):
+        _require_gpu_f32(t, name)
+    if not (x.shape == dx.shape == v.shape):
+        raise ValueError(f"sgd: shapes differ: x{tuple(x.shape)} dx{tuple(dx.shape)} v{tuple(v.shape)}")
+    v1 = torch.empty_like(dx) if v_out is None else v_out
+    x1 = torch.empty_like(dx) if x_out is None else x_out
+    check(_lib.optim().rafhip_sgd_f32(x.data_ptr(), dx.data_ptr(), v.data_ptr(), v1.data_ptr(),
+                                      x1.data_ptr(), x.numel(), float(learning_rate), float(mu),
+                                      _current_stream(x.device)))
+    return v1, x1
+
+
+def make_hparams(learning_rate=1e-3, beta1=0.9, beta2=0.999, eps=1e-6, bias_correction=1,
+                 weight_decay=0.01, grad_averaging=1, mode=1, normalize_grad=True,
+                 grad_unscale=1.0) -> LansHParams:
+    """Python numbers -> the fp32/int schema fields (bools become 0/1 like the reference's FFI)."""
+    return LansHParams(float(learning_rate), float(beta1), float(beta2), float(eps),
+                       int(bias_correction), float(weight_decay), int(grad_averaging), int(mode),
+                       int(bool(normalize_grad)), float(grad_unscale))
+
+
+def query_layout(numels: Sequence[int]):
+    """(n_chunks, workspace_bytes) for a tensor list; host arithmetic only, needs no GPU."""
+    n = len(numels)
+    arr = (c_int64 * max(n, 1))(*numels)
+    chunks, ws = c_int64(0), c_int64(0)
+    check(_lib.optim().rafhip_lans_query_layout(n, arr, ctypes.byref(chunks), ctypes.byref(ws)))
+    return chunks.value, ws.value
+
+
+class LansPlan:
+    """Owns a ``rafhip_lans_plan`` and a workspace tensor sized for it."""
+
+    def __init__(self, numels: Sequence[int], grad_dtype=torch.float32, device="cuda:0"):
+        self._h = c_void_p(None)
+        self.lib = _lib.optim()
+        self.device = torch.device(device)
+        self.numels = [int(n) for n in numels]
+        self.n = len(self.numels)
+        if grad_dtype == torch.float32:
+            code = RAFHIP_F32
+        elif grad_dtype == torch.float16:
+            code = RAFHIP_F16
+        else:
+            raise TypeError(f"LANS gradients must be float32 or float16, got {grad_dtype}")
+        self.grad_dtype = grad_dtype
+        arr = (c_int64 * max(self.n, 1))(*self.numels)
+        with torch.cuda.device(self.device):
+            check(self.lib.rafhip_lans_plan_create(self.n, arr, code, ctypes.byref(self._h)))
+        self.workspace_bytes = self.lib.rafhip_lans_workspace_bytes(self._h)
+        self.n_chunks = self.lib.rafhip_lans_plan_num_chunks(self._h)
+        self.total_elements = self.lib.rafhip_lans_plan_total_elements(self._h)
+        self.workspace = torch.empty(max(self.workspace_bytes, 256), dtype=torch.uint8,
+                                     device=self.device)
+
+    def close(self):
+        if self._h:
+            self.lib.rafhip_lans_plan_destroy(self._h)
+            self._h = c_void_p(None)
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:  # interpreter shutdown
+            pass
+
+    def _ptrs(self, tensors: Sequence[torch.Tensor], dtype, what: str):
+        if len(tensors) != self.n:
+            raise ValueError(f"{what}: expected {self.n} tensors, got {len(tensors)}")
+        arr = (c_void_p * max(self.n, 1))()
+        for i, t in enumerate(tensors):
+            if not t.is_cuda or t.dtype != dtype or not t.is_contiguous():
+                raise TypeError(f"{what}[{i}]: need a contiguous {dtype} GPU tensor, "
+                                f"got {t.dtype} on {t.device}")
+            if t.numel() != self.numels[i]:
+                raise ValueError(f"{what}[{i}]: {t.numel()} elements, plan has {self.numels[i]}")
+            arr[i] = t.data_ptr()
+        return arr
+
+    def step(self, g: Sequence[torch.Tensor], w: Sequence[torch.Tensor],
+             m: Sequence[torch.Tensor], v: Sequence[torch.Tensor], step, hp: LansHParams,
+             workspace: Optional[torch.Tensor] = None):
+        """``step`` is a 0-d fp32 GPU tensor (read on the device) or a Python int."""
+        ws = self.workspace if workspace is None else workspace
+        gp = self._ptrs(g, self.grad_dtype, "g")
+        wp = self._ptrs(w, torch.float32, "w")
+        mp = self._ptrs(m, torch.float32, "m")
+        vp = self._ptrs(v, torch.float32, "v")
+        if isinstance(step, torch.Tensor):
+            if step.dtype != torch.float32 or step.numel() != 1 or not step.is_cuda:
+                raise TypeError("step tensor must be a 0-d float32 GPU tensor")
+            step_dev, step_host = step.data_ptr(), 0
+        else:
+            step_dev, step_host = None, int(step)
+        check(self.lib.rafhip_lans_step(self._h, gp, wp, mp, vp, step_dev, step_host,
+                                        ctypes.byref(hp), ws.data_ptr(), ws.numel(),
+                                        _current_stream(self.device)))
+
+    def read_norms(self, workspace: Optional[torch.Tensor] = None):
+        """[n, 4] float64: ||g||, ||w||, ||u_m||, ||u_g|| of the last step."""
+        import numpy as np
+
+        ws = self.workspace if workspace is None else workspace
+        out = (c_double * max(4 * self.n, 1))()
+        check(self.lib.rafhip_lans_read_norms(self._h, ws.data_ptr(), out,
+                                              _current_stream(self.device)))
+        return np.array(out[:4 * self.n], dtype=np.float64).reshape(self.n, 4)
+
+    def timing_enable(self, slots: int):
+        check(self.lib.rafhip_lans_timing_enable(self._h, int(slots)))
+
+    def timing_read(self, slot: int) -> List[float]:
+        out = (c_float * 5)()
+        check(self.lib.rafhip_lans_timing_read(self._h, int(slot), out))
+        return list(out)
