@@ -1,0 +1,80 @@
+/*
+ * rafhip_dialect.h -- C entry points into the C++ host layer (OpEnv / dialect registry mirror and
+ * the `hip` dialect ops).  They exist so that a non-C++ caller (the Python mirror of RAF's
+ * frontend, ctypes) can drive an operator the way RAF's executors do:
+ *
+ *     make   = declare + dispatch + OpEnv construction   (src/impl/interpreter.cc:247-270,
+ *                                                          src/impl/op.cc:127-180)
+ *     execute = bind workspaces, set the stream, OpEnv::Execute(inputs, output), unbind
+ *                                                         (src/impl/vm/vm.cc:818-855, :1099-1111)
+ *
+ * Tensors cross as rafhip_tensor_desc (the DLTensor fields the ops read).  Every function returns
+ * 0 on success; on failure the message (a raf::Error text or a kernel-library error) is available
+ * from rafhip_raf_last_error() on the same thread.
+ */
+#ifndef RAFHIP_DIALECT_H_
+#define RAFHIP_DIALECT_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct rafhip_tensor_desc {
+  void* data;
+  int32_t device_type; /* 1 cpu, 2 cuda, 10 rocm (include/raf/device.h:37-50) */
+  int32_t device_id;
+  int32_t dtype_code;  /* DLPack: 0 int, 1 uint, 2 float */
+  int32_t dtype_bits;
+  int32_t ndim;
+  const int64_t* shape;
+} rafhip_tensor_desc;
+
+typedef struct rafhip_raf_env rafhip_raf_env; /* an OpEnv made by dispatch */
+
+const char* rafhip_raf_last_error(void);
+
+/* "dialect:dialect_op:plevel" entries joined by ';' in dispatch order for a base op on a device
+ * type, honouring the current preference; truncated to buflen. */
+int rafhip_raf_dispatch_list(const char* base_op, int32_t device_type, char* buf, int32_t buflen);
+
+/* Scoped dialect preference for this thread (the reference tests' with_dialect): names joined by
+ * ','; pass NULL or "" to clear. */
+int rafhip_raf_set_dialect_preference(const char* dialects_csv);
+
+/* hip-dialect extension: factor applied to LANS gradients, captured by the next LANS make. */
+int rafhip_raf_set_lans_grad_unscale(float factor);
+
+/* raf.op.sgd(x, dx, v, learning_rate, mu) -> (v1, x1); python/raf/optim/sgd.py:56 */
+int rafhip_raf_sgd_make(const rafhip_tensor_desc* x, const rafhip_tensor_desc* dx,
+                        const rafhip_tensor_desc* v, double learning_rate, double mu,
+                        rafhip_raf_env** env_out);
+int rafhip_raf_sgd_execute(rafhip_raf_env* env, const rafhip_tensor_desc* x,
+                           const rafhip_tensor_desc* dx, const rafhip_tensor_desc* v,
+                           const rafhip_tensor_desc* v1, const rafhip_tensor_desc* x1,
+                           void* stream);
+
+/* raf.op.lans(tensor_list, step, learning_rate, beta1, beta2, eps, bias_correction, weight_decay,
+ * grad_averaging, mode, normalize_grad); python/raf/optim/lans.py:90-102.  tensor_list holds 4n
+ * descriptors ordered g..., w..., m..., v... */
+int rafhip_raf_lans_make(int32_t list_len, const rafhip_tensor_desc* tensor_list,
+                         const rafhip_tensor_desc* step, float learning_rate, float beta1,
+                         float beta2, float eps, int32_t bias_correction, float weight_decay,
+                         int32_t grad_averaging, int32_t mode, int32_t normalize_grad,
+                         rafhip_raf_env** env_out);
+int rafhip_raf_lans_execute(rafhip_raf_env* env, int32_t list_len,
+                            const rafhip_tensor_desc* tensor_list, const rafhip_tensor_desc* step,
+                            void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Total bytes of the OpEnv's workspace requests (each rounded up to 256). */
+int64_t rafhip_raf_env_workspace_bytes(const rafhip_raf_env* env);
+/* OpEnv::name() and the dialect op the dispatcher picked; pointers stay valid until destroy. */
+const char* rafhip_raf_env_name(const rafhip_raf_env* env);
+const char* rafhip_raf_env_op(const rafhip_raf_env* env);
+int rafhip_raf_env_destroy(rafhip_raf_env* env);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RAFHIP_DIALECT_H_ */

@@ -76,7 +76,41 @@ OPTIM_SYMBOLS = {
     "rafhip_lans_timing_read": (c_int, [c_void_p, c_int32, POINTER(c_float)]),
 }
 
+class TensorDesc(Structure):
+    """``rafhip_tensor_desc`` of include/rafhip_dialect.h."""
+
+    _fields_ = [
+        ("data", c_void_p),
+        ("device_type", c_int32),
+        ("device_id", c_int32),
+        ("dtype_code", c_int32),
+        ("dtype_bits", c_int32),
+        ("ndim", c_int32),
+        ("shape", POINTER(c_int64)),
+    ]
+
+
+DIALECT_SYMBOLS = {
+    "rafhip_raf_last_error": (c_char_p, []),
+    "rafhip_raf_dispatch_list": (c_int, [c_char_p, c_int32, c_char_p, c_int32]),
+    "rafhip_raf_set_dialect_preference": (c_int, [c_char_p]),
+    "rafhip_raf_set_lans_grad_unscale": (c_int, [c_float]),
+    "rafhip_raf_sgd_make": (c_int, [POINTER(TensorDesc), POINTER(TensorDesc), POINTER(TensorDesc),
+                                    c_double, c_double, POINTER(c_void_p)]),
+    "rafhip_raf_sgd_execute": (c_int, [c_void_p] + [POINTER(TensorDesc)] * 5 + [c_void_p]),
+    "rafhip_raf_lans_make": (c_int, [c_int32, POINTER(TensorDesc), POINTER(TensorDesc), c_float,
+                                     c_float, c_float, c_float, c_int32, c_float, c_int32, c_int32,
+                                     c_int32, POINTER(c_void_p)]),
+    "rafhip_raf_lans_execute": (c_int, [c_void_p, c_int32, POINTER(TensorDesc),
+                                        POINTER(TensorDesc), c_void_p, c_int64, c_void_p]),
+    "rafhip_raf_env_workspace_bytes": (c_int64, [c_void_p]),
+    "rafhip_raf_env_name": (c_char_p, [c_void_p]),
+    "rafhip_raf_env_op": (c_char_p, [c_void_p]),
+    "rafhip_raf_env_destroy": (c_int, [c_void_p]),
+}
+
 _optim = None
+_dialect = None
 
 
 def _bind(lib, table):
@@ -107,3 +141,26 @@ def last_error() -> str:
 def check(status: int) -> None:
     if status != RAFHIP_OK:
         raise RafHipError(status, last_error())
+
+
+def dialect():
+    """The C++ host layer (OpEnv / dialect registry mirror + the `hip` dialect), loaded once."""
+    global _dialect
+    if _dialect is None:
+        optim()  # dependency, resolved through RTLD_GLOBAL / rpath
+        if not DIALECT_LIB.exists():
+            raise RuntimeError(
+                f"{DIALECT_LIB} is missing: build it with `python -m raf_amd.build`")
+        lib = ctypes.CDLL(str(DIALECT_LIB), mode=ctypes.RTLD_GLOBAL)
+        _bind(lib, DIALECT_SYMBOLS)
+        _dialect = lib
+    return _dialect
+
+
+class RafError(RuntimeError):
+    """The host layer raised (the reference would surface a TVMError from dmlc::Error)."""
+
+
+def check_raf(status: int) -> None:
+    if status != 0:
+        raise RafError(dialect().rafhip_raf_last_error().decode("utf-8", "replace"))

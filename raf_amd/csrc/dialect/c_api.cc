@@ -1,0 +1,217 @@
+// C entry points declared in rafhip_dialect.h: a minimal executor around the OpEnv mirror.
+#include <cstring>
+#include <memory>
+#include <sstream>
+#include <string>
+
+#include "hip_dialect.h"
+#include "raf_iface.h"
+#include "rafhip_dialect.h"
+
+using namespace raf;
+using namespace raf::op;
+
+struct rafhip_raf_env {
+  OpEnvPtr env;
+  CallValues call;
+  std::string name;
+  std::string op;
+};
+
+namespace {
+
+thread_local std::string g_error;
+thread_local std::unique_ptr<DialectPreference> g_pref;
+
+template <typename F>
+int Guard(F&& f) {
+  try {
+    g_error.clear();
+    f();
+    return 0;
+  } catch (const std::exception& e) {
+    g_error = e.what();
+    return 1;
+  } catch (...) {
+    g_error = "unknown C++ exception";
+    return 1;
+  }
+}
+
+value::TensorValue FromDesc(const rafhip_tensor_desc* d, const char* what) {
+  if (!d) throw Error(std::string(what) + ": null tensor descriptor");
+  if (d->ndim < 0 || (d->ndim > 0 && !d->shape)) throw Error(std::string(what) + ": bad shape");
+  TensorView t;
+  t.data = d->data;
+  t.device = Device(DevType(d->device_type), d->device_id);
+  t.dtype.code = d->dtype_code;
+  t.dtype.bits = d->dtype_bits;
+  t.shape.assign(d->shape, d->shape + d->ndim);
+  return value::MakeTensor(t);
+}
+
+constexpr int64_t kWsAlign = 256;
+int64_t RoundUp(int64_t x) { return (x + kWsAlign - 1) / kWsAlign * kWsAlign; }
+
+// What the executors do around Execute: point every requested workspace into the block the caller
+// provides, run, then take the pointers back (src/impl/vm/vm.cc:1099-1105, :846-853).
+struct WorkspaceBinding {
+  const std::vector<WorkspaceRequest>& reqs;
+  WorkspaceBinding(OpEnv* env, void* block, int64_t bytes) : reqs(env->workspace_requests()) {
+    int64_t need = 0;
+    for (const auto& r : reqs) need += RoundUp(r.nbytes);
+    if (need > 0 && (!block || bytes < need))
+      throw Error("workspace of " + std::to_string(bytes) + " bytes given, OpEnv requested " +
+                  std::to_string(need));
+    char* p = static_cast<char*>(block);
+    for (const auto& r : reqs) {
+      *r.dest = p;
+      p += RoundUp(r.nbytes);
+    }
+  }
+  ~WorkspaceBinding() {
+    for (const auto& r : reqs) *r.dest = nullptr;
+  }
+};
+
+rafhip_raf_env* Finish(const CallValues& call) {
+  RunDeclare(call);
+  std::string picked;
+  OpEnvPtr env = DispatchSingleOp(call, &picked);
+  auto* h = new rafhip_raf_env();
+  h->env = env;
+  h->call = call;
+  h->name = env->name();
+  h->op = picked;
+  return h;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* rafhip_raf_last_error(void) { return g_error.c_str(); }
+
+int rafhip_raf_dispatch_list(const char* base_op, int32_t device_type, char* buf, int32_t buflen) {
+  return Guard([&] {
+    if (!base_op || !buf || buflen <= 0) throw Error("rafhip_raf_dispatch_list: bad arguments");
+    std::ostringstream ss;
+    bool first = true;
+    for (const auto& e : OpDialect::GetDispatchList(base_op, DevType(device_type))) {
+      if (!first) ss << ';';
+      first = false;
+      ss << e.dialect << ':' << e.dialect_op << ':' << e.plevel;
+    }
+    std::string s = ss.str();
+    std::strncpy(buf, s.c_str(), (size_t)buflen - 1);
+    buf[buflen - 1] = '\0';
+  });
+}
+
+int rafhip_raf_set_dialect_preference(const char* dialects_csv) {
+  return Guard([&] {
+    g_pref.reset();
+    if (!dialects_csv || !*dialects_csv) return;
+    std::vector<std::string> names;
+    std::stringstream ss(dialects_csv);
+    std::string item;
+    while (std::getline(ss, item, ','))
+      if (!item.empty()) names.push_back(item);
+    g_pref.reset(new DialectPreference(std::move(names)));
+  });
+}
+
+int rafhip_raf_set_lans_grad_unscale(float factor) {
+  return Guard([&] { hip::SetLansGradUnscale(factor); });
+}
+
+int rafhip_raf_sgd_make(const rafhip_tensor_desc* x, const rafhip_tensor_desc* dx,
+                        const rafhip_tensor_desc* v, double learning_rate, double mu,
+                        rafhip_raf_env** env_out) {
+  return Guard([&] {
+    if (!env_out) throw Error("rafhip_raf_sgd_make: env_out is NULL");
+    *env_out = nullptr;
+    auto args = std::make_shared<schema::SgdArgs>();
+    args->x = FromDesc(x, "x");
+    args->dx = FromDesc(dx, "dx");
+    args->v = FromDesc(v, "v");
+    args->learning_rate = learning_rate;
+    args->mu = mu;
+    *env_out = Finish(MakeCall("raf.op.sgd", args));
+  });
+}
+
+int rafhip_raf_sgd_execute(rafhip_raf_env* env, const rafhip_tensor_desc* x,
+                           const rafhip_tensor_desc* dx, const rafhip_tensor_desc* v,
+                           const rafhip_tensor_desc* v1, const rafhip_tensor_desc* x1,
+                           void* stream) {
+  return Guard([&] {
+    if (!env) throw Error("rafhip_raf_sgd_execute: env is NULL");
+    std::vector<value::Value> inputs = {FromDesc(x, "x"), FromDesc(dx, "dx"), FromDesc(v, "v")};
+    value::Value out = value::MakeTuple({FromDesc(v1, "v1"), FromDesc(x1, "x1")});
+    OpEnv::SetStreamForAllBackends(env->call->device, stream);
+    WorkspaceBinding bind(env->env.get(), nullptr, 0);
+    env->env->Execute(inputs, out);
+  });
+}
+
+int rafhip_raf_lans_make(int32_t list_len, const rafhip_tensor_desc* tensor_list,
+                         const rafhip_tensor_desc* step, float learning_rate, float beta1,
+                         float beta2, float eps, int32_t bias_correction, float weight_decay,
+                         int32_t grad_averaging, int32_t mode, int32_t normalize_grad,
+                         rafhip_raf_env** env_out) {
+  return Guard([&] {
+    if (!env_out) throw Error("rafhip_raf_lans_make: env_out is NULL");
+    *env_out = nullptr;
+    if (list_len < 0 || (list_len > 0 && !tensor_list))
+      throw Error("rafhip_raf_lans_make: bad tensor list");
+    auto args = std::make_shared<schema::LansArgs>();
+    for (int32_t i = 0; i < list_len; ++i)
+      args->tensor_list.push_back(FromDesc(&tensor_list[i], "tensor_list"));
+    args->step = FromDesc(step, "step");
+    args->learning_rate = learning_rate;
+    args->beta1 = beta1;
+    args->beta2 = beta2;
+    args->eps = eps;
+    args->bias_correction = bias_correction;
+    args->weight_decay = weight_decay;
+    args->grad_averaging = grad_averaging;
+    args->mode = mode;
+    args->normalize_grad = normalize_grad != 0;
+    *env_out = Finish(MakeCall("raf.op.lans", args));
+  });
+}
+
+int rafhip_raf_lans_execute(rafhip_raf_env* env, int32_t list_len,
+                            const rafhip_tensor_desc* tensor_list, const rafhip_tensor_desc* step,
+                            void* workspace, int64_t workspace_bytes, void* stream) {
+  return Guard([&] {
+    if (!env) throw Error("rafhip_raf_lans_execute: env is NULL");
+    if (list_len < 0 || (list_len > 0 && !tensor_list))
+      throw Error("rafhip_raf_lans_execute: bad tensor list");
+    std::vector<value::Value> fields;
+    for (int32_t i = 0; i < list_len; ++i)
+      fields.push_back(FromDesc(&tensor_list[i], "tensor_list"));
+    value::Value tuple = value::MakeTuple(fields);
+    std::vector<value::Value> inputs = {tuple, FromDesc(step, "step")};
+    OpEnv::SetStreamForAllBackends(env->call->device, stream);
+    WorkspaceBinding bind(env->env.get(), workspace, workspace_bytes);
+    env->env->Execute(inputs, tuple);  // output aliases the inputs
+  });
+}
+
+int64_t rafhip_raf_env_workspace_bytes(const rafhip_raf_env* env) {
+  if (!env) return -1;
+  int64_t need = 0;
+  for (const auto& r : env->env->workspace_requests()) need += RoundUp(r.nbytes);
+  return need;
+}
+
+const char* rafhip_raf_env_name(const rafhip_raf_env* env) { return env ? env->name.c_str() : ""; }
+const char* rafhip_raf_env_op(const rafhip_raf_env* env) { return env ? env->op.c_str() : ""; }
+
+int rafhip_raf_env_destroy(rafhip_raf_env* env) {
+  return Guard([&] { delete env; });
+}
+
+}  // extern "C"

@@ -1,0 +1,227 @@
+// The `hip` dialect: OpEnv backends of raf.op.sgd and raf.op.lans for ROCm devices, written
+// against the OpEnv / dialect-op registration interface (raf_iface.h mirrors it) and calling the
+// gfx950 kernels through the C ABI of rafhip_optim.h only.
+//
+// Counterparts in the reference tree:
+//   LansHipEnv   LansImpl, src/op/dialect/cuda/lans.cc:25-165 (registration :164-165)
+//   SgdHipEnv    the RAF_TVM(sgd, ...) backend, src/op/dialect/tvm/optimizer.cc:22-45, whose
+//                Execute packs [x, dx, v, v1, x1] (src/op/dialect/tvm/tvm_utils.cc:92-133)
+// Differences on purpose: the stream is looked up at Execute time (the reference caches it in the
+// constructor, lans.cc:79-80); `step` stays on the device (the reference copies it to the host
+// and blocks, lans.cc:94-99); a single workspace holds partial sums and norms and there is no
+// per-element scratch (lans.cc:66); element counts are 64-bit (lans.cc:57 uses int); unsupported
+// arguments are reported through error_msgs so dispatch can fall through to another dialect.
+#include "hip_dialect.h"
+
+#include <sstream>
+
+#include "raf_iface.h"
+#include "rafhip_optim.h"
+
+namespace raf {
+namespace op {
+namespace hip {
+
+using device_api::DeviceAPI;
+using value::AsTensor;
+using value::AsTuple;
+using value::Value;
+
+namespace {
+
+float g_lans_grad_unscale = 1.0f;
+
+std::string KernelError(const char* what, int status) {
+  std::ostringstream ss;
+  ss << what << " failed with status " << status << ": " << rafhip_last_error();
+  return ss.str();
+}
+
+bool IsF32(const DType& t) { return t.code == kDLFloat && t.bits == 32; }
+bool IsF16(const DType& t) { return t.code == kDLFloat && t.bits == 16; }
+
+}  // namespace
+
+void SetLansGradUnscale(float factor) { g_lans_grad_unscale = factor; }
+float GetLansGradUnscale() { return g_lans_grad_unscale; }
+
+// ----------------------------------------------------------------------------------------- SGD
+class SgdHipEnv : public OpEnv {
+ public:
+  explicit SgdHipEnv(const CallValues& cv) {
+    const auto* args = cv->args_as<schema::SgdArgs>();
+    if (!args) {
+      error_msgs.push_back("raf.op.hip.sgd: call does not carry SgdArgs");
+      return;
+    }
+    // The VM passes the tensor fields as `inputs` (optimizer.cc:26-28 lists x, dx, v).
+    arg_indices = {args->FieldIndex("x"), args->FieldIndex("dx"), args->FieldIndex("v")};
+    learning_rate_ = args->learning_rate;
+    mu_ = args->mu;
+    const TensorView& x = args->x->tensor;
+    if (cv->device.device_type() != DevType::kROCM())
+      error_msgs.push_back("raf.op.hip.sgd: device is not rocm");
+    if (!IsF32(x.dtype) || !IsF32(args->dx->tensor.dtype) || !IsF32(args->v->tensor.dtype))
+      error_msgs.push_back("raf.op.hip.sgd: only float32 tensors are supported");
+    if (error_msgs.empty() && rafhip_device_count() <= 0)
+      error_msgs.push_back("raf.op.hip.sgd: no HIP device is visible");
+  }
+
+  std::string name() const override { return name_; }
+
+  void Execute(const CallValues& cv) override {
+    const auto* args = cv->args_as<schema::SgdArgs>();
+    RAF_CHECK(args != nullptr, "raf.op.hip.sgd expects SgdArgs");
+    Execute(std::vector<Value>{args->x, args->dx, args->v}, cv->out);
+  }
+
+  void Execute(const std::vector<Value>& inputs, Value output) override {
+    RAF_CHECK(inputs.size() == 3, "raf.op.hip.sgd takes x, dx, v");
+    const TensorView& x = AsTensor(inputs[0])->tensor;
+    const TensorView& dx = AsTensor(inputs[1])->tensor;
+    const TensorView& v = AsTensor(inputs[2])->tensor;
+    auto out = AsTuple(output);
+    RAF_CHECK(out->fields.size() == 2, "raf.op.hip.sgd produces (v1, x1)");
+    const TensorView& v1 = AsTensor(out->fields[0])->tensor;  // declare/optimizer.cc:42: (v1, x1)
+    const TensorView& x1 = AsTensor(out->fields[1])->tensor;
+    const int64_t n = dx.numel();
+    RAF_CHECK(x.numel() == n && v.numel() == n && v1.numel() == n && x1.numel() == n,
+              "raf.op.hip.sgd: tensor sizes differ");
+    void* stream = DeviceAPI::Get(DevType::kROCM())->GetStream();
+    int st = rafhip_sgd_f32(static_cast<const float*>(x.data), static_cast<const float*>(dx.data),
+                            static_cast<const float*>(v.data), static_cast<float*>(v1.data),
+                            static_cast<float*>(x1.data), n, learning_rate_, mu_, stream);
+    if (st != RAFHIP_OK) throw Error(KernelError("rafhip_sgd_f32", st));
+  }
+
+  static OpEnv* make(const CallValues& cv) { return new SgdHipEnv(cv); }
+
+ private:
+  double learning_rate_ = 0.0;
+  double mu_ = 0.0;
+  std::string name_ = TruncateName(GetUniqueName("raf.op.hip.sgd"));
+};
+
+// ---------------------------------------------------------------------------------------- LANS
+class LansHipEnv : public OpEnv {
+ public:
+  explicit LansHipEnv(const CallValues& cv) {
+    const auto* args = cv->args_as<schema::LansArgs>();
+    if (!args) {
+      error_msgs.push_back("raf.op.hip.lans: call does not carry LansArgs");
+      return;
+    }
+    arg_indices = {args->FieldIndex("tensor_list"), args->FieldIndex("step")};  // lans.cc:32-35
+    rafhip_lans_default_hparams(&hp_);
+    hp_.learning_rate = args->learning_rate;
+    hp_.beta1 = args->beta1;
+    hp_.beta2 = args->beta2;
+    hp_.eps = args->eps;
+    hp_.bias_correction = args->bias_correction;
+    hp_.weight_decay = args->weight_decay;
+    hp_.grad_averaging = args->grad_averaging;
+    hp_.mode = args->mode;
+    hp_.normalize_grad = args->normalize_grad ? 1 : 0;
+    hp_.grad_unscale = GetLansGradUnscale();
+
+    const size_t total = args->tensor_list.size();
+    if (total % 4 != 0) {  // lans.cc:53
+      error_msgs.push_back("raf.op.hip.lans: tensor_list must hold 4n tensors");
+      return;
+    }
+    n_ = (int32_t)(total / 4);
+    if (cv->device.device_type() != DevType::kROCM())
+      error_msgs.push_back("raf.op.hip.lans: device is not rocm");
+    if (hp_.mode != 0 && hp_.mode != 1)
+      error_msgs.push_back("raf.op.hip.lans: mode must be 0 (L2) or 1 (decoupled weight decay)");
+    int32_t grad_dtype = RAFHIP_F32;
+    std::vector<int64_t> numels;
+    for (int32_t i = 0; i < n_; ++i) {
+      const TensorView& g = args->tensor_list[i]->tensor;
+      const int32_t gd = IsF32(g.dtype) ? RAFHIP_F32 : IsF16(g.dtype) ? RAFHIP_F16 : -1;
+      if (gd < 0 || (i > 0 && gd != grad_dtype)) {
+        error_msgs.push_back("raf.op.hip.lans: gradients must all be float32 or all float16");
+        break;
+      }
+      grad_dtype = gd;
+      numels.push_back(g.numel());
+      for (int q = 1; q < 4; ++q) {  // w, m, v: fp32 (lans.cc:37-40) and as large as g
+        const TensorView& t = args->tensor_list[q * n_ + i]->tensor;
+        if (!IsF32(t.dtype)) error_msgs.push_back("raf.op.hip.lans: LANS only takes FP32 weights and state");
+        if (t.numel() != g.numel())
+          error_msgs.push_back("raf.op.hip.lans: g, w, m, v of one parameter differ in size");
+      }
+      if (!error_msgs.empty()) break;
+    }
+    if (!error_msgs.empty()) return;
+    if (rafhip_device_count() <= 0) {
+      error_msgs.push_back("raf.op.hip.lans: no HIP device is visible");
+      return;
+    }
+    int st = rafhip_lans_plan_create(n_, numels.data(), grad_dtype, &plan_);
+    if (st != RAFHIP_OK) {
+      error_msgs.push_back(KernelError("rafhip_lans_plan_create", st));
+      return;
+    }
+    RequestWorkspace(&workspace_, cv->device, rafhip_lans_workspace_bytes(plan_));
+    workspace_bytes_ = rafhip_lans_workspace_bytes(plan_);
+  }
+
+  ~LansHipEnv() override {
+    if (plan_) rafhip_lans_plan_destroy(plan_);
+  }
+
+  std::string name() const override { return name_; }
+
+  void Execute(const CallValues& cv) override {
+    const auto* args = cv->args_as<schema::LansArgs>();
+    RAF_CHECK(args != nullptr, "raf.op.hip.lans expects LansArgs");
+    std::vector<Value> fields(args->tensor_list.begin(), args->tensor_list.end());
+    Execute(std::vector<Value>{value::MakeTuple(std::move(fields)), args->step}, cv->out);
+  }
+
+  void Execute(const std::vector<Value>& inputs, Value output) override {
+    (void)output;  // aliases the inputs (declare/optimizer.cc:53-57); the update is in place
+    RAF_CHECK(inputs.size() == 2, "raf.op.hip.lans takes (tensor_list, step)");
+    auto tuple = AsTuple(inputs[0]);
+    RAF_CHECK((int64_t)tuple->fields.size() == 4 * (int64_t)n_,
+              "raf.op.hip.lans: tensor_list length changed since the OpEnv was made");
+    const TensorView& step = AsTensor(inputs[1])->tensor;
+    RAF_CHECK(step.ndim() == 0, "step must be a 0-d tensor");  // lans.cc:96
+    RAF_CHECK(IsF32(step.dtype), "step must be float32");
+    RAF_CHECK(workspace_ != nullptr || workspace_bytes_ == 0,
+              "raf.op.hip.lans: the executor did not provide the requested workspace");
+    std::vector<void*> ptrs(tuple->fields.size());
+    for (size_t i = 0; i < ptrs.size(); ++i) ptrs[i] = AsTensor(tuple->fields[i])->tensor.data;
+    void** p = ptrs.data();
+    void* stream = DeviceAPI::Get(DevType::kROCM())->GetStream();
+    int st = rafhip_lans_step(plan_, reinterpret_cast<const void* const*>(p),
+                              reinterpret_cast<float* const*>(p + n_),
+                              reinterpret_cast<float* const*>(p + 2 * n_),
+                              reinterpret_cast<float* const*>(p + 3 * n_),
+                              static_cast<const float*>(step.data), 0, &hp_, workspace_,
+                              workspace_bytes_, stream);
+    if (st != RAFHIP_OK) throw Error(KernelError("rafhip_lans_step", st));
+  }
+
+  static OpEnv* make(const CallValues& cv) { return new LansHipEnv(cv); }
+
+ private:
+  rafhip_lans_hparams hp_{};
+  int32_t n_ = 0;
+  rafhip_lans_plan* plan_ = nullptr;
+  void* workspace_ = nullptr;  // bound by the executor around each Execute
+  int64_t workspace_bytes_ = 0;
+  std::string name_ = TruncateName(GetUniqueName("raf.op.hip.lans"));
+};
+
+RAF_REGISTER_DIALECT("hip").set_enable(DevType::kROCM());
+// plevels above the reference's own backends (cuda lans = 20, tvm sgd = 10).
+RAF_REGISTER_DIALECT_OP(hip, lans, 30);
+RAF_OP_ENV_MAKER("raf.op.hip.lans", LansHipEnv::make);
+RAF_REGISTER_DIALECT_OP(hip, sgd, 30);
+RAF_OP_ENV_MAKER("raf.op.hip.sgd", SgdHipEnv::make);
+
+}  // namespace hip
+}  // namespace op
+}  // namespace raf

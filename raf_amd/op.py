@@ -1,0 +1,166 @@
+"""Imperative operator entry points with the signatures of the reference's generated
+``raf._op.imp.sgd`` / ``raf._op.imp.lans`` (argument lists: scripts/src_codegen/def_schema.py:671-694).
+
+Each call walks the same route as in RAF: arguments -> schema -> declare -> dialect dispatch ->
+``OpEnv`` -> ``Execute`` (src/impl/interpreter.cc:247-344), implemented by the C++ host layer in
+``libraf_hip_dialect.so``; the selected backend is the ``hip`` dialect, whose OpEnvs call the
+gfx950 kernels through the C ABI.  OpEnvs are cached per argument signature the way the VM caches
+them per (function, pc, shape key) (src/impl/vm/vm.cc:1053-1097).  Tensors are torch tensors on a
+ROCm device; torch supplies memory (including the per-call workspace, its caching allocator
+standing in for RAF's memory pool) and the current stream, nothing else.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_int64, c_void_p
+from typing import Dict, List, Sequence, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import TensorDesc, check_raf
+
+DEV_CPU, DEV_CUDA, DEV_ROCM = 1, 2, 10  # include/raf/device.h:37-50
+
+_DTYPES = {
+    torch.float32: (2, 32), torch.float16: (2, 16), torch.float64: (2, 64),
+    torch.bfloat16: (4, 16), torch.int32: (0, 32), torch.int64: (0, 64),
+}
+
+
+def _desc(t: torch.Tensor, keep: list) -> TensorDesc:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"expected a tensor, got {type(t).__name__}")
+    if not t.is_contiguous():
+        raise ValueError("tensors must be contiguous")
+    code, bits = _DTYPES[t.dtype]
+    shape = (c_int64 * max(t.dim(), 1))(*t.shape)
+    keep.append(shape)
+    # torch on ROCm reports its devices as "cuda"; they are ROCm devices for RAF's purposes.
+    dev_type = DEV_ROCM if t.is_cuda else DEV_CPU
+    dev_id = t.device.index if t.is_cuda and t.device.index is not None else 0
+    return TensorDesc(t.data_ptr(), dev_type, dev_id, code, bits, t.dim(),
+                      ctypes.cast(shape, ctypes.POINTER(c_int64)))
+
+
+def _stream(t: torch.Tensor):
+    return torch.cuda.current_stream(t.device).cuda_stream if t.is_cuda else None
+
+
+class _Env:
+    def __init__(self, handle):
+        self.handle = handle
+        lib = _lib.dialect()
+        self.name = lib.rafhip_raf_env_name(handle).decode()
+        self.op = lib.rafhip_raf_env_op(handle).decode()
+        self.workspace_bytes = lib.rafhip_raf_env_workspace_bytes(handle)
+
+    def __del__(self):
+        try:
+            _lib.dialect().rafhip_raf_env_destroy(self.handle)
+        except Exception:
+            pass
+
+
+_env_cache: Dict[Tuple, _Env] = {}
+
+
+def clear_op_env_cache() -> None:
+    _env_cache.clear()
+
+
+def _sig(t: torch.Tensor):
+    return (tuple(t.shape), t.dtype, str(t.device))
+
+
+def sgd(x, dx, v, learning_rate, mu):
+    """``raf._op.imp.sgd(x, dx, v, learning_rate, mu) -> (v1, x1)``: new tensors, inputs untouched
+    (src/op/declare/optimizer.cc:22-44)."""
+    lib = _lib.dialect()
+    keep: list = []
+    dx_, ddx, dv = _desc(x, keep), _desc(dx, keep), _desc(v, keep)
+    key = ("sgd", _sig(x), _sig(dx), _sig(v), float(learning_rate), float(mu))
+    env = _env_cache.get(key)
+    if env is None:
+        h = c_void_p(None)
+        check_raf(lib.rafhip_raf_sgd_make(dx_, ddx, dv, float(learning_rate), float(mu),
+                                          ctypes.byref(h)))
+        env = _env_cache[key] = _Env(h)
+    v1 = torch.empty_like(dx)  # the executor's AllocOutputBuffer (interpreter.cc:397-426)
+    x1 = torch.empty_like(dx)
+    check_raf(lib.rafhip_raf_sgd_execute(env.handle, dx_, ddx, dv, _desc(v1, keep), _desc(x1, keep),
+                                         _stream(dx)))
+    return v1, x1
+
+
+def lans(tensor_list: Sequence[torch.Tensor], step: torch.Tensor, learning_rate, beta1, beta2, eps,
+         bias_correction, weight_decay, grad_averaging, mode, normalize_grad):
+    """``raf._op.imp.lans(...)``: updates the w, m, v quarters of ``tensor_list`` in place and
+    returns the list (the op's output aliases its input, declare/optimizer.cc:53-57).  Booleans
+    become ints as the schema's ``int`` fields receive them (python/raf/optim/lans.py:51-54)."""
+    lib = _lib.dialect()
+    tensor_list = list(tensor_list)
+    keep: list = []
+    n4 = len(tensor_list)
+    descs = (TensorDesc * max(n4, 1))(*[_desc(t, keep) for t in tensor_list])
+    dstep = _desc(step, keep)
+    hp = (float(learning_rate), float(beta1), float(beta2), float(eps), int(bias_correction),
+          float(weight_decay), int(grad_averaging), int(mode), int(bool(normalize_grad)))
+    key = ("lans", tuple(_sig(t) for t in tensor_list), _sig(step), hp, get_lans_grad_unscale())
+    env = _env_cache.get(key)
+    if env is None:
+        h = c_void_p(None)
+        check_raf(lib.rafhip_raf_lans_make(n4, descs, dstep, *hp, ctypes.byref(h)))
+        env = _env_cache[key] = _Env(h)
+    ws = None
+    ws_ptr = None
+    if env.workspace_bytes > 0:
+        ws = torch.empty(env.workspace_bytes, dtype=torch.uint8, device=tensor_list[0].device)
+        ws_ptr = ws.data_ptr()
+    stream = _stream(tensor_list[0]) if n4 else None
+    check_raf(lib.rafhip_raf_lans_execute(env.handle, n4, descs, dstep, ws_ptr,
+                                          env.workspace_bytes, stream))
+    return tensor_list
+
+
+_lans_grad_unscale = 1.0
+
+
+def set_lans_grad_unscale(factor: float) -> None:
+    """hip-dialect extension: LANS multiplies every gradient by ``factor`` first (e.g. 1/1024 to
+    undo a loss scale on fp16 gradients).  Applies to LANS OpEnvs made afterwards."""
+    global _lans_grad_unscale
+    check_raf(_lib.dialect().rafhip_raf_set_lans_grad_unscale(float(factor)))
+    _lans_grad_unscale = float(factor)
+
+
+def get_lans_grad_unscale() -> float:
+    return _lans_grad_unscale
+
+
+def dispatch_list(base_op: str, device_type: int = DEV_ROCM) -> List[Tuple[str, str, int]]:
+    """[(dialect, dialect_op, plevel)] in dispatch order (OpDialect::GetDispatchList)."""
+    buf = ctypes.create_string_buffer(4096)
+    check_raf(_lib.dialect().rafhip_raf_dispatch_list(base_op.encode(), device_type, buf, 4096))
+    out = []
+    for item in buf.value.decode().split(";"):
+        if item:
+            d, o, p = item.split(":")
+            out.append((d, o, int(p)))
+    return out
+
+
+class with_dialect:
+    """Context manager pinning the dialects dispatch may use, like the reference's test helper
+    ``raf.testing.with_dialect`` (python/raf/testing/common.py:260-278)."""
+
+    def __init__(self, dialects):
+        self.dialects = [dialects] if isinstance(dialects, str) else list(dialects)
+
+    def __enter__(self):
+        check_raf(_lib.dialect().rafhip_raf_set_dialect_preference(",".join(self.dialects).encode()))
+        return self
+
+    def __exit__(self, *exc):
+        check_raf(_lib.dialect().rafhip_raf_set_dialect_preference(None))
+        return False

@@ -1,0 +1,189 @@
+// Host-side checks of the dialect registry mirror and of the `hip` dialect's registration, in the
+// manner of the reference's tests/cpp/test_op_dialect.cc:27-108 (two fake dialects on CPU with
+// plevels 10 and 12, dispatch-list order, IsDialectOp / GetDialect, maker lookup), extended with
+// the dispatcher's fall-through on error_msgs and the declare checks.  Plain asserts; prints the
+// name of each check so a failure names itself.  Runs without a GPU.
+#include <cstdio>
+#include <cstdlib>
+#include <string>
+
+#include "raf_iface.h"
+
+using namespace raf;
+using namespace raf::op;
+
+#define EXPECT(cond)                                                      \
+  do {                                                                    \
+    if (!(cond)) {                                                        \
+      std::fprintf(stderr, "FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond); \
+      std::exit(1);                                                       \
+    }                                                                     \
+  } while (0)
+
+template <typename F>
+static std::string Raises(F&& f) {
+  try {
+    f();
+  } catch (const raf::Error& e) {
+    return e.what();
+  }
+  return "";
+}
+
+class FakeEnv : public OpEnv {
+ public:
+  explicit FakeEnv(int type, bool refuse = false) : type(type) {
+    if (refuse) error_msgs.push_back("fake backend " + std::to_string(type) + " refuses");
+  }
+  int type;
+  std::string name() const override { return "cpptest.sgd"; }
+  void Execute(const CallValues&) override {}
+  void Execute(const std::vector<value::Value>&, value::Value) override {}
+};
+
+static bool g_refuse_high = false;
+
+RAF_REGISTER_DIALECT("mklShallowNN").set_enable(DevType::kCPU());
+RAF_REGISTER_DIALECT_OP(mklShallowNN, sgd, 10);
+RAF_OP_ENV_MAKER("raf.op.mklShallowNN.sgd", [](const CallValues&) -> OpEnv* { return new FakeEnv(0); });
+
+RAF_REGISTER_DIALECT("sshadow").set_enable(DevType::kCPU());
+RAF_REGISTER_DIALECT_OP(sshadow, sgd, 12);
+RAF_OP_ENV_MAKER("raf.op.sshadow.sgd",
+                 [](const CallValues&) -> OpEnv* { return new FakeEnv(1, g_refuse_high); });
+
+static value::TensorValue T(std::vector<int64_t> shape, DevType dev, int bits = 32) {
+  TensorView t;
+  t.shape = std::move(shape);
+  t.device = Device(dev, 0);
+  t.dtype.bits = bits;
+  return value::MakeTensor(t);
+}
+
+static CallValues SgdCall(DevType dev, std::vector<int64_t> xs = {4, 4},
+                          std::vector<int64_t> ds = {4, 4}) {
+  auto a = std::make_shared<schema::SgdArgs>();
+  a->x = T(xs, dev);
+  a->dx = T(ds, dev);
+  a->v = T(ds, dev);
+  a->learning_rate = 0.1;
+  a->mu = 0.9;
+  return MakeCall("raf.op.sgd", a);
+}
+
+int main() {
+  std::puts("dispatch list is plevel-descending and filtered by device type");
+  auto cpu = OpDialect::GetDispatchList("raf.op.sgd", DevType::kCPU());
+  EXPECT(cpu.size() == 2);
+  EXPECT(cpu.front().dialect == "sshadow" && cpu.front().plevel == 12);
+  EXPECT(cpu.back().dialect == "mklShallowNN" && cpu.back().dialect_op == "raf.op.mklShallowNN.sgd");
+  auto rocm = OpDialect::GetDispatchList("raf.op.sgd", DevType::kROCM());
+  EXPECT(rocm.size() == 1 && rocm.front().dialect == "hip" && rocm.front().plevel == 30);
+  auto lans = OpDialect::GetDispatchList("raf.op.lans", DevType::kROCM());
+  EXPECT(lans.size() == 1 && lans.front().dialect_op == "raf.op.hip.lans" && lans.front().plevel == 30);
+  EXPECT(OpDialect::GetDispatchList("raf.op.lans", DevType::kCUDA()).empty());
+  EXPECT(OpDialect::Dispatch("raf.op.sgd", DevType::kCPU()) == "raf.op.sshadow.sgd");
+  EXPECT(OpDialect::Dispatch("raf.op.sgd", DevType::kCPU(), {"sshadow"}) == "raf.op.mklShallowNN.sgd");
+
+  std::puts("dialect-op attributes and makers");
+  for (const auto& e : cpu) {
+    EXPECT(IsDialectOp(e.dialect_op));
+    EXPECT(GetDialect(e.dialect_op) == e.dialect);
+    EXPECT(GetBaseOp(e.dialect_op) == "raf.op.sgd");
+    EXPECT(OpEnvMaker::Get(e.dialect_op) != nullptr);
+  }
+  EXPECT(!IsDialectOp("raf.op.sgd"));
+  EXPECT(OpEnvMaker::Get("raf.op.hip.lans") != nullptr && OpEnvMaker::Get("raf.op.nope") == nullptr);
+  EXPECT(Dialect::IsEnabled("hip", DevType::kROCM()) && !Dialect::IsEnabled("hip", DevType::kCPU()));
+  EXPECT(!Raises([] { Dialect::IsEnabled("nope", DevType::kCPU()); }).empty());
+
+  std::puts("duplicate dialect or duplicate plevel on one base op is refused");
+  EXPECT(Raises([] {
+           OpDialect::RegisterOrGet("raf.op.sgd").add_dialect("sshadow", "raf.op.sshadow.sgd2", 99);
+         }).find("already has a registration on dialect sshadow") != std::string::npos);
+  Dialect::RegisterOrGet("third").set_name("third").set_enable(DevType::kCPU());
+  EXPECT(Raises([] {
+           OpDialect::RegisterOrGet("raf.op.sgd").add_dialect("third", "raf.op.third.sgd", 12);
+         }).find("same plevel=12") != std::string::npos);
+
+  std::puts("dispatch picks the highest plevel, falls through on error_msgs, reports when none fits");
+  auto call = SgdCall(DevType::kCPU());
+  RunDeclare(call);
+  std::string picked;
+  auto env = DispatchSingleOp(call, &picked);
+  EXPECT(static_cast<FakeEnv*>(env.get())->type == 1 && picked == "raf.op.sshadow.sgd");
+  g_refuse_high = true;
+  env = DispatchSingleOp(call, &picked);
+  EXPECT(static_cast<FakeEnv*>(env.get())->type == 0 && picked == "raf.op.mklShallowNN.sgd");
+  {
+    DialectPreference only({"sshadow"});
+    std::string msg = Raises([&] { DispatchSingleOp(call); });
+    EXPECT(msg.find("Cannot find a valid dispatch for op raf.op.sgd:") == 0);
+    EXPECT(msg.find("fake backend 1 refuses") != std::string::npos);
+  }
+  g_refuse_high = false;
+  {
+    DialectPreference order({"mklShallowNN", "sshadow"});  // preference order beats plevel
+    env = DispatchSingleOp(call, &picked);
+    EXPECT(picked == "raf.op.mklShallowNN.sgd");
+  }
+  EXPECT(DialectPreference::Current() == nullptr);
+
+  std::puts("hip OpEnvs report unsupported calls through error_msgs instead of throwing");
+  {
+    auto c = SgdCall(DevType::kCPU());
+    RunDeclare(c);
+    OpEnvPtr e((*OpEnvMaker::Get("raf.op.hip.sgd"))(c));
+    EXPECT(e->HasError() && e->error_msgs[0].find("not rocm") != std::string::npos);
+    EXPECT((e->arg_indices == std::vector<int>{0, 1, 2}));
+    EXPECT(e->name().find("raf_op_hip_sgd") == 0);
+    auto l = std::make_shared<schema::LansArgs>();
+    for (int i = 0; i < 4; ++i) l->tensor_list.push_back(T({8}, DevType::kROCM(), i == 1 ? 64 : 32));
+    l->step = T({}, DevType::kROCM());
+    l->mode = 1;
+    auto lc = MakeCall("raf.op.lans", l);
+    RunDeclare(lc);
+    EXPECT(value::AsTuple(lc->out)->fields.size() == 4 && lc->device.device_type() == DevType::kROCM());
+    EXPECT(value::AsTuple(lc->out)->fields[2] == l->tensor_list[2]);  // output aliases the inputs
+    OpEnvPtr le((*OpEnvMaker::Get("raf.op.hip.lans"))(lc));
+    EXPECT(le->HasError() && le->error_msgs[0].find("FP32") != std::string::npos);
+    EXPECT((le->arg_indices == std::vector<int>{0, 1}));
+  }
+
+  std::puts("declare checks");
+  EXPECT(Raises([] { RunDeclare(SgdCall(DevType::kCPU(), {4, 4}, {4, 5})); }).find("differ in shape") !=
+         std::string::npos);
+  EXPECT(Raises([] { RunDeclare(SgdCall(DevType::kCPU(), {4, 4}, {16})); }).find("differ in rank") !=
+         std::string::npos);
+  {
+    auto c = SgdCall(DevType::kCPU(), {2, 3}, {2, 3});
+    RunDeclare(c);
+    auto out = value::AsTuple(c->out);
+    EXPECT(out->fields.size() == 2);  // (v1, x1)
+    EXPECT(value::AsTensor(out->fields[0])->tensor.shape == (std::vector<int64_t>{2, 3}));
+    auto l = std::make_shared<schema::LansArgs>();
+    for (int i = 0; i < 6; ++i) l->tensor_list.push_back(T({8}, DevType::kROCM()));
+    l->step = T({}, DevType::kROCM());
+    EXPECT(Raises([&] { RunDeclare(MakeCall("raf.op.lans", l)); }).find("4n tensors") != std::string::npos);
+  }
+
+  std::puts("unique and truncated OpEnv names");
+  std::string a = GetUniqueName("raf.op.hip.zzz"), b = GetUniqueName("raf.op.hip.zzz");
+  EXPECT(a == "raf_op_hip_zzz" && b == "raf_op_hip_zzz_1");
+  EXPECT(TruncateName(std::string(200, 'x')).size() < 120);
+
+  std::puts("schema field indices");
+  schema::LansArgs la;
+  EXPECT(la.FieldIndex("tensor_list") == 0 && la.FieldIndex("step") == 1 && la.FieldIndex("normalize_grad") == 10);
+  EXPECT(!Raises([&] { la.FieldIndex("nope"); }).empty());
+
+  std::puts("stream plumbing");
+  int dummy = 0;
+  OpEnv::SetStreamForAllBackends(Device(DevType::kROCM(), 0), &dummy);
+  EXPECT(device_api::DeviceAPI::Get(DevType::kROCM())->GetStream() == &dummy);
+  EXPECT(device_api::DeviceAPI::Get(DevType::kCPU())->GetStream() == nullptr);
+  OpEnv::SetStreamForAllBackends(Device(DevType::kROCM(), 0), nullptr);
+
+  std::puts("ALL OK");
+  return 0;
+}

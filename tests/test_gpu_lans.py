@@ -1,0 +1,239 @@
+"""GPU parity of raf.op.lans: the HIP kernels, called through the C ABI, against the float64
+oracle.  Tolerances are the stated ones -- max relative error per element 1e-5 after one step and
+1e-4 after 100 steps -- on w, m and v; norms must agree to 1e-10."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import lans_f64
+from oracle.lans_f64 import LansHParams
+from tests.golden import make_fixtures as mf
+from tests.helpers import lans_inputs, max_rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL_1 = 1e-5
+TOL_100 = 1e-4
+
+
+def _to_dev(arrs):
+    return [torch.from_numpy(np.ascontiguousarray(a)).to(DEV) for a in arrs]
+
+
+def _khp(hp: LansHParams):
+    from raf_amd import kernels
+
+    return kernels.make_hparams(hp.learning_rate, hp.beta1, hp.beta2, hp.eps, hp.bias_correction,
+                                hp.weight_decay, hp.grad_averaging, hp.mode, hp.normalize_grad,
+                                hp.grad_unscale)
+
+
+def _gpu_steps(g, w, m, v, hp, first_step, steps=1, step_on_device=True):
+    from raf_amd import kernels
+
+    tg, tw, tm, tv = _to_dev(g), _to_dev(w), _to_dev(m), _to_dev(v)
+    plan = kernels.LansPlan([a.size for a in w], tg[0].dtype if tg else torch.float32, DEV)
+    for s in range(steps):
+        step = first_step + s
+        arg = torch.tensor(float(step), dtype=torch.float32, device=DEV) if step_on_device else step
+        plan.step(tg, tw, tm, tv, arg, _khp(hp))
+    torch.cuda.synchronize()
+    norms = plan.read_norms()
+    plan.close()
+    back = lambda ts: [t.cpu().numpy() for t in ts]
+    return back(tw), back(tm), back(tv), norms, back(tg)
+
+
+def _assert_close(got, want, tol, what):
+    for t, (a, b) in enumerate(zip(got, want)):
+        e = max_rel_err(a, b)
+        assert e <= tol, f"{what}[{t}] max rel err {e:.3e} > {tol}"
+
+
+def _assert_norms(got, want):
+    nz = want != 0
+    assert np.array_equal(got[~nz], want[~nz])
+    if nz.any():
+        assert np.max(np.abs(got[nz] - want[nz]) / want[nz]) < 1e-10
+
+
+# ------------------------------------------------------------------ committed fixtures
+@pytest.mark.parametrize("name", list(mf.LANS_CASES))
+def test_golden_fixture(native_libs, name):
+    z = np.load(mf.HERE / "lans_kat.npz")
+    kw, g16, first_step = mf.LANS_CASES[name]
+    hp = LansHParams(**kw)
+    nt = len(mf.LANS_SIZES)
+    g, w, m, v = ([z[f"{name}/{q}{t}"] for t in range(nt)] for q in "gwmv")
+    for steps in mf.LANS_STORED:
+        gw, gm, gv, norms, _ = _gpu_steps(g, w, m, v, hp, first_step, steps)
+        tol = TOL_1 if steps == 1 else TOL_100
+        for q, got in (("w", gw), ("m", gm), ("v", gv)):
+            _assert_close(got, [z[f"{name}/{q}{t}_after{steps}"] for t in range(nt)], tol, f"{name}/{q}")
+        _assert_norms(norms, z[f"{name}/norms_after{steps}"])
+
+
+# ------------------------------------------------------------------ edge sizes, flags, paths
+EDGE_SIZES = [1, 3, 4, 5, 0, 255, 256, 257, 1023, 1024, 1025, 16383, 16384, 16385, 65537, 100003]
+
+
+@pytest.mark.parametrize("g16", [False, True])
+@pytest.mark.parametrize("mode", [0, 1])
+def test_edge_sizes_against_oracle(native_libs, g16, mode):
+    hp = LansHParams(mode=mode, grad_unscale=(1 / 1024 if g16 else 1.0))
+    g, w, m, v = lans_inputs(EDGE_SIZES, cfg=60 + mode, g16=g16)
+    ow, om, ov, on = lans_f64.lans_step(g, w, m, v, 2, hp)
+    gw, gm, gv, gn, gg = _gpu_steps(g, w, m, v, hp, 2)
+    _assert_close(gw, ow, TOL_1, "w")
+    _assert_close(gm, om, TOL_1, "m")
+    _assert_close(gv, ov, TOL_1, "v")
+    _assert_norms(gn, on)
+    assert all(np.array_equal(a, b) for a, b in zip(gg, g)), "gradients must stay untouched"
+
+
+@pytest.mark.parametrize("flags", [
+    dict(bias_correction=0), dict(grad_averaging=0), dict(normalize_grad=False),
+    dict(weight_decay=0.0), dict(weight_decay=0.0, mode=0),
+    dict(learning_rate=0.02, beta1=0.8, beta2=0.99, eps=1e-8, weight_decay=0.1),
+])
+def test_flag_combinations(native_libs, flags):
+    hp = LansHParams(**flags)
+    sizes = [7, 1000, 20001]
+    g, w, m, v = lans_inputs(sizes, cfg=70)
+    ow, om, ov, on = lans_f64.lans_step(g, w, m, v, 5, hp)
+    gw, gm, gv, gn, _ = _gpu_steps(g, w, m, v, hp, 5)
+    _assert_close(gw, ow, TOL_1, "w")
+    _assert_close(gm, om, TOL_1, "m")
+    _assert_close(gv, ov, TOL_1, "v")
+    _assert_norms(gn, on)
+
+
+def test_step_from_device_tensor_equals_host_step(native_libs):
+    g, w, m, v = lans_inputs([3000, 17], cfg=71)
+    a = _gpu_steps(g, w, m, v, LansHParams(), 7, step_on_device=True)
+    b = _gpu_steps(g, w, m, v, LansHParams(), 7, step_on_device=False)
+    for x, y in zip(a[:3], b[:3]):
+        assert all(np.array_equal(p, q) for p, q in zip(x, y))
+
+
+def test_unaligned_tensors_take_the_scalar_path(native_libs):
+    from raf_amd import kernels
+
+    sizes = [5, 1001, 40000]
+    g, w, m, v = lans_inputs(sizes, cfg=72)
+    hp = LansHParams()
+    ow, om, ov, on = lans_f64.lans_step(g, w, m, v, 3, hp)
+
+    def shifted(arrs, off):  # views that start `off` elements into a larger buffer
+        out = []
+        for a in arrs:
+            buf = torch.zeros(a.size + 8, dtype=torch.float32, device=DEV)
+            buf[off:off + a.size] = torch.from_numpy(a).to(DEV)
+            out.append(buf[off:off + a.size])
+        return out
+
+    tg, tw, tm, tv = shifted(g, 1), shifted(w, 2), shifted(m, 3), shifted(v, 1)
+    assert tg[1].data_ptr() % 16 != 0
+    plan = kernels.LansPlan(sizes, torch.float32, DEV)
+    plan.step(tg, tw, tm, tv, 3, _khp(hp))
+    torch.cuda.synchronize()
+    _assert_close([t.cpu().numpy() for t in tw], ow, TOL_1, "w")
+    _assert_close([t.cpu().numpy() for t in tm], om, TOL_1, "m")
+    _assert_close([t.cpu().numpy() for t in tv], ov, TOL_1, "v")
+    _assert_norms(plan.read_norms(), on)
+
+
+def test_zero_norm_tensors(native_libs):
+    sizes = [100, 100, 100]
+    g, w, m, v = lans_inputs(sizes, cfg=73)
+    g[0][:] = 0  # ||g|| == 0: gradient not normalised
+    w[1][:] = 0  # ||w|| == 0: trust ratios fall back to lr
+    g[2][:] = 0
+    m[2][:] = 0
+    v[2][:] = 0
+    w[2][:] = 0  # everything zero: stays zero with eps > 0, is 0/0 = NaN with eps == 0
+    for eps, all_zero_gives_nan in ((1e-6, False), (0.0, True)):
+        hp = LansHParams(eps=eps)
+        with np.errstate(all="ignore"):
+            ow, om, ov, on = lans_f64.lans_step(g, w, m, v, 2, hp)
+        gw, gm, gv, gn, _ = _gpu_steps(g, w, m, v, hp, 2)
+        for t in (0, 1):
+            assert max_rel_err(gw[t], ow[t]) <= TOL_1 and max_rel_err(gm[t], om[t]) <= TOL_1
+            assert max_rel_err(gv[t], ov[t]) <= TOL_1
+        assert np.isnan(ow[2]).all() == all_zero_gives_nan  # the rule propagates NaN, so do we
+        assert np.array_equal(np.isnan(gw[2]), np.isnan(ow[2]))
+        assert np.array_equal(gw[2][~np.isnan(ow[2])], ow[2][~np.isnan(ow[2])])
+        assert gn[0][0] == 0.0 and gn[1][1] == 0.0
+
+
+def test_empty_list_and_empty_tensors(native_libs):
+    from raf_amd import kernels
+
+    plan = kernels.LansPlan([], torch.float32, DEV)
+    plan.step([], [], [], [], 1, _khp(LansHParams()))  # no-op
+    plan2 = kernels.LansPlan([0, 0], torch.float32, DEV)
+    z = [torch.empty(0, device=DEV), torch.empty(0, device=DEV)]
+    plan2.step(z, z, z, z, 1, _khp(LansHParams()))
+    torch.cuda.synchronize()
+
+
+# ------------------------------------------------------------------ properties
+def test_bitwise_determinism_and_order_independence(native_libs):
+    sizes = [40000, 3, 70001, 1 << 18]
+    g, w, m, v = lans_inputs(sizes, cfg=74)
+    a = _gpu_steps(g, w, m, v, LansHParams(), 2)
+    b = _gpu_steps(g, w, m, v, LansHParams(), 2)
+    perm = [3, 1, 0, 2]
+    c = _gpu_steps(*([x[i] for i in perm] for x in (g, w, m, v)), LansHParams(), 2)
+    for q in range(3):
+        for t in range(4):
+            assert np.array_equal(a[q][t], b[q][t])
+            assert np.array_equal(a[q][perm[t]], c[q][t])  # a tensor's result ignores its neighbours
+    assert np.array_equal(a[3], b[3])
+
+
+def test_hundred_steps_against_oracle(native_libs, c_oracle):
+    """100 consecutive steps, state carried in fp32 on both sides, gradient fixed."""
+    sizes = [1, 9, 4099, 70001]
+    g, w, m, v = lans_inputs(sizes, cfg=75, zero_state=True)
+    hp = LansHParams()
+    gw, gm, gv, gn, _ = _gpu_steps(g, w, m, v, hp, 1, steps=100)
+    ow, om, ov = [a.copy() for a in w], [a.copy() for a in m], [a.copy() for a in v]
+    for s in range(1, 101):
+        on = c_oracle.lans_step_inplace(g, ow, om, ov, s, hp, threads=4)
+    _assert_close(gw, ow, TOL_100, "w")
+    _assert_close(gm, om, TOL_100, "m")
+    _assert_close(gv, ov, TOL_100, "v")
+    _assert_norms(gn, on)
+    # and against the NumPy oracle on the small tensors (the C restatement is itself pinned to it)
+    nw, nm, nv = [a.copy() for a in w[:3]], [a.copy() for a in m[:3]], [a.copy() for a in v[:3]]
+    for s in range(1, 101):
+        nw, nm, nv, _ = lans_f64.lans_step(g[:3], nw, nm, nv, s, hp)
+    _assert_close(gw[:3], nw, TOL_100, "w(numpy)")
+
+
+# ------------------------------------------------------------------ error paths (no kernel runs)
+def test_workspace_and_argument_errors(native_libs):
+    from raf_amd import _lib, kernels
+
+    plan = kernels.LansPlan([1000], torch.float32, DEV)
+    t = [torch.zeros(1000, device=DEV)]
+    hp = _khp(LansHParams())
+    with pytest.raises(_lib.RafHipError) as e:
+        plan.step(t, t, t, t, 1, hp, workspace=torch.empty(64, dtype=torch.uint8, device=DEV))
+    assert e.value.status == _lib.RAFHIP_ERR_WORKSPACE
+    big = torch.empty(plan.workspace_bytes + 512, dtype=torch.uint8, device=DEV)
+    start = (256 - big.data_ptr() % 256) % 256 + 4  # 4 bytes past a 256-byte boundary
+    with pytest.raises(_lib.RafHipError, match="aligned"):
+        plan.step(t, t, t, t, 1, hp, workspace=big[start:])
+    bad = kernels.make_hparams(mode=2)
+    with pytest.raises(_lib.RafHipError, match="mode"):
+        plan.step(t, t, t, t, 1, bad)
+    with pytest.raises(ValueError):
+        plan.step(t + t, t, t, t, 1, hp)
+    with pytest.raises(TypeError):
+        plan.step([t[0].half()], t, t, t, 1, hp)
+    with pytest.raises(TypeError):
+        kernels.LansPlan([8], torch.bfloat16, DEV)

@@ -1,0 +1,108 @@
+"""GPU parity of raf.op.sgd: the HIP kernel, called through the C ABI, against the fp32 oracle --
+bit for bit (NaN lanes compared as NaN masks; payloads are not part of the contract)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import sgd_f32
+from tests.golden import make_fixtures as mf
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _bits_equal(got: torch.Tensor, want: np.ndarray):
+    g = got.detach().cpu().numpy().ravel()
+    w = np.ascontiguousarray(want).ravel()
+    nan = np.isnan(w)
+    assert np.array_equal(np.isnan(g), nan)
+    assert np.array_equal(g.view(np.uint32)[~nan], w.view(np.uint32)[~nan])
+
+
+def _rand(n, seed):
+    r = np.random.default_rng([2024, 1, seed])
+    return (r.normal(0, .02, n).astype(np.float32), r.normal(0, 1e-3, n).astype(np.float32),
+            r.normal(0, 1e-3, n).astype(np.float32))
+
+
+def test_golden_fixture_bitwise(native_libs):
+    from raf_amd import kernels
+
+    z = np.load(mf.HERE / "sgd_kat.npz")
+    x, dx, v = (torch.from_numpy(z[k]).to(DEV) for k in ("x0", "dx", "v0"))
+    v1, x1 = kernels.sgd_f32(x, dx, v, float(z["learning_rate"]), float(z["mu"]))
+    _bits_equal(v1, z["v1_bits"].view(np.float32))
+    _bits_equal(x1, z["x1_bits"].view(np.float32))
+    # inputs untouched (out-of-place op, src/op/declare/optimizer.cc:34-42)
+    assert np.array_equal(x.cpu().numpy().view(np.uint32), z["x0"].view(np.uint32))
+    assert np.array_equal(v.cpu().numpy().view(np.uint32), z["v0"].view(np.uint32))
+
+
+@pytest.mark.parametrize("n", [0, 1, 2, 3, 4, 5, 7, 255, 256, 257, 1023, 1025, 2048 * 3 + 1, 1 << 20])
+def test_sizes_and_tails(native_libs, n):
+    from raf_amd import kernels
+
+    x0, dx, v0 = _rand(n, n)
+    v1, x1 = kernels.sgd_f32(torch.from_numpy(x0).to(DEV), torch.from_numpy(dx).to(DEV),
+                             torch.from_numpy(v0).to(DEV), 0.01, 0.9)
+    ov, ox = sgd_f32.sgd_step(x0, dx, v0, 0.01, 0.9)
+    _bits_equal(v1, ov)
+    _bits_equal(x1, ox)
+
+
+@pytest.mark.parametrize("offset", [1, 2, 3])
+def test_unaligned_views_take_the_scalar_path(native_libs, offset):
+    from raf_amd import kernels
+
+    n = 10001
+    x0, dx, v0 = _rand(n + 8, 77 + offset)
+    tx, tdx, tv = (torch.from_numpy(a).to(DEV)[offset:offset + n] for a in (x0, dx, v0))
+    assert tx.data_ptr() % 16 != 0
+    v1, x1 = kernels.sgd_f32(tx, tdx, tv, 0.05, 0.5)
+    ov, ox = sgd_f32.sgd_step(x0[offset:offset + n], dx[offset:offset + n], v0[offset:offset + n], 0.05, 0.5)
+    _bits_equal(v1, ov)
+    _bits_equal(x1, ox)
+
+
+def test_outputs_may_alias_inputs(native_libs):
+    from raf_amd import kernels
+
+    x0, dx, v0 = _rand(100003, 5)
+    tx, tdx, tv = (torch.from_numpy(a).to(DEV) for a in (x0, dx, v0))
+    kernels.sgd_f32(tx, tdx, tv, 0.01, 0.9, v_out=tv, x_out=tx)
+    ov, ox = sgd_f32.sgd_step(x0, dx, v0, 0.01, 0.9)
+    _bits_equal(tv, ov)
+    _bits_equal(tx, ox)
+
+
+def test_config1_full_size_bitwise(native_libs, c_oracle):
+    """BASELINE config 1: one fp32 tensor of 4,194,304 elements, w~N(0,.02), grad~N(0,1e-3),
+    velocity 0, lr .01, momentum .9 -- every element compared."""
+    from raf_amd import kernels
+
+    n = 4_194_304
+    r = np.random.default_rng([2024, 1, 0])
+    x0 = r.normal(0, .02, n).astype(np.float32)
+    dx = r.normal(0, 1e-3, n).astype(np.float32)
+    v0 = np.zeros(n, np.float32)
+    tx, tdx, tv = (torch.from_numpy(a).to(DEV) for a in (x0, dx, v0))
+    for _ in range(3):  # three consecutive steps, state carried on both sides
+        tv, tx = kernels.sgd_f32(tx, tdx, tv, 0.01, 0.9)
+        v0, x0 = c_oracle.sgd_step(x0, dx, v0, 0.01, 0.9, threads=8)
+        _bits_equal(tv, v0)
+        _bits_equal(tx, x0)
+
+
+def test_2d_shape_and_shape_mismatch(native_libs):
+    from raf_amd import kernels
+
+    x0, dx, v0 = (a.reshape(37, 29) for a in _rand(37 * 29, 9))
+    v1, x1 = kernels.sgd_f32(torch.from_numpy(x0).to(DEV), torch.from_numpy(dx).to(DEV),
+                             torch.from_numpy(v0).to(DEV), 0.01, 0.9)
+    assert v1.shape == (37, 29)
+    ov, ox = sgd_f32.sgd_step(x0, dx, v0, 0.01, 0.9)
+    _bits_equal(v1.reshape(-1), ov.reshape(-1))
+    with pytest.raises(ValueError):
+        kernels.sgd_f32(torch.zeros(4, device=DEV), torch.zeros(5, device=DEV), torch.zeros(4, device=DEV), .1, .9)
+    with pytest.raises(TypeError):
+        kernels.sgd_f32(*(torch.zeros(4, device=DEV, dtype=torch.float16),) * 3, .1, .9)
