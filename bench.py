@@ -1,0 +1,299 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused optimizer step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A step is one pass of the hot path over one resident parameter set: for the default workload one
+`raf.op.lans` step over a BERT-large-shaped list (391 tensors, 335,141,888 elements; fp32 weights and
+state, fp16 gradients scaled by 1024 and unscaled in the kernel), called through the C ABI.  Inputs
+are synthetic (seeded, generated on the GPU) and resident in HBM before the timed region.  Prints
+ONE JSON line; `value` is algorithmic bytes per step divided by the wall time per step.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+
+# Algorithmic bytes per element of a three-pass LANS step, the figure the bandwidth is quoted on:
+#   norms of g and w (read g,w); norms of the update directions (read g,w,m,v); the update itself
+#   (read g,w,m,v, write w,m,v): 28 compulsory + 24 re-read = 52 B with fp32 gradients, 46 B with fp16.
+# The kernels move less than that (||w|| rides along with the second pass, saving its 4 B), which
+# is reported separately as `kernel_bytes_per_element`.
+def lans_bytes_per_elt(g_bytes: int):
+    a = g_bytes + 4
+    b = g_bytes + 12
+    c = g_bytes + 12 + 12
+    return a, b, c
+
+
+def lans_kernel_bytes_per_elt(g_bytes: int):
+    return g_bytes, g_bytes + 12, g_bytes + 12 + 12
+
+
+SGD_BYTES_PER_ELT = 20  # read x, dx, v; write v1, x1
+
+# HBM traffic per launch of the dominant kernel (bytes), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# runs scaled by a plain copy kernel of known size; see profiles/.  None = not measured.
+MEASURED_TRAFFIC = {}
+
+
+def workloads():
+    from raf_amd import shapes
+
+    return {
+        "lans_bert_large_fp16grad": dict(kind="lans", sizes=shapes.numels(shapes.bert_large_shapes()), g16=True,
+                                         zero_state=True, step0=1),
+        "lans_bert_large_fp32grad": dict(kind="lans", sizes=shapes.numels(shapes.bert_large_shapes()), g16=False,
+                                         zero_state=True, step0=1),
+        "lans_bert_base_fp32": dict(kind="lans", sizes=shapes.numels(shapes.bert_base_shapes()), g16=False,
+                                    zero_state=True, step0=1),
+        "lans_2000_small_tensors": dict(kind="lans", sizes=shapes.log_uniform_numels(), g16=False,
+                                        zero_state=False, step0=2),
+        "lans_gpt2_1p5b_fp32": dict(kind="lans", sizes=shapes.numels(shapes.gpt2_shapes()), g16=False,
+                                    zero_state=True, step0=1),
+        "sgd_4m_fp32": dict(kind="sgd", n=4_194_304),
+    }
+
+
+def gen_lans(sizes, g16, zero_state, dev, seed=2024):
+    import torch
+
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    g, w, m, v = [], [], [], []
+    for n in sizes:
+        gt = torch.randn(n, device=dev, generator=gen) * 1e-3
+        g.append((gt * 1024.0).half() if g16 else gt)
+        w.append(torch.randn(n, device=dev, generator=gen) * 0.02)
+        if zero_state:
+            m.append(torch.zeros(n, device=dev))
+            v.append(torch.zeros(n, device=dev))
+        else:
+            m.append(torch.randn(n, device=dev, generator=gen) * 1e-4)
+            v.append((torch.randn(n, device=dev, generator=gen) * 1e-6).abs())
+    return g, w, m, v
+
+
+def cpu_baseline_lans(sizes, g16, budget_s=12.0):
+    """The oracle's C restatement (a port: the reference has no CPU LANS) timed on the host cores
+    over a prefix of the same tensor list, large enough to be memory-bound."""
+    from oracle import c_oracle
+    from oracle.lans_f64 import LansHParams
+
+    threads = min(16, os.cpu_count() or 1, c_oracle.max_threads())
+    sample, total = [], 0
+    for n in sizes:
+        sample.append(n)
+        total += n
+        if total >= 64_000_000:
+            break
+    rng = np.random.default_rng(2024)
+    g = [(rng.standard_normal(n, dtype=np.float32) * (1.024 if g16 else 1e-3)).astype(np.float16 if g16 else np.float32)
+         for n in sample]
+    w = [rng.standard_normal(n, dtype=np.float32) * np.float32(0.02) for n in sample]
+    m = [np.zeros(n, np.float32) for n in sample]
+    v = [np.zeros(n, np.float32) for n in sample]
+    hp = LansHParams(grad_unscale=(1.0 / 1024 if g16 else 1.0))
+    best, reps, t_all = None, 0, time.perf_counter()
+    while reps < 5 and time.perf_counter() - t_all < budget_s:
+        t0 = time.perf_counter()
+        c_oracle.lans_step_inplace(g, w, m, v, reps + 1, hp, threads=threads)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+        reps += 1
+    bpe = sum(lans_bytes_per_elt(2 if g16 else 4))
+    return {"value": round(total * bpe / best / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"first {len(sample)} tensors of the list ({total} elements), best of {reps} steps, "
+                      f"float64 C restatement of the rule, OpenMP {threads} threads",
+            "ms_per_step_extrapolated": round(best * 1e3 * sum(sizes) / total, 1)}
+
+
+def cpu_baseline_sgd(n, budget_s=10.0):
+    from oracle import c_oracle
+
+    threads = min(16, os.cpu_count() or 1, c_oracle.max_threads())
+    rng = np.random.default_rng(2024)
+    x, dx, v = (rng.standard_normal(n, dtype=np.float32) for _ in range(3))
+    best, reps, t_all = None, 0, time.perf_counter()
+    while reps < 50 and time.perf_counter() - t_all < budget_s:
+        t0 = time.perf_counter()
+        c_oracle.sgd_step(x, dx, v, 0.01, 0.9, threads=threads)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+        reps += 1
+    return {"value": round(n * SGD_BYTES_PER_ELT / best / 1e9, 2), "unit": "GB/s", "cores": threads,
+            "kind": "port", "sample": f"the full tensor ({n} elements), best of {reps} steps, fp32 C restatement "
+                                      f"(-ffp-contract=off), OpenMP {threads} threads"}
+
+
+def bench_lans(name, wl, args):
+    import torch
+
+    from raf_amd import kernels
+
+    dev = torch.device("cuda:0")
+    sizes, g16 = wl["sizes"], wl["g16"]
+    total = sum(sizes)
+    g, w, m, v = gen_lans(sizes, g16, wl["zero_state"], dev)
+    plan = kernels.LansPlan(sizes, torch.float16 if g16 else torch.float32, dev)
+    plan.set_schedule(args.schedule)
+    hp = kernels.make_hparams(grad_unscale=(1.0 / 1024 if g16 else 1.0))
+    plan.bind(g, w, m, v, hp)
+    step_t = torch.full((), float(wl["step0"]), dtype=torch.float32, device=dev)
+
+    for _ in range(args.warmup):
+        plan.step_bound(step_t)
+        step_t.add_(1.0)
+    if not args.no_kernel_events:
+        plan.timing_enable(args.steps)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        plan.step_bound(step_t)
+        step_t.add_(1.0)  # the step counter lives on the device, as in the reference's traced optimizer
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+
+    a, b, c = lans_bytes_per_elt(2 if g16 else 4)
+    ka, kb, kc = lans_kernel_bytes_per_elt(2 if g16 else 4)
+    bytes_step = total * (a + b + c)
+    out = {
+        "metric": "LANS optimizer-step achieved HBM bandwidth (algorithmic bytes / step time); "
+                  "ms_per_step is the step time",
+        "value": round(bytes_step / (ms_per_step * 1e-3) / 1e9, 1),
+        "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f64", "data": "synthetic",
+        "config": {"workload": name, "tensors": len(sizes), "elements": total,
+                   "storage": "fp32 w/m/v, " + ("fp16 g (x1024, unscaled in kernel)" if g16 else "fp32 g"),
+                   "bytes_per_element": a + b + c, "bytes_per_step": bytes_step,
+                   "kernel_bytes_per_element": ka + kb + kc,
+                   "pct_of_hbm_peak": round(100 * bytes_step / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
+                   "schedule": args.schedule, "launches_per_step": 6 if args.schedule == "phased" else 2},
+    }
+    if not args.no_kernel_events:
+        ts = np.array([plan.timing_read(i) for i in range(args.steps)], dtype=np.float64)
+        avg = ts.mean(axis=0)
+        if args.schedule == "phased":
+            # dominant kernel: lans_apply (reads g,w,m,v, writes w,m,v)
+            apply_ms = float(avg[4])
+            achieved = total * c / (apply_ms * 1e-3) / 1e9
+            out["roofline"] = {"bound": "hbm", "kernel": "lans_apply", "achieved": round(achieved, 1),
+                               "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                               "traffic": MEASURED_TRAFFIC.get((name, "lans_apply")),
+                               "bytes_per_launch": total * c, "avg_launch_ms": round(apply_ms, 4)}
+            out["kernels_ms"] = {"lans_norm_g": round(float(avg[0]), 4), "lans_finish(a)": round(float(avg[1]), 4),
+                                 "lans_norm_u": round(float(avg[2]), 4), "lans_finish(b)": round(float(avg[3]), 4),
+                                 "lans_apply": round(apply_ms, 4)}
+            out["kernels_GBps"] = {"lans_norm_g": round(total * ka / avg[0] / 1e6, 1),
+                                   "lans_norm_u": round(total * kb / avg[2] / 1e6, 1),
+                                   "lans_apply": round(total * kc / avg[4] / 1e6, 1)}
+        else:
+            # one persistent kernel does all three passes
+            k_ms = float(avg[1])
+            achieved = bytes_step / (k_ms * 1e-3) / 1e9
+            out["roofline"] = {"bound": "hbm", "kernel": "lans_pipelined", "achieved": round(achieved, 1),
+                               "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                               "traffic": MEASURED_TRAFFIC.get((name, "lans_pipelined")),
+                               "bytes_per_launch": bytes_step, "avg_launch_ms": round(k_ms, 4)}
+            out["kernels_ms"] = {"lans_prepare": round(float(avg[0]), 4), "lans_pipelined": round(k_ms, 4)}
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline_lans(sizes, g16)
+    return out
+
+
+def bench_sgd(name, wl, args):
+    import torch
+
+    from raf_amd import kernels
+
+    dev = torch.device("cuda:0")
+    n = wl["n"]
+    # 84 MB per buffer set would sit in the 256 MB Infinity Cache: rotate over enough disjoint sets
+    # that every step streams from HBM.
+    sets = 8
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(2024)
+    bufs = []
+    for _ in range(sets):
+        x = torch.randn(n, device=dev, generator=gen) * 0.02
+        dx = torch.randn(n, device=dev, generator=gen) * 1e-3
+        v = torch.zeros(n, device=dev)
+        bufs.append((x, dx, v, torch.empty_like(x), torch.empty_like(x)))
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for i in range(args.warmup):
+        x, dx, v, v1, x1 = bufs[i % sets]
+        kernels.sgd_f32(x, dx, v, 0.01, 0.9, v_out=v1, x_out=x1)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(args.steps):
+        x, dx, v, v1, x1 = bufs[i % sets]
+        kernels.sgd_f32(x, dx, v, 0.01, 0.9, v_out=v1, x_out=x1)
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    dev_ms = start.elapsed_time(stop) / args.steps  # kernels run on torch's current stream
+    bytes_step = n * SGD_BYTES_PER_ELT
+    achieved = bytes_step / (dev_ms * 1e-3) / 1e9
+    out = {
+        "metric": "SGD momentum step achieved HBM bandwidth (algorithmic bytes / step time)",
+        "value": round(bytes_step / (ms_per_step * 1e-3) / 1e9, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": name, "elements": n, "bytes_per_element": SGD_BYTES_PER_ELT,
+                   "buffer_sets_rotated": sets},
+        "roofline": {"bound": "hbm", "kernel": "sgd_vec4_kernel", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC.get((name, "sgd_vec4_kernel")), "bytes_per_launch": bytes_step,
+                     "avg_launch_ms": round(dev_ms, 5)},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline_sgd(n)
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="lans_bert_large_fp16grad")
+    ap.add_argument("--schedule", default="phased", choices=["phased", "pipelined"],
+                    help="LANS launch schedule (bit-identical results)")
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline leg")
+    ap.add_argument("--no-kernel-events", action="store_true", help="do not record per-kernel HIP events")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this path is built and measured on ONE GPU (no collectives, no sharding); "
+                 "run with --gpus 1")
+    if args.steps < 1 or args.warmup < 0:
+        sys.exit("bench.py: --steps must be >= 1 and --warmup >= 0")
+    table = workloads()
+    if args.workload not in table:
+        sys.exit(f"bench.py: unknown workload {args.workload!r}; choose from {sorted(table)}")
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
+    from raf_amd import _lib
+
+    _lib.optim()  # fails loudly if the HIP library is not built
+    wl = table[args.workload]
+    out = bench_lans(args.workload, wl, args) if wl["kind"] == "lans" else bench_sgd(args.workload, wl, args)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

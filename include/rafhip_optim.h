@@ -101,12 +101,41 @@ typedef struct rafhip_lans_plan rafhip_lans_plan;
 int rafhip_lans_query_layout(int32_t n_tensors, const int64_t* numel, int64_t* n_chunks_out,
                              int64_t* workspace_bytes_out);
 
+/* Elements per chunk, the unit of work and of the per-chunk partial sums. */
+int32_t rafhip_lans_chunk_elements(void);
+
+/*
+ * Schedules of a step; both run the same per-chunk code and give bit-identical results.
+ *   PHASED     one launch per pass over all chunks of all tensors (set-up + 5 launches).
+ *   PIPELINED  set-up + ONE persistent launch whose work list interleaves the three passes of
+ *              neighbouring cache-sized tensor groups, so that a group's second and third reads
+ *              come from the 256 MB Infinity Cache instead of HBM.
+ * The default can be overridden per process with RAFHIP_LANS_SCHEDULE=phased|pipelined.
+ */
+typedef enum rafhip_lans_schedule {
+  RAFHIP_LANS_PHASED = 0,
+  RAFHIP_LANS_PIPELINED = 1
+} rafhip_lans_schedule;
+
+/*
+ * Pure host arithmetic: the work list of the pipelined schedule as int32 triples
+ * (kind, tensor, chunk), kind being 0 = pass A chunk, 1 = pass B chunk, 2 = pass C chunk,
+ * 3 = a one-chunk tensor taken through all three passes by one workgroup, 4 = finish pass A
+ * (add the tensor's partials, publish ||g||), 5 = finish pass B (publish ||w|| and the trust
+ * ratios).  group_elements <= 0 selects the default group size.  triples_out may be NULL to query
+ * the count.  The kernel's bounded waits rely on this order, per tensor: every pass-A chunk, then
+ * finish A, then every pass-B chunk, then finish B, then every pass-C chunk.
+ */
+int rafhip_lans_pipeline_order(int32_t n_tensors, const int64_t* numel, int64_t group_elements,
+                               int32_t* triples_out, int64_t capacity, int64_t* n_items_out);
+
 /* numel[i] >= 0 (zero-sized tensors are allowed and untouched); n_tensors >= 0. */
 int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t grad_dtype,
                             rafhip_lans_plan** out_plan);
 int rafhip_lans_plan_destroy(rafhip_lans_plan* plan);
+int rafhip_lans_plan_set_schedule(rafhip_lans_plan* plan, int32_t schedule);
 
-/* Bytes of caller-provided scratch a step needs (partial sums + per-tensor norms); 256-byte
+/* Bytes of caller-provided scratch a step needs (partial sums, per-tensor norms, flags); 256-byte
  * alignment required.  Returns a negative value on a NULL plan. */
 int64_t rafhip_lans_workspace_bytes(const rafhip_lans_plan* plan);
 int32_t rafhip_lans_plan_num_tensors(const rafhip_lans_plan* plan);
@@ -142,10 +171,21 @@ int rafhip_lans_read_norms(const rafhip_lans_plan* plan, const void* workspace, 
  * Optional per-kernel timing.  slots > 0 makes each following step record HIP events around its
  * five kernels on the step's stream into slot (step_index % slots); slots == 0 turns it off.
  * rafhip_lans_timing_read waits for that slot's last event and returns the five durations in
- * milliseconds: [0] norms of g,w  [1] finish  [2] norms of u_m,u_g  [3] finish  [4] apply.
+ * milliseconds.  Phased schedule: [0] norms of g,w  [1] finish  [2] norms of u_m,u_g  [3] finish
+ * [4] apply.  Pipelined schedule: [0] set-up  [1] the persistent kernel  [2..4] zero.
  */
 int rafhip_lans_timing_enable(rafhip_lans_plan* plan, int32_t slots);
 int rafhip_lans_timing_read(rafhip_lans_plan* plan, int32_t slot, float* ms_out5);
+
+/*
+ * Diagnostics of the pipelined schedule.  When the process runs with RAFHIP_LANS_TRACE=1, every
+ * pipelined step leaves four 64-bit words per work item, in work-list order: the 100 MHz device
+ * clock when the item was drawn, when its wait (if any) ended and when it finished, and the index
+ * of the workgroup that ran it.  n_items_out receives 0 when tracing is off.  Synchronises the
+ * device.
+ */
+int rafhip_lans_debug_trace(rafhip_lans_plan* plan, uint64_t* words_out, int64_t capacity_items,
+                            int64_t* n_items_out);
 
 #ifdef __cplusplus
 }

@@ -24,6 +24,9 @@ RAFHIP_ERR_NO_DEVICE = 5
 RAFHIP_F32 = 0
 RAFHIP_F16 = 1
 
+RAFHIP_LANS_PHASED = 0
+RAFHIP_LANS_PIPELINED = 1
+
 
 class RafHipError(RuntimeError):
     """A C-ABI call returned a non-zero status."""
@@ -60,6 +63,10 @@ OPTIM_SYMBOLS = {
     "rafhip_sgd_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_double,
                                c_double, c_void_p]),
     "rafhip_lans_default_hparams": (None, [POINTER(LansHParams)]),
+    "rafhip_lans_chunk_elements": (c_int32, []),
+    "rafhip_lans_pipeline_order": (c_int, [c_int32, POINTER(c_int64), c_int64, POINTER(c_int32), c_int64,
+                                           POINTER(c_int64)]),
+    "rafhip_lans_plan_set_schedule": (c_int, [c_void_p, c_int32]),
     "rafhip_lans_query_layout": (c_int, [c_int32, POINTER(c_int64), POINTER(c_int64),
                                          POINTER(c_int64)]),
     "rafhip_lans_plan_create": (c_int, [c_int32, POINTER(c_int64), c_int32, POINTER(c_void_p)]),
@@ -72,6 +79,7 @@ OPTIM_SYMBOLS = {
                                  POINTER(c_void_p), c_void_p, c_int32, POINTER(LansHParams),
                                  c_void_p, c_int64, c_void_p]),
     "rafhip_lans_read_norms": (c_int, [c_void_p, c_void_p, POINTER(c_double), c_void_p]),
+    "rafhip_lans_debug_trace": (c_int, [c_void_p, POINTER(ctypes.c_uint64), c_int64, POINTER(c_int64)]),
     "rafhip_lans_timing_enable": (c_int, [c_void_p, c_int32]),
     "rafhip_lans_timing_read": (c_int, [c_void_p, c_int32, POINTER(c_float)]),
 }

@@ -1,30 +1,43 @@
-// Device-side data layout and kernels of the multi-tensor LANS step for gfx950.
+// Device-side data layout and launchers of the multi-tensor LANS step for gfx950.
 //
 // Work decomposition.  Every tensor is cut into chunks of kChunk elements; the plan keeps, in HBM,
-// a tensor table (pointers, element count, first chunk) and a chunk table (tensor, index within
-// the tensor).  One workgroup handles one chunk per trip; a phase is ONE launch over all chunks of
-// all tensors, however many tensors there are.
+// a tensor table (pointers, element count, first chunk) and a work list of (phase, tensor, chunk)
+// items.  One workgroup handles one item at a time.
 //
-// A step is five launches on one stream:
-//   1. lans_norm_gw   read g,w            -> per-chunk partial sums of g^2 and w^2
-//   2. lans_finish_a  per tensor: add the chunk partials in a fixed order -> ||g||, ||w||,
-//                     1/(||g||+eps); also turns the device-resident step into bc1, bc2
-//   3. lans_norm_u    read g,w,m,v        -> per-chunk partial sums of u_m^2 and u_g^2
-//   4. lans_finish_b  per tensor: ||u_m||, ||u_g|| -> the two trust ratios
-//   5. lans_apply     read g,w,m,v, recompute the directions, write w,m,v
-// No per-element scratch exists: the two update directions are recomputed in 5 instead of being
-// stored (the reference stores them: 16 B/element of extra traffic plus a 4 B/element buffer).
+// The rule needs three passes over a tensor, separated by tensor-wide reductions:
+//   A  read g             -> per-chunk partial sums of g^2                  -> ||g||
+//   B  read g,w,m,v       -> per-chunk partial sums of u_m^2, u_g^2, w^2  -> ||w||, trust ratios
+//   C  read g,w,m,v, recompute the update directions, write w,m,v
+// No per-element scratch exists: the directions are recomputed in C instead of being stored (the
+// reference stores them: 16 B/element of extra traffic plus a 4 B/element buffer).
+//
+// Two schedules run the same per-chunk code and give bit-identical results:
+//   phased     five launches (A, finish, B, finish, C), each over all chunks of all tensors.
+//   pipelined  one small set-up launch plus ONE persistent launch.  Tensors are packed into groups
+//              whose working set is a fraction of the 256 MB Infinity Cache, and the work list
+//              interleaves pass A of group s with pass B of group s-1 and pass C of group s-2, so a
+//              group's second and third reads are served by the cache instead of HBM.  Workgroups
+//              draw items from an atomic ticket.  Chunk items of pass A and B just store their
+//              partial sums; a "finish" item per tensor and pass, placed after them in the list,
+//              waits for those partials, adds them and publishes the tensor's statistics; items of
+//              pass B (C) wait for the statistics they need.  All waiting is on single 8-byte words
+//              that go from a "not ready" pattern to their final value exactly once per step, so
+//              no counters, flags or fences are involved.  Every item a waiter depends on has an
+//              earlier ticket and is therefore already held by a running workgroup, so the waits
+//              always end; they are bounded anyway, and a time-out raises an error flag instead
+//              of hanging.
 //
 // Determinism.  A chunk's partial sum depends only on the chunk (fixed lane order, fixed wave
-// tree), and the per-tensor finish adds the partials in a fixed order, so results are bit-identical
-// from run to run and independent of the grid size.  No atomics anywhere.
+// tree); a tensor's total adds its chunk partials in a fixed order whichever workgroup does it.
+// Results are bit-identical from run to run, across grid sizes and across the two schedules.
+// Atomics are used for tickets, counters and flags only, never to accumulate values.
 //
 // Arithmetic.  Loads and stores are fp32 (fp16 for the optional half gradients); every
 // per-element operation and every accumulation is float64, rounded once on store.  The weight
 // update subtracts a ~1e-5-sized step from the weight, so an fp32 evaluation of the step (or of the
 // norms behind the trust ratio) would leave errors far above 1e-5 *relative* on the weights that
-// land near zero; float64 keeps every element within an fp32 ulp of the exactly rounded rule.
-// gfx950 issues FP64 FMAs at the full vector rate, and the kernels stay HBM-bound.
+// land near zero.  gfx950 issues FP64 FMAs at the full vector rate; square root and reciprocal are
+// the hardware approximations (2^-24) plus one Newton step (2^-47), ample for an fp32 result.
 #pragma once
 #include <hip/hip_runtime.h>
 
@@ -32,10 +45,11 @@
 
 namespace rafhip {
 
-constexpr int kLansBlock = 256;                 // 4 wavefronts
+constexpr int kLansBlock = 256;  // 4 wavefronts
 constexpr int kLansWaves = kLansBlock / 64;
-constexpr int kChunk = 16384;                   // elements per chunk (multiple of 4 * kLansBlock)
-constexpr int kUnroll = 2;                      // 4-element groups in flight per lane per trip
+constexpr int kChunk = 8192;     // elements per chunk (multiple of 4 * kLansBlock)
+constexpr int kUnroll = 2;       // 4-element groups in flight per lane per trip
+constexpr int kPartialSlots = 4; // doubles per chunk: [0] sum g^2 | [1] sum u_m^2 [2] sum u_g^2 [3] sum w^2
 
 struct TensorRec {  // 48 bytes, one per tensor
   const void* g;
@@ -44,48 +58,78 @@ struct TensorRec {  // 48 bytes, one per tensor
   float* v;
   int64_t numel;
   int32_t first_chunk;
-  int32_t vec_ok;  // 1: every base pointer allows 128-bit (fp16 g: 64-bit) lane accesses
+  int32_t vec_ok;  // 1: every base pointer is 16-byte aligned: 128-bit lane accesses
 };
 
-struct ChunkRec {  // 8 bytes, one per chunk
+// One unit of work: kind in the top three bits of `chunk_phase`, chunk number within the tensor
+// below.  A/B/C: one chunk of that pass.  FinishA/FinishB: add the tensor's chunk partials of the
+// pass and publish its statistics.  Whole: a one-chunk tensor taken through all three passes by
+// one workgroup.
+enum : uint32_t {
+  kPhaseA = 0,
+  kPhaseB = 1,
+  kPhaseC = 2,
+  kPhaseWhole = 3,
+  kPhaseFinishA = 4,
+  kPhaseFinishB = 5
+};
+struct WorkItem {
   int32_t tensor;
-  int32_t index;  // chunk number inside its tensor
+  uint32_t chunk_phase;
 };
+constexpr uint32_t kPhaseShift = 29;
+constexpr uint32_t kChunkMask = (1u << kPhaseShift) - 1;
 
-// Global scalars of a step, produced on the device by lans_finish_a (256 bytes reserved).
+// Global scalars of a step, produced on the device from the step tensor (256 bytes reserved).
 struct StepScalars {
   double beta1, beta2, one_minus_beta2, beta3;
   double eps, wd, inv_bc1, inv_bc2;
   double lr;
-  int32_t mode;
+  double decay_into_grad;  // 1 in L2 mode (decay joins the scaled gradient), else 0
+  double decay_into_dir;   // 1 in decoupled mode (decay is added to both directions), else 0
+  int32_t normalize_grad;
   int32_t pad;
 };
 
-struct TensorStats {  // 64 bytes, one per tensor
+struct TensorStats {  // 64 bytes = 8 words, one per tensor; "not ready" pattern until published
   double grad_norm, param_norm, inv_grad_div;  // inv_grad_div = 1/(||g||+eps) or 1
   double um_norm, ug_norm;
   double ratio_m, ratio_g;  // beta1 * trust ratio of u_m, beta3 * trust ratio of u_g
   double reserved;
 };
 
-// Host-side copy of the hyper-parameters handed to lans_finish_a by value.
+// Synchronisation words of the pipelined schedule; reset by the set-up launch of every step.
+struct SyncHeader {
+  uint32_t ticket;  // next work item
+  uint32_t error;   // 1 if a bounded wait ran out
+  uint32_t pad[2];
+};
+
 struct HParamsPod {
   float learning_rate, beta1, beta2, eps, weight_decay;
   int32_t bias_correction, grad_averaging, mode, normalize_grad;
 };
 
-void launch_norm_gw(int grad_dtype, unsigned grid, hipStream_t s, const TensorRec* tensors,
-                    const ChunkRec* chunks, int64_t n_chunks, float unscale, double* partials);
-void launch_finish_a(unsigned grid, hipStream_t s, const TensorRec* tensors, int32_t n_tensors,
-                     const double* partials, TensorStats* stats, StepScalars* scalars,
-                     const float* step_dev, int32_t step_host, HParamsPod hp);
-void launch_norm_u(int grad_dtype, unsigned grid, hipStream_t s, const TensorRec* tensors,
-                   const ChunkRec* chunks, int64_t n_chunks, float unscale,
-                   const StepScalars* scalars, const TensorStats* stats, double* partials);
-void launch_finish_b(unsigned grid, hipStream_t s, const TensorRec* tensors, int32_t n_tensors,
-                     const double* partials, TensorStats* stats, const StepScalars* scalars);
-void launch_apply(int grad_dtype, unsigned grid, hipStream_t s, const TensorRec* tensors,
-                  const ChunkRec* chunks, int64_t n_chunks, float unscale,
-                  const StepScalars* scalars, const TensorStats* stats);
+struct LansDeviceArgs {
+  const TensorRec* tensors;
+  int32_t n_tensors;
+  const WorkItem* items;  // phased: [A items][B items][C items], each n_chunks long
+  int64_t n_chunks;
+  uint32_t n_items;       // pipelined work-list length
+  const WorkItem* pipeline_items;
+  float unscale;
+  StepScalars* scalars;
+  TensorStats* stats;
+  double* partials;       // kPartialSlots doubles per chunk
+  SyncHeader* sync;
+  uint64_t* trace;        // optional diagnostics: 4 words per pipelined item, or nullptr
+};
+
+void launch_prepare(hipStream_t s, const LansDeviceArgs& a, const float* step_dev,
+                    int32_t step_host, HParamsPod hp);
+void launch_phased(int grad_dtype, hipStream_t s, const LansDeviceArgs& a, hipEvent_t* marks);
+void launch_pipelined(int grad_dtype, unsigned grid, hipStream_t s, const LansDeviceArgs& a);
+// Resident workgroups per CU of the pipelined kernel (occupancy query), 0 on failure.
+int pipelined_blocks_per_cu(int grad_dtype);
 
 }  // namespace rafhip

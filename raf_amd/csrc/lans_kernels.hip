@@ -1,45 +1,70 @@
-// gfx950 kernels of the multi-tensor LANS step; layout and phase order are described in
+// gfx950 kernels of the multi-tensor LANS step; layout, schedules and numerics are described in
 // lans_kernels.h.  The rule follows the reference's fp32 CUDA functors
 // (src/op/dialect/cuda/kernels/multi_tensor_lans.cu:283-307 stage 1, :346-352 and :386 stage 2,
-// :95-185 norms) evaluated in float64.
+// :95-185 norms; host scalars src/op/dialect/cuda/lans.cc:94-109) evaluated in float64.
 #include "lans_kernels.h"
-
-#include <hip/hip_fp16.h>
 
 #include "rafhip_optim.h"
 
 namespace rafhip {
 namespace {
 
+// Global-address-space views: tensor pointers come out of a table in memory, so without these the
+// compiler falls back to flat (generic) loads and stores.
+#define RAFHIP_GLOBAL __attribute__((address_space(1)))
+typedef float f32x4 __attribute__((ext_vector_type(4)));  // native vector: HIP's f32x4 is a class
+typedef RAFHIP_GLOBAL const f32x4 gc_float4;
+typedef RAFHIP_GLOBAL f32x4 g_float4;
+typedef RAFHIP_GLOBAL const float gc_float;
+typedef RAFHIP_GLOBAL float g_float;
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef RAFHIP_GLOBAL const half4_t gc_half4;
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef RAFHIP_GLOBAL const half8_t gc_half8;
+typedef RAFHIP_GLOBAL const _Float16 gc_half;
 
 // ------------------------------------------------------------------ gradient ingest
-// Four consecutive gradients as fp32, already multiplied by the unscale factor (one fp32 rounding,
-// exact for power-of-two loss scales).
+// Gradients as fp32, already multiplied by the unscale factor (one fp32 rounding, exact for
+// power-of-two loss scales).
 template <typename G>
 struct GradIO;
 
 template <>
 struct GradIO<float> {
-  static __device__ __forceinline__ float4 load4(const float* g, int i4, float us) {
-    const float4 r = reinterpret_cast<const float4*>(g)[i4];
-    return make_float4(__fmul_rn(r.x, us), __fmul_rn(r.y, us), __fmul_rn(r.z, us),
-                       __fmul_rn(r.w, us));
+  // Widest single-lane access used when the gradient is the only array read (pass A): 16 bytes.
+  static constexpr int kWide = 4;
+  static __device__ __forceinline__ void load_wide(const void* g, int iw, float us,
+                                                   float (&out)[kWide]) {
+    const f32x4 r = ((gc_float4*)g)[iw];
+    out[0] = r.x * us;
+    out[1] = r.y * us;
+    out[2] = r.z * us;
+    out[3] = r.w * us;
   }
-  static __device__ __forceinline__ float load1(const float* g, int i, float us) {
-    return __fmul_rn(g[i], us);
+  static __device__ __forceinline__ f32x4 load4(const void* g, int i4, float us) {
+    const f32x4 r = ((gc_float4*)g)[i4];
+    return f32x4{r.x * us, r.y * us, r.z * us, r.w * us};
+  }
+  static __device__ __forceinline__ float load1(const void* g, int i, float us) {
+    return ((gc_float*)g)[i] * us;
   }
 };
 
 template <>
 struct GradIO<_Float16> {
-  static __device__ __forceinline__ float4 load4(const _Float16* g, int i4, float us) {
-    const half4_t r = reinterpret_cast<const half4_t*>(g)[i4];
-    return make_float4(__fmul_rn((float)r.x, us), __fmul_rn((float)r.y, us),
-                       __fmul_rn((float)r.z, us), __fmul_rn((float)r.w, us));
+  static constexpr int kWide = 8;
+  static __device__ __forceinline__ void load_wide(const void* g, int iw, float us,
+                                                   float (&out)[kWide]) {
+    const half8_t r = ((gc_half8*)g)[iw];
+#pragma unroll
+    for (int j = 0; j < kWide; ++j) out[j] = (float)r[j] * us;
   }
-  static __device__ __forceinline__ float load1(const _Float16* g, int i, float us) {
-    return __fmul_rn((float)g[i], us);
+  static __device__ __forceinline__ f32x4 load4(const void* g, int i4, float us) {
+    const half4_t r = ((gc_half4*)g)[i4];
+    return f32x4{(float)r.x * us, (float)r.y * us, (float)r.z * us, (float)r.w * us};
+  }
+  static __device__ __forceinline__ float load1(const void* g, int i, float us) {
+    return (float)((gc_half*)g)[i] * us;
   }
 };
 
@@ -51,55 +76,153 @@ __device__ __forceinline__ double wave_sum(double x) {
   return x;
 }
 
-// Block-wide sums of two values; results valid in thread 0.  `red` is [2][kLansWaves] doubles of
-// LDS.  The leading barrier makes the helper safe to call once per trip of a chunk loop.
-__device__ __forceinline__ void block_sum2(double& a, double& b, double (*red)[kLansWaves]) {
-  a = wave_sum(a);
-  b = wave_sum(b);
+// Block-wide sums of N values, returned to every thread.  `red` is [3][kLansWaves] doubles of
+// LDS.  The leading barrier makes the helper safe to call repeatedly on the same LDS.
+template <int N>
+__device__ __forceinline__ void block_sum(double (&x)[N], double (*red)[kLansWaves]) {
+  static_assert(N <= 3, "red holds three rows");
+#pragma unroll
+  for (int j = 0; j < N; ++j) x[j] = wave_sum(x[j]);
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   __syncthreads();
   if (lane == 0) {
-    red[0][wave] = a;
-    red[1][wave] = b;
+#pragma unroll
+    for (int j = 0; j < N; ++j) red[j][wave] = x[j];
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    double sa = red[0][0], sb = red[1][0];
 #pragma unroll
-    for (int k = 1; k < kLansWaves; ++k) {
-      sa += red[0][k];
-      sb += red[1][k];
-    }
-    a = sa;
-    b = sb;
+  for (int j = 0; j < N; ++j) {
+    double s = red[j][0];
+#pragma unroll
+    for (int k = 1; k < kLansWaves; ++k) s += red[j][k];
+    x[j] = s;
   }
 }
 
+// Loads/stores that are coherent across the whole device (they go past the per-XCD L2), used for
+// the few words that workgroups exchange inside the persistent kernel.  Because every exchanged
+// word moves this way, the kernel never needs a device-scope fence (which would write back and
+// invalidate a whole L2 while other workgroups stream through it): "publish, then signal" only has
+// to wait for the publishing stores to complete, which a workgroup-scope release fence does.
+__device__ __forceinline__ double ld_dev(const double* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_dev(double* p, double v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+constexpr uint64_t kNotReady = 0xFFFFFFFFFFFFFFFFull;
+constexpr uint32_t kSpinLimit = 1u << 22;  // bounded wait: far beyond any real dependency latency
+
+__device__ __forceinline__ uint64_t ld_bits(const double* p) {
+  return __hip_atomic_load(reinterpret_cast<const uint64_t*>(p), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Words that travel between workgroups of the pipelined schedule (chunk partials, per-tensor
+// statistics) double as their own "ready" flags: the set-up launch fills them with kNotReady (a
+// NaN pattern no computation produces, because published values are canonicalised), each is
+// written exactly once per step with a single 8-byte store, and a consumer re-reads a word until
+// it differs.  No ordering between words is needed.  A wait that runs out raises the error word
+// and returns whatever is there, so the grid always drains.
+__device__ __forceinline__ void publish(double* p, double v) {
+  st_dev(p, v != v ? __builtin_nan("") : v);
+}
+__device__ __forceinline__ double wait_published(const double* word, SyncHeader* sync) {
+  uint64_t bits = ld_bits(word);
+  uint32_t spins = 0;
+  while (bits == kNotReady) {
+    if (++spins > kSpinLimit) {
+      __hip_atomic_store(&sync->error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      break;
+    }
+    __builtin_amdgcn_s_sleep(8);
+    bits = ld_bits(word);
+  }
+  return __longlong_as_double((long long)bits);
+}
+
+// Several words at once: all loads are issued together, and only words that were not ready are
+// read again.
+template <int N>
+__device__ __forceinline__ void wait_published_n(const double* const (&words)[N], double (&out)[N],
+                                                 SyncHeader* sync) {
+  uint64_t bits[N];
+#pragma unroll
+  for (int j = 0; j < N; ++j) bits[j] = ld_bits(words[j]);
+#pragma unroll
+  for (int j = 0; j < N; ++j)
+    out[j] = bits[j] != kNotReady ? __longlong_as_double((long long)bits[j])
+                                  : wait_published(words[j], sync);
+}
+
+// A tensor's totals from its chunk partials (kPartialSlots doubles per chunk, N of them starting
+// at `slot`): thread t adds chunks t, t+256, ... in order, then the fixed block tree.  The order
+// depends on nothing but the chunk count.  With kWait the partials are awaited one by one.
+template <int N, bool kWait>
+__device__ __forceinline__ void tensor_totals(const double* partials, int slot, int64_t n_chunks,
+                                              double (&tot)[N], double (*red)[kLansWaves],
+                                              SyncHeader* sync) {
+#pragma unroll
+  for (int j = 0; j < N; ++j) tot[j] = 0.0;
+  for (int64_t i = threadIdx.x; i < n_chunks; i += kLansBlock) {
+    const double* p = partials + kPartialSlots * i + slot;
+    if (kWait) {
+      const double* words[N];
+      double val[N];
+#pragma unroll
+      for (int j = 0; j < N; ++j) words[j] = p + j;
+      wait_published_n<N>(words, val, sync);
+#pragma unroll
+      for (int j = 0; j < N; ++j) tot[j] += val[j];
+    } else {
+#pragma unroll
+      for (int j = 0; j < N; ++j) tot[j] += ld_dev(p + j);
+    }
+  }
+  block_sum<N>(tot, red);
+}
+
 // ------------------------------------------------------------------ the rule, per element
+// sqrt(x) for x >= 0: hardware rsq (2^-24) and one coupled Newton step (2^-47).  The clamp keeps
+// x == 0 exact (0 * rsq(tiny) = 0) without a branch.
+__device__ __forceinline__ double sqrt_nonneg(double x) {
+  const double y = __builtin_amdgcn_rsq(fmax(x, 1e-300));
+  const double g = x * y;
+  const double h = 0.5 * y;
+  const double r = __builtin_fma(-h, g, 0.5);
+  return __builtin_fma(g, r, g);
+}
+
+// 1/d: hardware rcp (2^-24), one Newton step, then div_fixup restores the IEEE results for the
+// special operands (1/0 = inf, 1/inf = 0, NaN).
+__device__ __forceinline__ double reciprocal(double d) {
+  const double r0 = __builtin_amdgcn_rcp(d);
+  const double e = __builtin_fma(-d, r0, 1.0);
+  const double r1 = __builtin_fma(r0, e, r0);
+  return __builtin_amdgcn_div_fixup(r1, d, 1.0);
+}
+
 struct Directions {
   double m1, v1, um, ug;
 };
 
 // Stage 1 of the rule for one element (multi_tensor_lans.cu:283-307).  inv_gdiv is
-// 1/(||g||+eps) when the gradient is normalised and 1 otherwise.
+// 1/(||g||+eps) when the gradient is normalised and 1 otherwise.  The two decay switches fold the
+// L2 / decoupled modes into multiplications by 0 or 1.
 __device__ __forceinline__ Directions lans_directions(double g, double w, double m, double v,
                                                       double inv_gdiv, const StepScalars& k) {
-  double sg = g * inv_gdiv;
   const double wp = (k.wd != 0.0) ? w : 0.0;  // reference skips the weight when wd == 0 (:264-269)
   const double decay = k.wd * wp;
-  double sp = decay;
-  if (k.mode == 0) {  // L2 mode: decay joins the scaled gradient, nothing is added afterwards
-    sg += decay;
-    sp = 0.0;
-  }
+  const double sg = __builtin_fma(k.decay_into_grad, decay, g * inv_gdiv);
+  const double sp = k.decay_into_dir * decay;
   Directions d;
-  d.m1 = m * k.beta1 + k.beta3 * sg;
-  d.v1 = v * k.beta2 + k.one_minus_beta2 * sg * sg;
-  const double den = sqrt(d.v1 * k.inv_bc2) + k.eps;
-  const double inv_den = 1.0 / den;
-  d.um = (d.m1 * k.inv_bc1) * inv_den + sp;
-  d.ug = sg * inv_den + sp;
+  d.m1 = __builtin_fma(k.beta3, sg, m * k.beta1);
+  d.v1 = __builtin_fma(k.one_minus_beta2 * sg, sg, v * k.beta2);
+  const double inv_den = reciprocal(sqrt_nonneg(d.v1 * k.inv_bc2) + k.eps);
+  d.um = __builtin_fma(d.m1 * k.inv_bc1, inv_den, sp);
+  d.ug = __builtin_fma(sg, inv_den, sp);
   return d;
 }
 
@@ -108,16 +231,13 @@ struct ChunkView {
   float* w;
   float* m;
   float* v;
-  int len;     // elements in this chunk
+  int len;  // elements in this chunk
   int vec_ok;
-  int tensor;
 };
 
-__device__ __forceinline__ ChunkView chunk_view(const TensorRec* tensors, const ChunkRec* chunks,
-                                                int64_t c, int g_elem_bytes) {
-  const ChunkRec cr = chunks[c];
-  const TensorRec tr = tensors[cr.tensor];
-  const int64_t base = (int64_t)cr.index * kChunk;
+__device__ __forceinline__ ChunkView chunk_view(const TensorRec& tr, uint32_t chunk,
+                                                int g_elem_bytes) {
+  const int64_t base = (int64_t)chunk * kChunk;
   const int64_t rest = tr.numel - base;
   ChunkView cv;
   cv.g = static_cast<const char*>(tr.g) + base * g_elem_bytes;
@@ -126,338 +246,499 @@ __device__ __forceinline__ ChunkView chunk_view(const TensorRec* tensors, const 
   cv.v = tr.v + base;
   cv.len = rest < kChunk ? (int)rest : kChunk;
   cv.vec_ok = tr.vec_ok;
-  cv.tensor = cr.tensor;
   return cv;
 }
 
-// ------------------------------------------------------------------ phase 1: sum g^2, sum w^2
+// ------------------------------------------------------------------ pass A on one chunk
+// Per-thread contribution to sum g^2 (block reduction is the caller's).  Only the gradient is read:
+// ||w|| is not needed before the trust ratios, so its sum rides along with pass B.
 template <typename G>
-__global__ __launch_bounds__(kLansBlock) void lans_norm_gw(const TensorRec* __restrict__ tensors,
-                                                           const ChunkRec* __restrict__ chunks,
-                                                           int64_t n_chunks, float unscale,
-                                                           double* __restrict__ partials) {
-  __shared__ double red[2][kLansWaves];
-  for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
-    const ChunkView cv = chunk_view(tensors, chunks, c, (int)sizeof(G));
-    const G* g = static_cast<const G*>(cv.g);
-    double ag[4] = {0.0, 0.0, 0.0, 0.0}, aw[4] = {0.0, 0.0, 0.0, 0.0};
-    if (cv.vec_ok) {
-      const int n4 = cv.len >> 2;
-      for (int i0 = threadIdx.x; i0 < n4; i0 += kLansBlock * kUnroll) {
-        float4 gv[kUnroll], wv[kUnroll];
+__device__ __forceinline__ double chunk_sum_g(const ChunkView& cv, float unscale) {
+  constexpr int kW = GradIO<G>::kWide;  // elements per 16-byte lane access
+  constexpr int kU = 4;                 // accesses in flight per lane per trip
+  double acc[4] = {0.0, 0.0, 0.0, 0.0};
+  if (cv.vec_ok) {
+    const int nw = cv.len / kW;
+    for (int i0 = threadIdx.x; i0 < nw; i0 += kLansBlock * kU) {
+      float x[kU][kW];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-          const int i = i0 + u * kLansBlock;
-          if (i < n4) {
-            gv[u] = GradIO<G>::load4(g, i, unscale);
-            wv[u] = reinterpret_cast<const float4*>(cv.w)[i];
-          } else {
-            gv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-            wv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-          }
-        }
+      for (int u = 0; u < kU; ++u) {
+        const int i = i0 + u * kLansBlock;
+        if (i < nw) {
+          GradIO<G>::load_wide(cv.g, i, unscale, x[u]);
+        } else {
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-          ag[0] += (double)gv[u].x * (double)gv[u].x;
-          ag[1] += (double)gv[u].y * (double)gv[u].y;
-          ag[2] += (double)gv[u].z * (double)gv[u].z;
-          ag[3] += (double)gv[u].w * (double)gv[u].w;
-          aw[0] += (double)wv[u].x * (double)wv[u].x;
-          aw[1] += (double)wv[u].y * (double)wv[u].y;
-          aw[2] += (double)wv[u].z * (double)wv[u].z;
-          aw[3] += (double)wv[u].w * (double)wv[u].w;
+          for (int j = 0; j < kW; ++j) x[u][j] = 0.f;
         }
       }
-      const int tail = (n4 << 2) + threadIdx.x;  // the < 4 leftover elements of a last chunk
-      if (tail < cv.len) {
-        const double gx = GradIO<G>::load1(g, tail, unscale), wx = cv.w[tail];
-        ag[0] += gx * gx;
-        aw[0] += wx * wx;
-      }
-    } else {
-      for (int i = threadIdx.x; i < cv.len; i += kLansBlock) {
-        const double gx = GradIO<G>::load1(g, i, unscale), wx = cv.w[i];
-        ag[0] += gx * gx;
-        aw[0] += wx * wx;
-      }
+#pragma unroll
+      for (int u = 0; u < kU; ++u)
+#pragma unroll
+        for (int j = 0; j < kW; ++j) acc[j & 3] += (double)x[u][j] * (double)x[u][j];
     }
-    double sg = (ag[0] + ag[1]) + (ag[2] + ag[3]);
-    double sw = (aw[0] + aw[1]) + (aw[2] + aw[3]);
-    block_sum2(sg, sw, red);
-    if (threadIdx.x == 0) {
-      partials[2 * c] = sg;
-      partials[2 * c + 1] = sw;
+    const int tail = nw * kW + threadIdx.x;  // the < kW leftover elements of a last chunk
+    if (tail < cv.len) {
+      const double gx = GradIO<G>::load1(cv.g, tail, unscale);
+      acc[0] += gx * gx;
+    }
+  } else {
+    for (int i = threadIdx.x; i < cv.len; i += kLansBlock) {
+      const double gx = GradIO<G>::load1(cv.g, i, unscale);
+      acc[0] += gx * gx;
+    }
+  }
+  return (acc[0] + acc[1]) + (acc[2] + acc[3]);
+}
+
+// ------------------------------------------------------------------ passes B and C: shared loads
+// One trip's worth of the four arrays for one lane: kUnroll groups of 4 consecutive elements.
+struct Batch {
+  f32x4 g[kUnroll], w[kUnroll], m[kUnroll], v[kUnroll];
+};
+
+template <typename G>
+__device__ __forceinline__ void load_batch(Batch& b, const ChunkView& cv, int i0, int n4,
+                                           float unscale) {
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    const int i = i0 + u * kLansBlock;
+    if (i < n4) {
+      b.g[u] = GradIO<G>::load4(cv.g, i, unscale);
+      b.w[u] = ((gc_float4*)cv.w)[i];
+      b.m[u] = ((gc_float4*)cv.m)[i];
+      b.v[u] = ((gc_float4*)cv.v)[i];
     }
   }
 }
 
-// ------------------------------------------------------------------ phases 2 and 4: per-tensor finish
-// One wavefront per tensor adds that tensor's chunk partials: lane l takes chunks l, l+64, ... in
-// order, then the fixed butterfly.  The order depends on nothing but the chunk count.
-__device__ __forceinline__ void tensor_totals(const TensorRec& tr, const double* partials,
-                                              int lane, double& a, double& b) {
-  const int64_t n_chunks = (tr.numel + kChunk - 1) / kChunk;
-  const double* p = partials + 2 * (int64_t)tr.first_chunk;
-  a = 0.0;
-  b = 0.0;
-  for (int64_t i = lane; i < n_chunks; i += 64) {
-    a += p[2 * i];
-    b += p[2 * i + 1];
-  }
-  a = wave_sum(a);
-  b = wave_sum(b);
-}
-
-__global__ __launch_bounds__(kLansBlock) void lans_finish_a(
-    const TensorRec* __restrict__ tensors, int32_t n_tensors, const double* __restrict__ partials,
-    TensorStats* __restrict__ stats, StepScalars* __restrict__ scalars,
-    const float* __restrict__ step_dev, int32_t step_host, HParamsPod hp) {
-  const int t = (int)((blockIdx.x * (unsigned)kLansBlock + threadIdx.x) >> 6);
-  const int lane = threadIdx.x & 63;
-  if (t < n_tensors) {
-    double sg, sw;
-    tensor_totals(tensors[t], partials, lane, sg, sw);
-    if (lane == 0) {
-      const double gn = sqrt(sg), pn = sqrt(sw);
-      TensorStats st;
-      st.grad_norm = gn;
-      st.param_norm = pn;
-      // multi_tensor_lans.cu:284-286: divide only when normalising and the norm is non-zero
-      st.inv_grad_div = (hp.normalize_grad && gn != 0.0) ? 1.0 / (gn + (double)hp.eps) : 1.0;
-      st.um_norm = st.ug_norm = st.ratio_m = st.ratio_g = st.reserved = 0.0;
-      stats[t] = st;
+// ------------------------------------------------------------------ pass B on one chunk
+// Per-thread contributions to sum u_m^2, sum u_g^2 and sum w^2.  `get_inv_gdiv` supplies the
+// tensor's gradient divisor (the pipelined schedule may have to wait for it).
+// (Issuing trip i+1's loads before evaluating trip i was tried: the extra registers cost a wave of
+// occupancy and the kernels got slower.)
+template <typename G, typename GetInvGdiv>
+__device__ __forceinline__ void chunk_sums_u(const ChunkView& cv, float unscale,
+                                             const StepScalars& k, GetInvGdiv&& get_inv_gdiv,
+                                             double (&sums)[3]) {
+  double am = 0.0, au = 0.0, aw = 0.0;
+  if (cv.vec_ok) {
+    const int n4 = cv.len >> 2;
+    constexpr int kStride = kLansBlock * kUnroll;
+    const double inv_gdiv = get_inv_gdiv();
+    for (int i0 = threadIdx.x; i0 < n4; i0 += kStride) {
+      Batch cur;
+      load_batch<G>(cur, cv, i0, n4, unscale);
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        if (i0 + u * kLansBlock < n4) {
+          const Directions d0 = lans_directions(cur.g[u].x, cur.w[u].x, cur.m[u].x, cur.v[u].x, inv_gdiv, k);
+          const Directions d1 = lans_directions(cur.g[u].y, cur.w[u].y, cur.m[u].y, cur.v[u].y, inv_gdiv, k);
+          const Directions d2 = lans_directions(cur.g[u].z, cur.w[u].z, cur.m[u].z, cur.v[u].z, inv_gdiv, k);
+          const Directions d3 = lans_directions(cur.g[u].w, cur.w[u].w, cur.m[u].w, cur.v[u].w, inv_gdiv, k);
+          am += (d0.um * d0.um + d1.um * d1.um) + (d2.um * d2.um + d3.um * d3.um);
+          au += (d0.ug * d0.ug + d1.ug * d1.ug) + (d2.ug * d2.ug + d3.ug * d3.ug);
+          aw += ((double)cur.w[u].x * (double)cur.w[u].x + (double)cur.w[u].y * (double)cur.w[u].y) +
+                ((double)cur.w[u].z * (double)cur.w[u].z + (double)cur.w[u].w * (double)cur.w[u].w);
+        }
+      }
+    }
+    const int tail = (n4 << 2) + threadIdx.x;
+    if (tail < cv.len) {
+      const double wx = ((gc_float*)cv.w)[tail];
+      const Directions d = lans_directions(GradIO<G>::load1(cv.g, tail, unscale), wx,
+                                           ((gc_float*)cv.m)[tail], ((gc_float*)cv.v)[tail],
+                                           inv_gdiv, k);
+      am += d.um * d.um;
+      au += d.ug * d.ug;
+      aw += wx * wx;
+    }
+  } else {
+    const double inv_gdiv = get_inv_gdiv();
+    for (int i = threadIdx.x; i < cv.len; i += kLansBlock) {
+      const double wx = ((gc_float*)cv.w)[i];
+      const Directions d = lans_directions(GradIO<G>::load1(cv.g, i, unscale), wx,
+                                           ((gc_float*)cv.m)[i], ((gc_float*)cv.v)[i], inv_gdiv, k);
+      am += d.um * d.um;
+      au += d.ug * d.ug;
+      aw += wx * wx;
     }
   }
-  if (blockIdx.x == 0 && threadIdx.x == 0) {
-    // Host scalars of the reference (src/op/dialect/cuda/lans.cc:94-109), evaluated on the device so
-    // the step tensor never has to be copied to the host.
+  sums[0] = am;
+  sums[1] = au;
+  sums[2] = aw;
+}
+
+// ------------------------------------------------------------------ pass C on one chunk
+struct Applied {
+  float w, m, v;
+};
+
+struct ApplyParams {
+  double inv_gdiv, rm, rg;
+};
+
+__device__ __forceinline__ Applied apply_one(double g, double w, double m, double v,
+                                             const ApplyParams& p, const StepScalars& k) {
+  const Directions d = lans_directions(g, w, m, v, p.inv_gdiv, k);
+  Applied o;
+  // multi_tensor_lans.cu:386: p - ratio_m*update_m - ratio_g*update_g, left to right
+  o.w = (float)__builtin_fma(-p.rg, d.ug, __builtin_fma(-p.rm, d.um, w));
+  o.m = (float)d.m1;
+  o.v = (float)d.v1;
+  return o;
+}
+
+// `get_params` supplies the tensor's divisor and trust ratios.
+template <typename G, typename GetParams>
+__device__ __forceinline__ void chunk_apply(const ChunkView& cv, float unscale,
+                                            const StepScalars& k, GetParams&& get_params) {
+  if (cv.vec_ok) {
+    const int n4 = cv.len >> 2;
+    constexpr int kStride = kLansBlock * kUnroll;
+    const ApplyParams p = get_params();
+    for (int i0 = threadIdx.x; i0 < n4; i0 += kStride) {
+      Batch cur;
+      load_batch<G>(cur, cv, i0, n4, unscale);
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int i = i0 + u * kLansBlock;
+        if (i < n4) {
+          const Applied a0 = apply_one(cur.g[u].x, cur.w[u].x, cur.m[u].x, cur.v[u].x, p, k);
+          const Applied a1 = apply_one(cur.g[u].y, cur.w[u].y, cur.m[u].y, cur.v[u].y, p, k);
+          const Applied a2 = apply_one(cur.g[u].z, cur.w[u].z, cur.m[u].z, cur.v[u].z, p, k);
+          const Applied a3 = apply_one(cur.g[u].w, cur.w[u].w, cur.m[u].w, cur.v[u].w, p, k);
+          ((g_float4*)cv.w)[i] = f32x4{a0.w, a1.w, a2.w, a3.w};
+          ((g_float4*)cv.m)[i] = f32x4{a0.m, a1.m, a2.m, a3.m};
+          ((g_float4*)cv.v)[i] = f32x4{a0.v, a1.v, a2.v, a3.v};
+        }
+      }
+    }
+    const int tail = (n4 << 2) + threadIdx.x;
+    if (tail < cv.len) {
+      const Applied o = apply_one(GradIO<G>::load1(cv.g, tail, unscale), ((gc_float*)cv.w)[tail],
+                                  ((gc_float*)cv.m)[tail], ((gc_float*)cv.v)[tail], p, k);
+      ((g_float*)cv.w)[tail] = o.w;
+      ((g_float*)cv.m)[tail] = o.m;
+      ((g_float*)cv.v)[tail] = o.v;
+    }
+  } else {
+    const ApplyParams p = get_params();
+    for (int i = threadIdx.x; i < cv.len; i += kLansBlock) {
+      const Applied o = apply_one(GradIO<G>::load1(cv.g, i, unscale), ((gc_float*)cv.w)[i],
+                                  ((gc_float*)cv.m)[i], ((gc_float*)cv.v)[i], p, k);
+      ((g_float*)cv.w)[i] = o.w;
+      ((g_float*)cv.m)[i] = o.m;
+      ((g_float*)cv.v)[i] = o.v;
+    }
+  }
+}
+
+// ------------------------------------------------------------------ per-tensor finishes
+// From the total of pass A: the gradient norm and divisor (multi_tensor_lans.cu:284-286: divide
+// only when normalising and the norm is non-zero).  Executed by one thread.
+__device__ __forceinline__ double stats_after_a(TensorStats* st, double sum_g,
+                                                const StepScalars& k) {
+  const double gn = sqrt(sum_g);
+  const double inv_gdiv = (k.normalize_grad && gn != 0.0) ? 1.0 / (gn + k.eps) : 1.0;
+  publish(&st->grad_norm, gn);
+  publish(&st->inv_grad_div, inv_gdiv);
+  return inv_gdiv;
+}
+
+// From the totals of pass B: ||w|| and the two trust ratios (multi_tensor_lans.cu:349-352) with
+// beta1 / beta3 folded in.  Executed by one thread.
+__device__ __forceinline__ void stats_after_b(TensorStats* st, const double (&tot)[3],
+                                              const StepScalars& k, double& ratio_m,
+                                              double& ratio_g) {
+  const double unm = sqrt(tot[0]), ung = sqrt(tot[1]), pn = sqrt(tot[2]);
+  const double rm = (unm != 0.0 && pn != 0.0) ? k.lr * (pn / unm) : k.lr;
+  const double rg = (ung != 0.0 && pn != 0.0) ? k.lr * (pn / ung) : k.lr;
+  ratio_m = rm * k.beta1;
+  ratio_g = rg * k.beta3;
+  publish(&st->param_norm, pn);
+  publish(&st->um_norm, unm);
+  publish(&st->ug_norm, ung);
+  publish(&st->ratio_m, ratio_m);
+  publish(&st->ratio_g, ratio_g);
+}
+
+__device__ __forceinline__ int64_t chunks_of(const TensorRec& tr) {
+  return (tr.numel + kChunk - 1) / kChunk;
+}
+
+// ------------------------------------------------------------------ set-up launch
+// Host scalars of the reference (lans.cc:94-109), evaluated on the device so that the step tensor
+// never has to be copied to the host; also marks every word the pipelined schedule waits on
+// (chunk partials, per-tensor statistics) as not ready and rewinds the ticket.
+__global__ __launch_bounds__(kLansBlock) void lans_prepare(LansDeviceArgs a, const float* step_dev,
+                                                           int32_t step_host, HParamsPod hp) {
+  const uint64_t tid = (uint64_t)blockIdx.x * kLansBlock + threadIdx.x;
+  const uint64_t nthr = (uint64_t)gridDim.x * kLansBlock;
+  uint64_t* stat_words = reinterpret_cast<uint64_t*>(a.stats);
+  for (uint64_t i = tid; i < 8u * (uint64_t)a.n_tensors; i += nthr) stat_words[i] = kNotReady;
+  uint64_t* part_words = reinterpret_cast<uint64_t*>(a.partials);
+  for (uint64_t i = tid; i < (uint64_t)kPartialSlots * (uint64_t)a.n_chunks; i += nthr)
+    part_words[i] = kNotReady;
+  if (tid == 0) {
+    a.sync->ticket = 0u;
+    a.sync->error = 0u;
     const int step = step_dev ? (int)(*step_dev) : step_host;
     float bc1 = 1.0f, bc2 = 1.0f;
     if (hp.bias_correction == 1) {  // double pow, then one rounding to fp32 (lans.cc:103-104)
       bc1 = (float)(1.0 - pow((double)hp.beta1, (double)step));
       bc2 = (float)(1.0 - pow((double)hp.beta2, (double)step));
     }
-    const float beta3 = (hp.grad_averaging == 1) ? __fsub_rn(1.0f, hp.beta1) : 1.0f;
     StepScalars k;
     k.beta1 = hp.beta1;
     k.beta2 = hp.beta2;
-    k.one_minus_beta2 = __fsub_rn(1.0f, hp.beta2);  // fp32 subtraction (multi_tensor_lans.cu:291)
-    k.beta3 = beta3;
+    k.one_minus_beta2 = 1.0f - hp.beta2;                             // fp32 subtraction (:291)
+    k.beta3 = (hp.grad_averaging == 1) ? (1.0f - hp.beta1) : 1.0f;  // fp32 (lans.cc:107-109)
     k.eps = hp.eps;
     k.wd = hp.weight_decay;
     k.inv_bc1 = 1.0 / (double)bc1;
     k.inv_bc2 = 1.0 / (double)bc2;
     k.lr = hp.learning_rate;
-    k.mode = hp.mode;
+    k.decay_into_grad = hp.mode == 0 ? 1.0 : 0.0;
+    k.decay_into_dir = hp.mode == 0 ? 0.0 : 1.0;
+    k.normalize_grad = hp.normalize_grad;
     k.pad = 0;
-    *scalars = k;
+    *a.scalars = k;
   }
 }
 
-__global__ __launch_bounds__(kLansBlock) void lans_finish_b(
-    const TensorRec* __restrict__ tensors, int32_t n_tensors, const double* __restrict__ partials,
-    TensorStats* __restrict__ stats, const StepScalars* __restrict__ scalars) {
-  const int t = (int)((blockIdx.x * (unsigned)kLansBlock + threadIdx.x) >> 6);
-  const int lane = threadIdx.x & 63;
-  if (t >= n_tensors) return;
-  double sm, sgg;
-  tensor_totals(tensors[t], partials, lane, sm, sgg);
-  if (lane == 0) {
-    const StepScalars k = *scalars;
-    const double unm = sqrt(sm), ung = sqrt(sgg);
-    const double pn = stats[t].param_norm;
-    // multi_tensor_lans.cu:349-352
-    double rm = (unm != 0.0 && pn != 0.0) ? k.lr * (pn / unm) : k.lr;
-    double rg = (ung != 0.0 && pn != 0.0) ? k.lr * (pn / ung) : k.lr;
-    stats[t].um_norm = unm;
-    stats[t].ug_norm = ung;
-    stats[t].ratio_m = rm * k.beta1;
-    stats[t].ratio_g = rg * k.beta3;
-  }
-}
-
-// ------------------------------------------------------------------ phase 3: sum u_m^2, sum u_g^2
+// ------------------------------------------------------------------ phased schedule
 template <typename G>
-__global__ __launch_bounds__(kLansBlock) void lans_norm_u(
-    const TensorRec* __restrict__ tensors, const ChunkRec* __restrict__ chunks, int64_t n_chunks,
-    float unscale, const StepScalars* __restrict__ scalars, const TensorStats* __restrict__ stats,
-    double* __restrict__ partials) {
-  __shared__ double red[2][kLansWaves];
-  const StepScalars k = *scalars;
-  for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
-    const ChunkView cv = chunk_view(tensors, chunks, c, (int)sizeof(G));
-    const G* g = static_cast<const G*>(cv.g);
-    const double inv_gdiv = stats[cv.tensor].inv_grad_div;
-    double am = 0.0, au = 0.0;
-    if (cv.vec_ok) {
-      const int n4 = cv.len >> 2;
-      for (int i0 = threadIdx.x; i0 < n4; i0 += kLansBlock * kUnroll) {
-        float4 gv[kUnroll], wv[kUnroll], mv[kUnroll], vv[kUnroll];
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-          const int i = i0 + u * kLansBlock;
-          if (i < n4) {
-            gv[u] = GradIO<G>::load4(g, i, unscale);
-            wv[u] = reinterpret_cast<const float4*>(cv.w)[i];
-            mv[u] = reinterpret_cast<const float4*>(cv.m)[i];
-            vv[u] = reinterpret_cast<const float4*>(cv.v)[i];
-          }
-        }
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-          const int i = i0 + u * kLansBlock;
-          if (i < n4) {
-            const Directions d0 = lans_directions(gv[u].x, wv[u].x, mv[u].x, vv[u].x, inv_gdiv, k);
-            const Directions d1 = lans_directions(gv[u].y, wv[u].y, mv[u].y, vv[u].y, inv_gdiv, k);
-            const Directions d2 = lans_directions(gv[u].z, wv[u].z, mv[u].z, vv[u].z, inv_gdiv, k);
-            const Directions d3 = lans_directions(gv[u].w, wv[u].w, mv[u].w, vv[u].w, inv_gdiv, k);
-            am += (d0.um * d0.um + d1.um * d1.um) + (d2.um * d2.um + d3.um * d3.um);
-            au += (d0.ug * d0.ug + d1.ug * d1.ug) + (d2.ug * d2.ug + d3.ug * d3.ug);
-          }
-        }
-      }
-      const int tail = (n4 << 2) + threadIdx.x;
-      if (tail < cv.len) {
-        const Directions d = lans_directions(GradIO<G>::load1(g, tail, unscale), cv.w[tail],
-                                             cv.m[tail], cv.v[tail], inv_gdiv, k);
-        am += d.um * d.um;
-        au += d.ug * d.ug;
-      }
-    } else {
-      for (int i = threadIdx.x; i < cv.len; i += kLansBlock) {
-        const Directions d = lans_directions(GradIO<G>::load1(g, i, unscale), cv.w[i], cv.m[i],
-                                             cv.v[i], inv_gdiv, k);
-        am += d.um * d.um;
-        au += d.ug * d.ug;
-      }
-    }
-    block_sum2(am, au, red);
+__global__ __launch_bounds__(kLansBlock) void lans_norm_g(LansDeviceArgs a) {
+  __shared__ double red[3][kLansWaves];
+  for (int64_t c = blockIdx.x; c < a.n_chunks; c += gridDim.x) {
+    const WorkItem it = a.items[c];
+    const TensorRec tr = a.tensors[it.tensor];
+    const ChunkView cv = chunk_view(tr, it.chunk_phase & kChunkMask, (int)sizeof(G));
+    double s[1] = {chunk_sum_g<G>(cv, a.unscale)};
+    block_sum<1>(s, red);
+    if (threadIdx.x == 0) publish(&a.partials[kPartialSlots * c], s[0]);
+  }
+}
+
+// One workgroup per tensor.
+__global__ __launch_bounds__(kLansBlock) void lans_finish(LansDeviceArgs a, int after_b) {
+  __shared__ double red[3][kLansWaves];
+  const int t = blockIdx.x;
+  const TensorRec tr = a.tensors[t];
+  const double* part = a.partials + kPartialSlots * (int64_t)tr.first_chunk;
+  const StepScalars k = *a.scalars;
+  if (after_b) {
+    double tot[3], r0, r1;
+    tensor_totals<3, false>(part, 1, chunks_of(tr), tot, red, nullptr);
+    if (threadIdx.x == 0) stats_after_b(&a.stats[t], tot, k, r0, r1);
+  } else {
+    double tot[1];
+    tensor_totals<1, false>(part, 0, chunks_of(tr), tot, red, nullptr);
+    if (threadIdx.x == 0) stats_after_a(&a.stats[t], tot[0], k);
+  }
+}
+
+template <typename G>
+__global__ __launch_bounds__(kLansBlock) void lans_norm_u(LansDeviceArgs a) {
+  __shared__ double red[3][kLansWaves];
+  const StepScalars k = *a.scalars;
+  for (int64_t c = blockIdx.x; c < a.n_chunks; c += gridDim.x) {
+    const WorkItem it = a.items[c];
+    const TensorRec tr = a.tensors[it.tensor];
+    const ChunkView cv = chunk_view(tr, it.chunk_phase & kChunkMask, (int)sizeof(G));
+    const double inv_gdiv = a.stats[it.tensor].inv_grad_div;
+    double s[3];
+    chunk_sums_u<G>(cv, a.unscale, k, [&] { return inv_gdiv; }, s);
+    block_sum<3>(s, red);
     if (threadIdx.x == 0) {
-      partials[2 * c] = am;
-      partials[2 * c + 1] = au;
+      publish(&a.partials[kPartialSlots * c + 1], s[0]);
+      publish(&a.partials[kPartialSlots * c + 2], s[1]);
+      publish(&a.partials[kPartialSlots * c + 3], s[2]);
     }
   }
 }
 
-// ------------------------------------------------------------------ phase 5: apply
-__device__ __forceinline__ void apply_one(double g, double w, double m, double v, double inv_gdiv,
-                                          const StepScalars& k, double rm, double rg, float& w_out,
-                                          float& m_out, float& v_out) {
-  const Directions d = lans_directions(g, w, m, v, inv_gdiv, k);
-  // multi_tensor_lans.cu:386: p - ratio_m*update_m - ratio_g*update_g, left to right
-  w_out = (float)((w - rm * d.um) - rg * d.ug);
-  m_out = (float)d.m1;
-  v_out = (float)d.v1;
+template <typename G>
+__global__ __launch_bounds__(kLansBlock) void lans_apply(LansDeviceArgs a) {
+  const StepScalars k = *a.scalars;
+  for (int64_t c = blockIdx.x; c < a.n_chunks; c += gridDim.x) {
+    const WorkItem it = a.items[c];
+    const TensorRec tr = a.tensors[it.tensor];
+    const ChunkView cv = chunk_view(tr, it.chunk_phase & kChunkMask, (int)sizeof(G));
+    const TensorStats st = a.stats[it.tensor];
+    const ApplyParams p{st.inv_grad_div, st.ratio_m, st.ratio_g};
+    chunk_apply<G>(cv, a.unscale, k, [&] { return p; });
+  }
 }
 
+// ------------------------------------------------------------------ pipelined schedule
 template <typename G>
-__global__ __launch_bounds__(kLansBlock) void lans_apply(
-    const TensorRec* __restrict__ tensors, const ChunkRec* __restrict__ chunks, int64_t n_chunks,
-    float unscale, const StepScalars* __restrict__ scalars,
-    const TensorStats* __restrict__ stats) {
-  const StepScalars k = *scalars;
-  for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
-    const ChunkView cv = chunk_view(tensors, chunks, c, (int)sizeof(G));
-    const G* g = static_cast<const G*>(cv.g);
-    const TensorStats st = stats[cv.tensor];
-    const double inv_gdiv = st.inv_grad_div, rm = st.ratio_m, rg = st.ratio_g;
-    if (cv.vec_ok) {
-      const int n4 = cv.len >> 2;
-      for (int i0 = threadIdx.x; i0 < n4; i0 += kLansBlock * kUnroll) {
-        float4 gv[kUnroll], wv[kUnroll], mv[kUnroll], vv[kUnroll];
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-          const int i = i0 + u * kLansBlock;
-          if (i < n4) {
-            gv[u] = GradIO<G>::load4(g, i, unscale);
-            wv[u] = reinterpret_cast<const float4*>(cv.w)[i];
-            mv[u] = reinterpret_cast<const float4*>(cv.m)[i];
-            vv[u] = reinterpret_cast<const float4*>(cv.v)[i];
-          }
-        }
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-          const int i = i0 + u * kLansBlock;
-          if (i < n4) {
-            float4 wo, mo, vo;
-            apply_one(gv[u].x, wv[u].x, mv[u].x, vv[u].x, inv_gdiv, k, rm, rg, wo.x, mo.x, vo.x);
-            apply_one(gv[u].y, wv[u].y, mv[u].y, vv[u].y, inv_gdiv, k, rm, rg, wo.y, mo.y, vo.y);
-            apply_one(gv[u].z, wv[u].z, mv[u].z, vv[u].z, inv_gdiv, k, rm, rg, wo.z, mo.z, vo.z);
-            apply_one(gv[u].w, wv[u].w, mv[u].w, vv[u].w, inv_gdiv, k, rm, rg, wo.w, mo.w, vo.w);
-            reinterpret_cast<float4*>(cv.w)[i] = wo;
-            reinterpret_cast<float4*>(cv.m)[i] = mo;
-            reinterpret_cast<float4*>(cv.v)[i] = vo;
-          }
-        }
-      }
-      const int tail = (n4 << 2) + threadIdx.x;
-      if (tail < cv.len) {
-        float wo, mo, vo;
-        apply_one(GradIO<G>::load1(g, tail, unscale), cv.w[tail], cv.m[tail], cv.v[tail], inv_gdiv,
-                  k, rm, rg, wo, mo, vo);
-        cv.w[tail] = wo;
-        cv.m[tail] = mo;
-        cv.v[tail] = vo;
-      }
-    } else {
-      for (int i = threadIdx.x; i < cv.len; i += kLansBlock) {
-        float wo, mo, vo;
-        apply_one(GradIO<G>::load1(g, i, unscale), cv.w[i], cv.m[i], cv.v[i], inv_gdiv, k, rm, rg,
-                  wo, mo, vo);
-        cv.w[i] = wo;
-        cv.m[i] = mo;
-        cv.v[i] = vo;
-      }
+__global__ __launch_bounds__(kLansBlock) void lans_pipelined(LansDeviceArgs a) {
+  __shared__ double red[3][kLansWaves];
+  __shared__ double s_bcast[3];
+  __shared__ uint32_t s_ticket;
+  const StepScalars k = *a.scalars;
+
+  // Thread 0 draws tickets two items ahead, so an atomic's round trip is hidden behind a whole
+  // item, and every thread reads the NEXT item's descriptor and tensor record while the current
+  // item is being processed.  Every workgroup draws exactly two tickets past the end of the list.
+  auto draw = [&]() -> uint32_t {
+    return __hip_atomic_fetch_add(&a.sync->ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  };
+  uint32_t ahead = 0;  // thread 0 only: the ticket after next
+  if (threadIdx.x == 0) {
+    s_ticket = draw();
+    ahead = draw();
+  }
+  __syncthreads();
+  // readfirstlane tells the compiler the value is wave-uniform: the descriptor and tensor-record
+  // reads below become scalar loads into SGPRs instead of per-lane loads into VGPRs.
+  uint32_t ticket = __builtin_amdgcn_readfirstlane(s_ticket);
+  WorkItem it = ticket < a.n_items ? a.pipeline_items[ticket] : WorkItem{0, 0};
+  TensorRec tr = ticket < a.n_items ? a.tensors[it.tensor] : TensorRec{};
+
+  while (ticket < a.n_items) {  // uniform
+    __syncthreads();            // everyone has read s_ticket and is done with the previous item
+    if (threadIdx.x == 0) {
+      s_ticket = ahead;
+      ahead = draw();
     }
+    __syncthreads();
+    const uint32_t next_ticket = __builtin_amdgcn_readfirstlane(s_ticket);
+    const WorkItem next_it =
+        next_ticket < a.n_items ? a.pipeline_items[next_ticket] : WorkItem{0, 0};
+    const TensorRec next_tr = next_ticket < a.n_items ? a.tensors[next_it.tensor] : TensorRec{};
+
+    uint64_t t_claim = 0;
+    if (a.trace && threadIdx.x == 0) t_claim = wall_clock64();
+    const int t = it.tensor;
+    const uint32_t phase = it.chunk_phase >> kPhaseShift;
+    const uint32_t chunk = it.chunk_phase & kChunkMask;
+    const ChunkView cv = chunk_view(tr, chunk, (int)sizeof(G));
+    const int64_t n_chunks = chunks_of(tr);
+    double* part = a.partials + kPartialSlots * ((int64_t)tr.first_chunk + chunk);
+    const double* tensor_part = a.partials + kPartialSlots * (int64_t)tr.first_chunk;
+    TensorStats* st = &a.stats[t];
+
+    if (phase == kPhaseA) {
+      double s[1] = {chunk_sum_g<G>(cv, a.unscale)};
+      block_sum<1>(s, red);
+      if (threadIdx.x == 0) publish(part, s[0]);
+    } else if (phase == kPhaseFinishA) {
+      double tot[1];
+      tensor_totals<1, true>(tensor_part, 0, n_chunks, tot, red, a.sync);
+      if (threadIdx.x == 0) stats_after_a(st, tot[0], k);
+    } else if (phase == kPhaseB) {
+      double s[3];
+      chunk_sums_u<G>(cv, a.unscale, k,
+                      [&] { return wait_published(&st->inv_grad_div, a.sync); }, s);
+      block_sum<3>(s, red);
+      if (threadIdx.x == 0) {
+        publish(part + 1, s[0]);
+        publish(part + 2, s[1]);
+        publish(part + 3, s[2]);
+      }
+    } else if (phase == kPhaseFinishB) {
+      double tot[3], r0, r1;
+      tensor_totals<3, true>(tensor_part, 1, n_chunks, tot, red, a.sync);
+      if (threadIdx.x == 0) stats_after_b(st, tot, k, r0, r1);
+    } else if (phase == kPhaseC) {
+      chunk_apply<G>(cv, a.unscale, k, [&] {
+        const double* const words[3] = {&st->inv_grad_div, &st->ratio_m, &st->ratio_g};
+        double val[3];
+        wait_published_n<3>(words, val, a.sync);
+        return ApplyParams{val[0], val[1], val[2]};
+      });
+    } else {
+      // A one-chunk tensor: all three passes here, no other workgroup involved.  The totals equal
+      // the single chunk partials, exactly as the general path computes them, and travel between
+      // the threads through LDS.
+      double s1[1] = {chunk_sum_g<G>(cv, a.unscale)};
+      block_sum<1>(s1, red);
+      if (threadIdx.x == 0) s_bcast[0] = stats_after_a(st, s1[0], k);
+      __syncthreads();
+      const double inv_gdiv = s_bcast[0];
+      double s3[3];
+      chunk_sums_u<G>(cv, a.unscale, k, [&] { return inv_gdiv; }, s3);
+      block_sum<3>(s3, red);
+      if (threadIdx.x == 0) stats_after_b(st, s3, k, s_bcast[1], s_bcast[2]);
+      __syncthreads();
+      const ApplyParams p{inv_gdiv, s_bcast[1], s_bcast[2]};
+      chunk_apply<G>(cv, a.unscale, k, [&] { return p; });
+    }
+    if (a.trace && threadIdx.x == 0) {  // diagnostics: when the item was started and finished
+      uint64_t* rec = a.trace + 4 * (uint64_t)ticket;
+      rec[0] = t_claim;
+      rec[1] = t_claim;
+      rec[2] = wall_clock64();
+      rec[3] = blockIdx.x;
+    }
+    ticket = next_ticket;
+    it = next_it;
+    tr = next_tr;
   }
 }
 
 }  // namespace
 
 // ------------------------------------------------------------------ launchers
-void launch_norm_gw(int grad_dtype, unsigned grid, hipStream_t s, const TensorRec* tensors,
-                    const ChunkRec* chunks, int64_t n_chunks, float unscale, double* partials) {
-  if (grad_dtype == RAFHIP_F16)
-    hipLaunchKernelGGL(lans_norm_gw<_Float16>, dim3(grid), dim3(kLansBlock), 0, s, tensors, chunks,
-                       n_chunks, unscale, partials);
+void launch_prepare(hipStream_t s, const LansDeviceArgs& a, const float* step_dev,
+                    int32_t step_host, HParamsPod hp) {
+  const uint64_t words = 8u * (uint64_t)a.n_tensors + (uint64_t)kPartialSlots * (uint64_t)a.n_chunks;
+  uint64_t grid = (words + kLansBlock * 4 - 1) / (kLansBlock * 4);
+  if (grid < 1) grid = 1;
+  if (grid > 256) grid = 256;
+  hipLaunchKernelGGL(lans_prepare, dim3((unsigned)grid), dim3(kLansBlock), 0, s, a, step_dev,
+                     step_host, hp);
+}
+
+void launch_phased(int grad_dtype, hipStream_t s, const LansDeviceArgs& a, hipEvent_t* marks) {
+  const unsigned grid = (unsigned)(a.n_chunks < (1 << 20) ? a.n_chunks : (1 << 20));
+  const bool f16 = grad_dtype == RAFHIP_F16;
+  auto mark = [&](int i) {
+    if (marks) (void)hipEventRecord(marks[i], s);
+  };
+  mark(0);
+  if (f16)
+    hipLaunchKernelGGL(lans_norm_g<_Float16>, dim3(grid), dim3(kLansBlock), 0, s, a);
   else
-    hipLaunchKernelGGL(lans_norm_gw<float>, dim3(grid), dim3(kLansBlock), 0, s, tensors, chunks,
-                       n_chunks, unscale, partials);
-}
-
-void launch_finish_a(unsigned grid, hipStream_t s, const TensorRec* tensors, int32_t n_tensors,
-                     const double* partials, TensorStats* stats, StepScalars* scalars,
-                     const float* step_dev, int32_t step_host, HParamsPod hp) {
-  hipLaunchKernelGGL(lans_finish_a, dim3(grid), dim3(kLansBlock), 0, s, tensors, n_tensors,
-                     partials, stats, scalars, step_dev, step_host, hp);
-}
-
-void launch_norm_u(int grad_dtype, unsigned grid, hipStream_t s, const TensorRec* tensors,
-                   const ChunkRec* chunks, int64_t n_chunks, float unscale,
-                   const StepScalars* scalars, const TensorStats* stats, double* partials) {
-  if (grad_dtype == RAFHIP_F16)
-    hipLaunchKernelGGL(lans_norm_u<_Float16>, dim3(grid), dim3(kLansBlock), 0, s, tensors, chunks,
-                       n_chunks, unscale, scalars, stats, partials);
+    hipLaunchKernelGGL(lans_norm_g<float>, dim3(grid), dim3(kLansBlock), 0, s, a);
+  mark(1);
+  hipLaunchKernelGGL(lans_finish, dim3((unsigned)a.n_tensors), dim3(kLansBlock), 0, s, a, 0);
+  mark(2);
+  if (f16)
+    hipLaunchKernelGGL(lans_norm_u<_Float16>, dim3(grid), dim3(kLansBlock), 0, s, a);
   else
-    hipLaunchKernelGGL(lans_norm_u<float>, dim3(grid), dim3(kLansBlock), 0, s, tensors, chunks,
-                       n_chunks, unscale, scalars, stats, partials);
-}
-
-void launch_finish_b(unsigned grid, hipStream_t s, const TensorRec* tensors, int32_t n_tensors,
-                     const double* partials, TensorStats* stats, const StepScalars* scalars) {
-  hipLaunchKernelGGL(lans_finish_b, dim3(grid), dim3(kLansBlock), 0, s, tensors, n_tensors,
-                     partials, stats, scalars);
-}
-
-void launch_apply(int grad_dtype, unsigned grid, hipStream_t s, const TensorRec* tensors,
-                  const ChunkRec* chunks, int64_t n_chunks, float unscale,
-                  const StepScalars* scalars, const TensorStats* stats) {
-  if (grad_dtype == RAFHIP_F16)
-    hipLaunchKernelGGL(lans_apply<_Float16>, dim3(grid), dim3(kLansBlock), 0, s, tensors, chunks,
-                       n_chunks, unscale, scalars, stats);
+    hipLaunchKernelGGL(lans_norm_u<float>, dim3(grid), dim3(kLansBlock), 0, s, a);
+  mark(3);
+  hipLaunchKernelGGL(lans_finish, dim3((unsigned)a.n_tensors), dim3(kLansBlock), 0, s, a, 1);
+  mark(4);
+  if (f16)
+    hipLaunchKernelGGL(lans_apply<_Float16>, dim3(grid), dim3(kLansBlock), 0, s, a);
   else
-    hipLaunchKernelGGL(lans_apply<float>, dim3(grid), dim3(kLansBlock), 0, s, tensors, chunks,
-                       n_chunks, unscale, scalars, stats);
+    hipLaunchKernelGGL(lans_apply<float>, dim3(grid), dim3(kLansBlock), 0, s, a);
+  mark(5);
+}
+
+void launch_pipelined(int grad_dtype, unsigned grid, hipStream_t s, const LansDeviceArgs& a) {
+  if (grad_dtype == RAFHIP_F16)
+    hipLaunchKernelGGL(lans_pipelined<_Float16>, dim3(grid), dim3(kLansBlock), 0, s, a);
+  else
+    hipLaunchKernelGGL(lans_pipelined<float>, dim3(grid), dim3(kLansBlock), 0, s, a);
+}
+
+int pipelined_blocks_per_cu(int grad_dtype) {
+  int n = 0;
+  hipError_t e = grad_dtype == RAFHIP_F16
+                     ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, lans_pipelined<_Float16>,
+                                                                    kLansBlock, 0)
+                     : hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, lans_pipelined<float>,
+                                                                    kLansBlock, 0);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return n;
 }
 
 }  // namespace rafhip

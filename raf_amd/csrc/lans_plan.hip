@@ -1,10 +1,12 @@
-// Host side of the multi-tensor LANS step: the plan (chunk table, tensor table, timing events) and
+// Host side of the multi-tensor LANS step: the plan (tensor table, work lists, timing events) and
 // the C-ABI entry points.  The plan plays the part of the reference's LansImpl constructor
 // (src/op/dialect/cuda/lans.cc:27-83) and rafhip_lans_step that of LansImpl::Execute (:92-131),
 // without its blocking copy of `step` to the host and without its per-element scratch buffer.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <array>
+#include <cstdlib>
 #include <cstring>
 #include <limits>
 #include <new>
@@ -21,25 +23,110 @@ constexpr int64_t kAlign = 256;
 inline int64_t align_up(int64_t x) { return (x + kAlign - 1) / kAlign * kAlign; }
 
 struct WorkspaceLayout {
-  int64_t scalars_off, stats_off, partials_off, total;
+  int64_t scalars_off, stats_off, partials_off, sync_off, total;
 };
+
+WorkspaceLayout make_layout(int32_t n_tensors, int64_t n_chunks) {
+  WorkspaceLayout l;
+  l.scalars_off = 0;
+  l.stats_off = align_up((int64_t)sizeof(StepScalars));
+  l.partials_off = l.stats_off + align_up((int64_t)sizeof(TensorStats) * n_tensors);
+  l.sync_off = l.partials_off + align_up((int64_t)sizeof(double) * kPartialSlots * n_chunks);
+  l.total = l.sync_off + align_up((int64_t)sizeof(SyncHeader));
+  return l;
+}
+
+inline int64_t chunks_of(int64_t numel) { return (numel + kChunk - 1) / kChunk; }
+
+// Default size of a cache group in elements: the pipelined schedule keeps about three groups'
+// worth of g, w, m, v (14-16 bytes per element) live in the 256 MB Infinity Cache.
+constexpr int64_t kDefaultGroupElems = 4608 * 1024;
+
+inline WorkItem make_item(int32_t tensor, uint32_t phase, int64_t chunk) {
+  return WorkItem{tensor, (phase << kPhaseShift) | (uint32_t)chunk};
+}
+
+// The pipelined work list.  Tensors are packed, in list order, into groups of at most group_elems
+// elements (a larger tensor is a group of its own).  "Round" r holds pass A of group r, then pass
+// B of group r-1, then pass C of group r-2.  (Merging the three so that they advance together was
+// measured too: items then sit right behind the ones they depend on and the kernel waits more.)
+// Invariant the kernel's waits rely on, per tensor: pass-A chunks, then its finish-A item, then
+// pass-B chunks, then its finish-B item, then pass-C chunks.
+std::vector<WorkItem> build_pipeline(int32_t n, const int64_t* numel, int64_t group_elems) {
+  struct Group {
+    std::vector<WorkItem> a, b, c;
+  };
+  std::vector<Group> groups;
+  int64_t in_group = 0;
+  for (int32_t t = 0; t < n; ++t) {
+    if (numel[t] == 0) continue;
+    if (groups.empty() || (in_group > 0 && in_group + numel[t] > group_elems)) {
+      groups.emplace_back();
+      in_group = 0;
+    }
+    in_group += numel[t];
+    Group& g = groups.back();
+    const int64_t nc = chunks_of(numel[t]);
+    if (nc == 1) {
+      g.a.push_back(make_item(t, kPhaseWhole, 0));  // one workgroup does all three passes
+      continue;
+    }
+    for (int64_t c = 0; c < nc; ++c) {
+      g.a.push_back(make_item(t, kPhaseA, c));
+      g.b.push_back(make_item(t, kPhaseB, c));
+      g.c.push_back(make_item(t, kPhaseC, c));
+    }
+    g.a.push_back(make_item(t, kPhaseFinishA, 0));  // after the tensor's chunks of the pass
+    g.b.push_back(make_item(t, kPhaseFinishB, 0));
+  }
+  std::vector<WorkItem> out;
+  const int64_t ng = (int64_t)groups.size();
+  for (int64_t r = 0; r < ng + 2; ++r) {
+    if (r < ng) out.insert(out.end(), groups[r].a.begin(), groups[r].a.end());
+    if (r >= 1 && r - 1 < ng) out.insert(out.end(), groups[r - 1].b.begin(), groups[r - 1].b.end());
+    if (r >= 2 && r - 2 < ng) out.insert(out.end(), groups[r - 2].c.begin(), groups[r - 2].c.end());
+  }
+  return out;
+}
+
+int64_t group_elems_setting() {
+  if (const char* e = std::getenv("RAFHIP_LANS_GROUP_ELEMS")) {
+    const long long v = std::atoll(e);
+    if (v > 0) return v;
+  }
+  return kDefaultGroupElems;
+}
+
+int schedule_setting() {
+  if (const char* e = std::getenv("RAFHIP_LANS_SCHEDULE")) {
+    if (!std::strcmp(e, "phased")) return RAFHIP_LANS_PHASED;
+    if (!std::strcmp(e, "pipelined")) return RAFHIP_LANS_PIPELINED;
+  }
+  return RAFHIP_LANS_PHASED;
+}
 
 }  // namespace
 
 struct rafhip_lans_plan {
   int device = 0;
+  int n_cus = 256;
   int32_t n_tensors = 0;
   int32_t grad_dtype = RAFHIP_F32;
+  int32_t schedule = RAFHIP_LANS_PHASED;
   int64_t n_chunks = 0;
   int64_t total_elements = 0;
+  uint32_t n_pipeline_items = 0;
+  unsigned pipeline_grid = 0;
   std::vector<int64_t> numel;
   std::vector<int32_t> first_chunk;
   WorkspaceLayout ws{};
 
-  // Device tables: [TensorRec x n_tensors][ChunkRec x n_chunks] in one allocation.
+  // Device tables in one allocation: [TensorRec x n][phased items x n_chunks][pipeline items].
   void* d_tables = nullptr;
   TensorRec* d_tensors = nullptr;
-  ChunkRec* d_chunks = nullptr;
+  WorkItem* d_items = nullptr;
+  WorkItem* d_pipeline = nullptr;
+  uint64_t* d_trace = nullptr;  // diagnostics, only with RAFHIP_LANS_TRACE=1
 
   // Tensor-table upload: pinned staging + the records last sent, so a step whose pointers did not
   // move sends nothing.
@@ -68,11 +155,26 @@ void free_plan(rafhip_lans_plan* p) {
   if (p->staging_free) (void)hipEventDestroy(p->staging_free);
   if (p->h_staging) (void)hipHostFree(p->h_staging);
   if (p->d_tables) (void)hipFree(p->d_tables);
+  if (p->d_trace) (void)hipFree(p->d_trace);
   delete p;
 }
 
 inline bool aligned_to(const void* p, uintptr_t a) {
   return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0;
+}
+
+int validate_list(const char* who, int32_t n_tensors, const int64_t* numel) {
+  if (n_tensors < 0) return fail(RAFHIP_ERR_INVALID_ARG, "%s: n_tensors = %d < 0", who, n_tensors);
+  if (n_tensors > 0 && !numel) return fail(RAFHIP_ERR_INVALID_ARG, "%s: numel is NULL", who);
+  int64_t chunks = 0;
+  for (int32_t t = 0; t < n_tensors; ++t) {
+    if (numel[t] < 0)
+      return fail(RAFHIP_ERR_INVALID_ARG, "%s: numel[%d] = %lld < 0", who, t, (long long)numel[t]);
+    chunks += chunks_of(numel[t]);
+    if (chunks >= (int64_t)kChunkMask / 4)
+      return fail(RAFHIP_ERR_UNSUPPORTED, "%s: too many chunks (more than 2^28)", who);
+  }
+  return RAFHIP_OK;
 }
 
 }  // namespace
@@ -94,23 +196,37 @@ void rafhip_lans_default_hparams(rafhip_lans_hparams* hp) {
   hp->grad_unscale = 1.0f;
 }
 
+int32_t rafhip_lans_chunk_elements(void) { return kChunk; }
+
 int rafhip_lans_query_layout(int32_t n_tensors, const int64_t* numel, int64_t* n_chunks_out,
                              int64_t* workspace_bytes_out) {
   clear_error();
-  if (n_tensors < 0 || (n_tensors > 0 && !numel))
-    return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_query_layout: bad tensor list");
+  if (int st = validate_list("rafhip_lans_query_layout", n_tensors, numel)) return st;
   int64_t chunks = 0;
-  for (int32_t t = 0; t < n_tensors; ++t) {
-    if (numel[t] < 0)
-      return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_query_layout: numel[%d] = %lld < 0", t,
-                  (long long)numel[t]);
-    chunks += (numel[t] + kChunk - 1) / kChunk;
-  }
+  for (int32_t t = 0; t < n_tensors; ++t) chunks += chunks_of(numel[t]);
   if (n_chunks_out) *n_chunks_out = chunks;
-  if (workspace_bytes_out)
-    *workspace_bytes_out = align_up((int64_t)sizeof(StepScalars)) +
-                           align_up((int64_t)sizeof(TensorStats) * n_tensors) +
-                           align_up((int64_t)sizeof(double) * 2 * chunks);
+  if (workspace_bytes_out) *workspace_bytes_out = make_layout(n_tensors, chunks).total;
+  return RAFHIP_OK;
+}
+
+int rafhip_lans_pipeline_order(int32_t n_tensors, const int64_t* numel, int64_t group_elements,
+                               int32_t* triples_out, int64_t capacity, int64_t* n_items_out) {
+  clear_error();
+  if (int st = validate_list("rafhip_lans_pipeline_order", n_tensors, numel)) return st;
+  if (!n_items_out) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_pipeline_order: n_items_out is NULL");
+  const std::vector<WorkItem> items =
+      build_pipeline(n_tensors, numel, group_elements > 0 ? group_elements : kDefaultGroupElems);
+  *n_items_out = (int64_t)items.size();
+  if (triples_out) {
+    if (capacity < (int64_t)items.size())
+      return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_pipeline_order: capacity %lld < %zu items",
+                  (long long)capacity, items.size());
+    for (size_t i = 0; i < items.size(); ++i) {
+      triples_out[3 * i + 0] = (int32_t)(items[i].chunk_phase >> kPhaseShift);
+      triples_out[3 * i + 1] = items[i].tensor;
+      triples_out[3 * i + 2] = (int32_t)(items[i].chunk_phase & kChunkMask);
+    }
+  }
   return RAFHIP_OK;
 }
 
@@ -119,10 +235,7 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
   clear_error();
   if (!out_plan) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_plan_create: out_plan is NULL");
   *out_plan = nullptr;
-  if (n_tensors < 0)
-    return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_plan_create: n_tensors = %d < 0", n_tensors);
-  if (n_tensors > 0 && !numel)
-    return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_plan_create: numel is NULL");
+  if (int st = validate_list("rafhip_lans_plan_create", n_tensors, numel)) return st;
   if (grad_dtype != RAFHIP_F32 && grad_dtype != RAFHIP_F16)
     return fail(RAFHIP_ERR_UNSUPPORTED,
                 "rafhip_lans_plan_create: gradient dtype %d (LANS takes fp32 weights and state; "
@@ -133,63 +246,77 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
   if (!p) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_plan_create: out of host memory");
   p->n_tensors = n_tensors;
   p->grad_dtype = grad_dtype;
+  p->schedule = schedule_setting();
   p->numel.assign(numel, numel + n_tensors);
   p->first_chunk.resize(n_tensors);
   int64_t chunks = 0, total = 0;
   for (int32_t t = 0; t < n_tensors; ++t) {
-    if (numel[t] < 0) {
-      free_plan(p);
-      return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_plan_create: numel[%d] = %lld < 0", t,
-                  (long long)numel[t]);
-    }
     p->first_chunk[t] = (int32_t)chunks;
-    chunks += (numel[t] + kChunk - 1) / kChunk;
+    chunks += chunks_of(numel[t]);
     total += numel[t];
-    if (chunks > std::numeric_limits<int32_t>::max()) {
-      free_plan(p);
-      return fail(RAFHIP_ERR_UNSUPPORTED, "rafhip_lans_plan_create: more than 2^31 chunks");
-    }
   }
   p->n_chunks = chunks;
   p->total_elements = total;
-  p->ws.scalars_off = 0;
-  p->ws.stats_off = align_up((int64_t)sizeof(StepScalars));
-  p->ws.partials_off = p->ws.stats_off + align_up((int64_t)sizeof(TensorStats) * n_tensors);
-  p->ws.total = p->ws.partials_off + align_up((int64_t)sizeof(double) * 2 * chunks);
+  p->ws = make_layout(n_tensors, chunks);
 
   if (hipGetDevice(&p->device) != hipSuccess) {
     (void)hipGetLastError();
     free_plan(p);
     return fail(RAFHIP_ERR_NO_DEVICE, "rafhip_lans_plan_create: no HIP device available");
   }
+  int cus = 0;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, p->device) == hipSuccess &&
+      cus > 0)
+    p->n_cus = cus;
 
   if (n_tensors > 0) {
+    std::vector<WorkItem> phased((size_t)chunks);
+    size_t k = 0;
+    for (int32_t t = 0; t < n_tensors; ++t)
+      for (int64_t c = 0; c < chunks_of(numel[t]); ++c) phased[k++] = make_item(t, kPhaseA, c);
+    const std::vector<WorkItem> pipeline = build_pipeline(n_tensors, numel, group_elems_setting());
+    p->n_pipeline_items = (uint32_t)pipeline.size();
+    // Resident workgroups per CU: never more than fit (every workgroup must be running), and by
+    // default three: a larger window of in-flight items measured slower on MI355X (it crowds the
+    // Infinity Cache).  RAFHIP_LANS_BLOCKS_PER_CU overrides the default downwards or up to the fit.
+    const int fit = pipelined_blocks_per_cu(grad_dtype);
+    int per_cu = fit > 0 ? (fit < 3 ? fit : 3) : 2;
+    if (const char* e = std::getenv("RAFHIP_LANS_BLOCKS_PER_CU")) {
+      const int want = std::atoi(e);
+      if (want > 0) per_cu = (fit > 0 && want > fit) ? fit : want;
+    }
+    p->pipeline_grid = (unsigned)(p->n_cus * per_cu);
+    if (p->pipeline_grid > p->n_pipeline_items) p->pipeline_grid = p->n_pipeline_items;
+
     const size_t tensors_bytes = (size_t)align_up((int64_t)sizeof(TensorRec) * n_tensors);
-    const size_t chunk_bytes = sizeof(ChunkRec) * (size_t)chunks;
-    hipError_t e = hipMalloc(&p->d_tables, tensors_bytes + (chunk_bytes ? chunk_bytes : 8));
-    if (e == hipSuccess) e = hipHostMalloc(reinterpret_cast<void**>(&p->h_staging),
-                                           sizeof(TensorRec) * (size_t)n_tensors, hipHostMallocDefault);
+    const size_t phased_bytes = (size_t)align_up((int64_t)sizeof(WorkItem) * (int64_t)phased.size());
+    const size_t pipe_bytes = (size_t)align_up((int64_t)sizeof(WorkItem) * (int64_t)pipeline.size());
+    hipError_t e = hipMalloc(&p->d_tables, tensors_bytes + phased_bytes + pipe_bytes + kAlign);
+    if (e == hipSuccess)
+      e = hipHostMalloc(reinterpret_cast<void**>(&p->h_staging),
+                        sizeof(TensorRec) * (size_t)n_tensors, hipHostMallocDefault);
     if (e == hipSuccess) e = hipEventCreateWithFlags(&p->staging_free, hipEventDisableTiming);
     if (e != hipSuccess) {
       free_plan(p);
       return fail(RAFHIP_ERR_HIP, "rafhip_lans_plan_create: allocation failed: %s",
                   hipGetErrorString(e));
     }
-    p->d_tensors = static_cast<TensorRec*>(p->d_tables);
-    p->d_chunks = reinterpret_cast<ChunkRec*>(static_cast<char*>(p->d_tables) + tensors_bytes);
-    if (chunks > 0) {
-      std::vector<ChunkRec> table((size_t)chunks);
-      size_t k = 0;
-      for (int32_t t = 0; t < n_tensors; ++t) {
-        const int64_t nc = (numel[t] + kChunk - 1) / kChunk;
-        for (int64_t i = 0; i < nc; ++i) table[k++] = ChunkRec{t, (int32_t)i};
-      }
-      e = hipMemcpy(p->d_chunks, table.data(), chunk_bytes, hipMemcpyHostToDevice);
-      if (e != hipSuccess) {
-        free_plan(p);
-        return fail(RAFHIP_ERR_HIP, "rafhip_lans_plan_create: chunk table upload failed: %s",
-                    hipGetErrorString(e));
-      }
+    char* base = static_cast<char*>(p->d_tables);
+    p->d_tensors = reinterpret_cast<TensorRec*>(base);
+    p->d_items = reinterpret_cast<WorkItem*>(base + tensors_bytes);
+    p->d_pipeline = reinterpret_cast<WorkItem*>(base + tensors_bytes + phased_bytes);
+    if (!phased.empty())
+      e = hipMemcpy(p->d_items, phased.data(), sizeof(WorkItem) * phased.size(),
+                    hipMemcpyHostToDevice);
+    if (e == hipSuccess && !pipeline.empty())
+      e = hipMemcpy(p->d_pipeline, pipeline.data(), sizeof(WorkItem) * pipeline.size(),
+                    hipMemcpyHostToDevice);
+    if (e == hipSuccess && std::getenv("RAFHIP_LANS_TRACE") && !pipeline.empty())
+      e = hipMalloc(reinterpret_cast<void**>(&p->d_trace), 32 * pipeline.size());
+    if (e != hipSuccess) {
+      free_plan(p);
+      return fail(RAFHIP_ERR_HIP, "rafhip_lans_plan_create: work list upload failed: %s",
+                  hipGetErrorString(e));
     }
   }
   *out_plan = p;
@@ -199,6 +326,15 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
 int rafhip_lans_plan_destroy(rafhip_lans_plan* plan) {
   clear_error();
   free_plan(plan);
+  return RAFHIP_OK;
+}
+
+int rafhip_lans_plan_set_schedule(rafhip_lans_plan* plan, int32_t schedule) {
+  clear_error();
+  if (!plan) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_plan_set_schedule: plan is NULL");
+  if (schedule != RAFHIP_LANS_PHASED && schedule != RAFHIP_LANS_PIPELINED)
+    return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_plan_set_schedule: schedule = %d", schedule);
+  plan->schedule = schedule;
   return RAFHIP_OK;
 }
 
@@ -237,9 +373,9 @@ int rafhip_lans_step(rafhip_lans_plan* plan, const void* const* g, float* const*
                 workspace);
 
   // Build this call's tensor table; 4-byte (fp16 g: 2-byte) alignment is the hard requirement,
-  // wider alignment only selects the vector path.
+  // 16-byte alignment of all four selects the vector path.
   const uintptr_t g_elem = plan->grad_dtype == RAFHIP_F16 ? 2 : 4;
-  const uintptr_t g_vec = plan->grad_dtype == RAFHIP_F16 ? 8 : 16;
+  const uintptr_t g_vec = 16;  // pass A reads the gradient with 16-byte lane accesses
   std::vector<TensorRec> recs((size_t)n);
   for (int32_t t = 0; t < n; ++t) {
     TensorRec& r = recs[t];
@@ -275,9 +411,19 @@ int rafhip_lans_step(rafhip_lans_plan* plan, const void* const* g, float* const*
   }
 
   char* ws = static_cast<char*>(workspace);
-  StepScalars* scalars = reinterpret_cast<StepScalars*>(ws + plan->ws.scalars_off);
-  TensorStats* stats = reinterpret_cast<TensorStats*>(ws + plan->ws.stats_off);
-  double* partials = reinterpret_cast<double*>(ws + plan->ws.partials_off);
+  LansDeviceArgs a;
+  a.tensors = plan->d_tensors;
+  a.n_tensors = n;
+  a.items = plan->d_items;
+  a.n_chunks = plan->n_chunks;
+  a.n_items = plan->n_pipeline_items;
+  a.pipeline_items = plan->d_pipeline;
+  a.unscale = hp->grad_unscale;
+  a.scalars = reinterpret_cast<StepScalars*>(ws + plan->ws.scalars_off);
+  a.stats = reinterpret_cast<TensorStats*>(ws + plan->ws.stats_off);
+  a.partials = reinterpret_cast<double*>(ws + plan->ws.partials_off);
+  a.sync = reinterpret_cast<SyncHeader*>(ws + plan->ws.sync_off);
+  a.trace = plan->d_trace;
 
   HParamsPod pod;
   pod.learning_rate = hp->learning_rate;
@@ -290,30 +436,21 @@ int rafhip_lans_step(rafhip_lans_plan* plan, const void* const* g, float* const*
   pod.mode = hp->mode;
   pod.normalize_grad = hp->normalize_grad ? 1 : 0;
 
-  const unsigned chunk_grid = (unsigned)(plan->n_chunks < (1 << 20) ? plan->n_chunks : (1 << 20));
-  const unsigned finish_grid = (unsigned)((n + kLansWaves - 1) / kLansWaves);
+  hipEvent_t* marks = nullptr;
+  if (!plan->timing.empty())
+    marks = plan->timing[plan->steps_done % (int64_t)plan->timing.size()].data();
 
-  std::array<hipEvent_t, 6>* ev = nullptr;
-  if (!plan->timing.empty()) ev = &plan->timing[plan->steps_done % (int64_t)plan->timing.size()];
-#define RAFHIP_MARK(i) \
-  if (ev) RAFHIP_HIP_TRY(hipEventRecord((*ev)[i], s))
-
-  RAFHIP_MARK(0);
-  launch_norm_gw(plan->grad_dtype, chunk_grid, s, plan->d_tensors, plan->d_chunks, plan->n_chunks,
-                 hp->grad_unscale, partials);
-  RAFHIP_MARK(1);
-  launch_finish_a(finish_grid, s, plan->d_tensors, n, partials, stats, scalars, step_dev, step_host,
-                  pod);
-  RAFHIP_MARK(2);
-  launch_norm_u(plan->grad_dtype, chunk_grid, s, plan->d_tensors, plan->d_chunks, plan->n_chunks,
-                hp->grad_unscale, scalars, stats, partials);
-  RAFHIP_MARK(3);
-  launch_finish_b(finish_grid, s, plan->d_tensors, n, partials, stats, scalars);
-  RAFHIP_MARK(4);
-  launch_apply(plan->grad_dtype, chunk_grid, s, plan->d_tensors, plan->d_chunks, plan->n_chunks,
-               hp->grad_unscale, scalars, stats);
-  RAFHIP_MARK(5);
-#undef RAFHIP_MARK
+  if (plan->schedule == RAFHIP_LANS_PIPELINED) {
+    if (marks) RAFHIP_HIP_TRY(hipEventRecord(marks[0], s));
+    launch_prepare(s, a, step_dev, step_host, pod);
+    if (marks) RAFHIP_HIP_TRY(hipEventRecord(marks[1], s));
+    launch_pipelined(plan->grad_dtype, plan->pipeline_grid, s, a);
+    if (marks)
+      for (int i = 2; i < 6; ++i) RAFHIP_HIP_TRY(hipEventRecord(marks[i], s));
+  } else {
+    launch_prepare(s, a, step_dev, step_host, pod);
+    launch_phased(plan->grad_dtype, s, a, marks);
+  }
   RAFHIP_HIP_TRY(hipGetLastError());
   plan->steps_done++;
   return RAFHIP_OK;
@@ -327,17 +464,41 @@ int rafhip_lans_read_norms(const rafhip_lans_plan* plan, const void* workspace, 
   const int32_t n = plan->n_tensors;
   if (n == 0) return RAFHIP_OK;
   std::vector<TensorStats> st((size_t)n);
+  SyncHeader sync{};
   hipStream_t s = static_cast<hipStream_t>(stream);
-  RAFHIP_HIP_TRY(hipMemcpyAsync(st.data(),
-                                static_cast<const char*>(workspace) + plan->ws.stats_off,
-                                sizeof(TensorStats) * (size_t)n, hipMemcpyDeviceToHost, s));
+  const char* ws = static_cast<const char*>(workspace);
+  RAFHIP_HIP_TRY(hipMemcpyAsync(st.data(), ws + plan->ws.stats_off, sizeof(TensorStats) * (size_t)n,
+                                hipMemcpyDeviceToHost, s));
+  RAFHIP_HIP_TRY(hipMemcpyAsync(&sync, ws + plan->ws.sync_off, sizeof(sync), hipMemcpyDeviceToHost, s));
   RAFHIP_HIP_TRY(hipStreamSynchronize(s));
   for (int32_t t = 0; t < n; ++t) {
+    if (plan->numel[t] == 0) {  // no chunks, nothing was computed: an empty tensor has zero norms
+      for (int q = 0; q < 4; ++q) host_out[4 * t + q] = 0.0;
+      continue;
+    }
     host_out[4 * t + 0] = st[t].grad_norm;
     host_out[4 * t + 1] = st[t].param_norm;
     host_out[4 * t + 2] = st[t].um_norm;
     host_out[4 * t + 3] = st[t].ug_norm;
   }
+  if (plan->n_chunks > 0 && sync.error != 0)
+    return fail(RAFHIP_ERR_HIP,
+                "rafhip_lans_read_norms: the last pipelined step ran out of a bounded wait; its "
+                "results are invalid");
+  return RAFHIP_OK;
+}
+
+int rafhip_lans_debug_trace(rafhip_lans_plan* plan, uint64_t* words_out, int64_t capacity_items,
+                            int64_t* n_items_out) {
+  clear_error();
+  if (!plan || !n_items_out) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_debug_trace: null argument");
+  *n_items_out = plan->d_trace ? (int64_t)plan->n_pipeline_items : 0;
+  if (!plan->d_trace || !words_out) return RAFHIP_OK;
+  if (capacity_items < (int64_t)plan->n_pipeline_items)
+    return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_debug_trace: capacity too small");
+  RAFHIP_HIP_TRY(hipDeviceSynchronize());
+  RAFHIP_HIP_TRY(hipMemcpy(words_out, plan->d_trace, 32 * (size_t)plan->n_pipeline_items,
+                           hipMemcpyDeviceToHost));
   return RAFHIP_OK;
 }
 

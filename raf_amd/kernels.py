@@ -61,6 +61,18 @@ def query_layout(numels: Sequence[int]):
     return chunks.value, ws.value
 
 
+def pipeline_order(numels: Sequence[int], group_elements: int = 0):
+    """[(pass, tensor, chunk)] in the order the pipelined schedule hands out work; host arithmetic."""
+    n = len(numels)
+    arr = (c_int64 * max(n, 1))(*numels)
+    count = c_int64(0)
+    lib = _lib.optim()
+    check(lib.rafhip_lans_pipeline_order(n, arr, group_elements, None, 0, ctypes.byref(count)))
+    buf = (ctypes.c_int32 * max(3 * count.value, 1))()
+    check(lib.rafhip_lans_pipeline_order(n, arr, group_elements, buf, count.value, ctypes.byref(count)))
+    return [(buf[3 * i], buf[3 * i + 1], buf[3 * i + 2]) for i in range(count.value)]
+
+
 class LansPlan:
     """Owns a ``rafhip_lans_plan`` and a workspace tensor sized for it."""
 
@@ -85,6 +97,11 @@ class LansPlan:
         self.total_elements = self.lib.rafhip_lans_plan_total_elements(self._h)
         self.workspace = torch.empty(max(self.workspace_bytes, 256), dtype=torch.uint8,
                                      device=self.device)
+
+    def set_schedule(self, schedule: str):
+        """"phased" (one launch per pass) or "pipelined" (one persistent, cache-aware launch)."""
+        code = {"phased": _lib.RAFHIP_LANS_PHASED, "pipelined": _lib.RAFHIP_LANS_PIPELINED}[schedule]
+        check(self.lib.rafhip_lans_plan_set_schedule(self._h, code))
 
     def close(self):
         if self._h:
@@ -129,6 +146,21 @@ class LansPlan:
                                         ctypes.byref(hp), ws.data_ptr(), ws.numel(),
                                         _current_stream(self.device)))
 
+    def bind(self, g, w, m, v, hp: LansHParams, workspace: Optional[torch.Tensor] = None):
+        """Marshal the pointer lists once for tensors that stay where they are; ``step_bound`` then
+        costs one foreign call per step (a training loop updates the same buffers every step)."""
+        ws = self.workspace if workspace is None else workspace
+        self._bound = (self._ptrs(g, self.grad_dtype, "g"), self._ptrs(w, torch.float32, "w"),
+                       self._ptrs(m, torch.float32, "m"), self._ptrs(v, torch.float32, "v"),
+                       hp, ws, (list(g), list(w), list(m), list(v)))
+
+    def step_bound(self, step: torch.Tensor):
+        """One step on the tensors given to ``bind``; ``step`` is the 0-d fp32 GPU step tensor."""
+        gp, wp, mp, vp, hp, ws, _ = self._bound
+        check(self.lib.rafhip_lans_step(self._h, gp, wp, mp, vp, step.data_ptr(), 0,
+                                        ctypes.byref(hp), ws.data_ptr(), ws.numel(),
+                                        _current_stream(self.device)))
+
     def read_norms(self, workspace: Optional[torch.Tensor] = None):
         """[n, 4] float64: ||g||, ||w||, ||u_m||, ||u_g|| of the last step."""
         import numpy as np
@@ -138,6 +170,20 @@ class LansPlan:
         check(self.lib.rafhip_lans_read_norms(self._h, ws.data_ptr(), out,
                                               _current_stream(self.device)))
         return np.array(out[:4 * self.n], dtype=np.float64).reshape(self.n, 4)
+
+    def debug_trace(self):
+        """[n_items, 4] uint64 (drawn, unblocked, finished, workgroup) of the last pipelined step, or
+        None unless the process runs with RAFHIP_LANS_TRACE=1."""
+        import numpy as np
+
+        n = c_int64(0)
+        check(self.lib.rafhip_lans_debug_trace(self._h, None, 0, ctypes.byref(n)))
+        if n.value == 0:
+            return None
+        buf = np.zeros((n.value, 4), dtype=np.uint64)
+        check(self.lib.rafhip_lans_debug_trace(
+            self._h, buf.ctypes.data_as(ctypes.POINTER(ctypes.c_uint64)), n.value, ctypes.byref(n)))
+        return buf
 
     def timing_enable(self, slots: int):
         check(self.lib.rafhip_lans_timing_enable(self._h, int(slots)))

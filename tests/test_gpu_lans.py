@@ -237,3 +237,40 @@ def test_workspace_and_argument_errors(native_libs):
         plan.step([t[0].half()], t, t, t, 1, hp)
     with pytest.raises(TypeError):
         kernels.LansPlan([8], torch.bfloat16, DEV)
+
+
+# ------------------------------------------------------------------ the two schedules
+@pytest.mark.parametrize("g16", [False, True])
+def test_pipelined_schedule_is_bitwise_equal_to_phased(native_libs, g16):
+    """The persistent, cache-aware schedule runs the same per-chunk code and adds the same partials
+    in the same order as the five-launch schedule: every output bit must agree, and both must
+    match the oracle."""
+    from raf_amd import kernels, shapes
+
+    cases = {
+        "edge": [1, 3, 4, 5, 0, 255, 1023, 8191, 8192, 8193, 16385, 65537, 100003],
+        "many small": shapes.log_uniform_numels(400, seed=3),
+        "several groups": [1 << 20, 3, 5000, (1 << 22) + 7, 1 << 19, 12345, 1 << 21, 3 << 20],
+    }
+    hp = LansHParams(grad_unscale=(1 / 1024 if g16 else 1.0))
+    for name, sizes in cases.items():
+        g, w, m, v = lans_inputs(sizes, cfg=80, g16=g16)
+        results = {}
+        for schedule in ("phased", "pipelined"):
+            tg, tw, tm, tv = _to_dev(g), _to_dev(w), _to_dev(m), _to_dev(v)
+            plan = kernels.LansPlan(sizes, tg[0].dtype, DEV)
+            plan.set_schedule(schedule)
+            for step in (2, 3):
+                plan.step(tg, tw, tm, tv, torch.tensor(float(step), device=DEV), _khp(hp))
+            torch.cuda.synchronize()
+            norms = plan.read_norms()  # also raises if a bounded wait of the pipelined kernel ran out
+            results[schedule] = ([t.cpu().numpy() for t in tw + tm + tv], norms)
+            plan.close()
+        for a, b in zip(results["phased"][0], results["pipelined"][0]):
+            assert np.array_equal(a, b), name
+        assert np.array_equal(results["phased"][1], results["pipelined"][1]), name
+        ow, om, ov = w, m, v
+        for step in (2, 3):
+            ow, om, ov, on = lans_f64.lans_step(g, ow, om, ov, step, hp)
+        _assert_close(results["pipelined"][0], ow + om + ov, TOL_1, name)
+        _assert_norms(results["pipelined"][1], on)

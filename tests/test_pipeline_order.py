@@ -1,0 +1,75 @@
+"""Host logic of the pipelined LANS schedule (no GPU): the work list must contain every unit of work
+exactly once and respect the per-tensor order that makes the kernel's waits finite."""
+import pytest
+
+KIND_A, KIND_B, KIND_C, KIND_WHOLE, KIND_FIN_A, KIND_FIN_B = range(6)
+
+
+def _check(order, sizes, chunk):
+    n_chunks = [-(-n // chunk) for n in sizes]
+    seen = {}
+    for pos, (kind, t, c) in enumerate(order):
+        assert 0 <= t < len(sizes) and sizes[t] > 0, "empty tensors contribute no work"
+        assert (kind, t, c) not in seen, "duplicate work item"
+        seen[(kind, t, c)] = pos
+    for t, nc in enumerate(n_chunks):
+        if nc == 0:
+            continue
+        if nc == 1:
+            assert (KIND_WHOLE, t, 0) in seen
+            assert not any((k, t, 0) in seen for k in (KIND_A, KIND_B, KIND_C, KIND_FIN_A, KIND_FIN_B))
+            continue
+        a = [seen[(KIND_A, t, c)] for c in range(nc)]
+        b = [seen[(KIND_B, t, c)] for c in range(nc)]
+        cc = [seen[(KIND_C, t, c)] for c in range(nc)]
+        fa, fb = seen[(KIND_FIN_A, t, 0)], seen[(KIND_FIN_B, t, 0)]
+        assert max(a) < fa < min(b), f"tensor {t}: finish A must follow its chunks and precede pass B"
+        assert max(b) < fb < min(cc), f"tensor {t}: finish B must follow its chunks and precede pass C"
+    expect = sum(1 if nc == 1 else 3 * nc + 2 for nc in n_chunks if nc)
+    assert len(order) == expect
+
+
+@pytest.mark.parametrize("group", [0, 1, 100_000, 10**12])
+def test_order_invariants(native_libs, group):
+    from raf_amd import kernels, shapes
+
+    chunk = native_libs.optim().rafhip_lans_chunk_elements()
+    lists = [
+        [1, 3, 0, chunk - 1, chunk, chunk + 1, 5 * chunk + 7, 0, 2 * chunk, 17],
+        shapes.log_uniform_numels(300, seed=7),
+        shapes.numels(shapes.bert_base_shapes()),
+        [],
+        [0, 0],
+    ]
+    for sizes in lists:
+        _check(kernels.pipeline_order(sizes, group), sizes, chunk)
+
+
+def test_groups_bound_the_reuse_distance(native_libs):
+    """Between a tensor's pass-A chunks and its pass-C chunks lie at most a few groups' worth of
+    other tensors' work, which is what keeps the tensor in the Infinity Cache."""
+    from raf_amd import kernels
+
+    chunk = native_libs.optim().rafhip_lans_chunk_elements()
+    sizes = [8 * chunk] * 40  # 40 equal tensors, group = 2 tensors
+    order = kernels.pipeline_order(sizes, 16 * chunk)
+    first_a = {t: min(i for i, (k, tt, _) in enumerate(order) if k == KIND_A and tt == t) for t in range(40)}
+    last_c = {t: max(i for i, (k, tt, _) in enumerate(order) if k == KIND_C and tt == t) for t in range(40)}
+    per_group = 2 * (3 * 8 + 2)
+    for t in range(40):
+        assert last_c[t] - first_a[t] <= 3 * per_group
+    # one giant group degenerates into pass-major order: all of A, then all of B, then all of C
+    order = kernels.pipeline_order(sizes, 10**12)
+    kinds = [k for k, _, _ in order]
+    assert max(i for i, k in enumerate(kinds) if k in (KIND_A, KIND_FIN_A)) < min(
+        i for i, k in enumerate(kinds) if k == KIND_B)
+
+
+def test_bert_large_group_structure(native_libs):
+    from raf_amd import kernels, shapes
+
+    sizes = shapes.numels(shapes.bert_large_shapes())
+    order = kernels.pipeline_order(sizes)
+    chunk = native_libs.optim().rafhip_lans_chunk_elements()
+    _check(order, sizes, chunk)
+    assert sum(1 for k, _, _ in order if k == KIND_WHOLE) == sum(1 for n in sizes if 0 < n <= chunk)
