@@ -39,9 +39,12 @@ def lans_kernel_bytes_per_elt(g_bytes: int):
 
 SGD_BYTES_PER_ELT = 20  # read x, dx, v; write v1, x1
 
-# HBM traffic per launch of the dominant kernel (bytes), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs scaled by a plain copy kernel of known size; see profiles/.  None = not measured.
-MEASURED_TRAFFIC = {}
+# Memory traffic per launch of the dominant kernel (bytes), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# runs scaled by a plain 1 GiB copy (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); figures and commands are in
+# profiles/lans_phased_bert_large_fp16grad.md.  Workloads not listed were not measured (null).
+MEASURED_TRAFFIC = {
+    ("lans_bert_large_fp16grad", "lans_apply"): 8_717_300_000,
+}
 
 
 def workloads():
@@ -59,6 +62,9 @@ def workloads():
         "lans_gpt2_1p5b_fp32": dict(kind="lans", sizes=shapes.numels(shapes.gpt2_shapes()), g16=False,
                                     zero_state=True, step0=1),
         "sgd_4m_fp32": dict(kind="sgd", n=4_194_304),
+        # a plain device-to-device copy of known size: the yardstick that rocprofv3's FETCH_SIZE /
+        # WRITE_SIZE counters are scaled by when HBM traffic is measured
+        "copy_1gib": dict(kind="copy", nbytes=1 << 30),
     }
 
 
@@ -264,6 +270,36 @@ def bench_sgd(name, wl, args):
     return out
 
 
+def bench_copy(name, wl, args):
+    import torch
+
+    dev = torch.device("cuda:0")
+    n = wl["nbytes"] // 4
+    src = torch.randn(n, device=dev)
+    dst = torch.empty_like(src)
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(args.warmup):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(args.steps):
+        dst.copy_(src)
+    stop.record()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    dev_ms = start.elapsed_time(stop) / args.steps
+    moved = 2 * wl["nbytes"]
+    return {"metric": "device-to-device copy bandwidth (read + write bytes / time)",
+            "value": round(moved / (ms_per_step * 1e-3) / 1e9, 1), "unit": "GB/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": name, "bytes_read_per_step": wl["nbytes"], "bytes_written_per_step": wl["nbytes"]},
+            "roofline": {"bound": "hbm", "kernel": "torch copy", "achieved": round(moved / (dev_ms * 1e-3) / 1e9, 1),
+                         "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(moved / (dev_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                         "traffic": None, "bytes_per_launch": moved, "avg_launch_ms": round(dev_ms, 4)}}
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -291,7 +327,8 @@ def main():
 
     _lib.optim()  # fails loudly if the HIP library is not built
     wl = table[args.workload]
-    out = bench_lans(args.workload, wl, args) if wl["kind"] == "lans" else bench_sgd(args.workload, wl, args)
+    fn = {"lans": bench_lans, "sgd": bench_sgd, "copy": bench_copy}[wl["kind"]]
+    out = fn(args.workload, wl, args)
     print(json.dumps(out), flush=True)
 
 
