@@ -101,8 +101,10 @@ typedef struct rafhip_lans_plan rafhip_lans_plan;
 int rafhip_lans_query_layout(int32_t n_tensors, const int64_t* numel, int64_t* n_chunks_out,
                              int64_t* workspace_bytes_out);
 
-/* Elements per chunk, the unit of work and of the per-chunk partial sums. */
+/* Elements per chunk, the unit of work and of the partial sums of the second and third pass, and
+ * elements per unit of the first pass (a multiple of the chunk: that pass reads the gradient only). */
 int32_t rafhip_lans_chunk_elements(void);
+int32_t rafhip_lans_pass_a_unit_elements(void);
 
 /*
  * Schedules of a step; both run the same per-chunk code and give bit-identical results.
@@ -119,11 +121,11 @@ typedef enum rafhip_lans_schedule {
 
 /*
  * Pure host arithmetic: the work list of the pipelined schedule as int32 triples
- * (kind, tensor, chunk), kind being 0 = pass A chunk, 1 = pass B chunk, 2 = pass C chunk,
+ * (kind, tensor, index), kind being 0 = pass A unit, 1 = pass B chunk, 2 = pass C chunk,
  * 3 = a one-chunk tensor taken through all three passes by one workgroup, 4 = finish pass A
  * (add the tensor's partials, publish ||g||), 5 = finish pass B (publish ||w|| and the trust
  * ratios).  group_elements <= 0 selects the default group size.  triples_out may be NULL to query
- * the count.  The kernel's bounded waits rely on this order, per tensor: every pass-A chunk, then
+ * the count.  The kernel's bounded waits rely on this order, per tensor: every pass-A unit, then
  * finish A, then every pass-B chunk, then finish B, then every pass-C chunk.
  */
 int rafhip_lans_pipeline_order(int32_t n_tensors, const int64_t* numel, int64_t group_elements,

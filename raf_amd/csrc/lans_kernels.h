@@ -48,6 +48,8 @@ namespace rafhip {
 constexpr int kLansBlock = 256;  // 4 wavefronts
 constexpr int kLansWaves = kLansBlock / 64;
 constexpr int kChunk = 8192;     // elements per chunk (multiple of 4 * kLansBlock)
+constexpr int kChunksPerA = 8;   // pass A reads 2-4 bytes per element, so its unit of work (and of
+                                 // partial sums) is 8 chunks; its partial lives in the first one's slot
 constexpr int kUnroll = 2;       // 4-element groups in flight per lane per trip
 constexpr int kPartialSlots = 4; // doubles per chunk: [0] sum g^2 | [1] sum u_m^2 [2] sum u_g^2 [3] sum w^2
 
@@ -113,8 +115,10 @@ struct HParamsPod {
 struct LansDeviceArgs {
   const TensorRec* tensors;
   int32_t n_tensors;
-  const WorkItem* items;  // phased: [A items][B items][C items], each n_chunks long
+  const WorkItem* items;  // phased, passes B and C: every chunk of every tensor, n_chunks long
   int64_t n_chunks;
+  const WorkItem* items_a;  // phased, pass A: every pass-A unit (kChunksPerA chunks), n_items_a long
+  int64_t n_items_a;
   uint32_t n_items;       // pipelined work-list length
   const WorkItem* pipeline_items;
   float unscale;

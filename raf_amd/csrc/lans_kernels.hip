@@ -23,6 +23,35 @@ typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef RAFHIP_GLOBAL const half8_t gc_half8;
 typedef RAFHIP_GLOBAL const _Float16 gc_half;
 
+// ------------------------------------------------------------------ cache policy
+// Every pass streams far more data than the 256 MB Infinity Cache holds.  Loads and stores that
+// carry the non-temporal hint do not allocate lines there, and on MI355X that alone is worth
+// 10-15 % of HBM bandwidth (measured: the read-only pass goes from 6.2 to 6.9 TB/s).  The one
+// stream worth caching is the gradient in passes B and C: it is the smallest array, pass B walks
+// the list back to front and pass C front to back, so pass C finds the gradients of the front
+// third of the list still cached.  Measured best of nine combinations on the BERT-large list.
+// The pipelined schedule keeps passes A and B temporal because it WANTS their lines to stay.
+struct CachePolicy {  // true = non-temporal
+  bool a_g, b_g, b_wmv, c_g, c_wmv, c_stores;
+};
+constexpr CachePolicy kPhasedPolicy = {true, false, true, false, true, true};
+constexpr CachePolicy kPipelinedPolicy = {false, false, false, true, true, true};
+
+template <bool kNT, typename T>
+__device__ __forceinline__ T ldg(const RAFHIP_GLOBAL T* p) {
+  if constexpr (kNT)
+    return __builtin_nontemporal_load(p);
+  else
+    return *p;
+}
+template <bool kNT, typename T>
+__device__ __forceinline__ void stg(RAFHIP_GLOBAL T* p, T v) {
+  if constexpr (kNT)
+    __builtin_nontemporal_store(v, p);
+  else
+    *p = v;
+}
+
 // ------------------------------------------------------------------ gradient ingest
 // Gradients as fp32, already multiplied by the unscale factor (one fp32 rounding, exact for
 // power-of-two loss scales).
@@ -33,16 +62,18 @@ template <>
 struct GradIO<float> {
   // Widest single-lane access used when the gradient is the only array read (pass A): 16 bytes.
   static constexpr int kWide = 4;
+  template <bool kNT>
   static __device__ __forceinline__ void load_wide(const void* g, int iw, float us,
                                                    float (&out)[kWide]) {
-    const f32x4 r = ((gc_float4*)g)[iw];
+    const f32x4 r = ldg<kNT>((gc_float4*)g + iw);
     out[0] = r.x * us;
     out[1] = r.y * us;
     out[2] = r.z * us;
     out[3] = r.w * us;
   }
+  template <bool kNT>
   static __device__ __forceinline__ f32x4 load4(const void* g, int i4, float us) {
-    const f32x4 r = ((gc_float4*)g)[i4];
+    const f32x4 r = ldg<kNT>((gc_float4*)g + i4);
     return f32x4{r.x * us, r.y * us, r.z * us, r.w * us};
   }
   static __device__ __forceinline__ float load1(const void* g, int i, float us) {
@@ -53,14 +84,16 @@ struct GradIO<float> {
 template <>
 struct GradIO<_Float16> {
   static constexpr int kWide = 8;
+  template <bool kNT>
   static __device__ __forceinline__ void load_wide(const void* g, int iw, float us,
                                                    float (&out)[kWide]) {
-    const half8_t r = ((gc_half8*)g)[iw];
+    const half8_t r = ldg<kNT>((gc_half8*)g + iw);
 #pragma unroll
     for (int j = 0; j < kWide; ++j) out[j] = (float)r[j] * us;
   }
+  template <bool kNT>
   static __device__ __forceinline__ f32x4 load4(const void* g, int i4, float us) {
-    const half4_t r = ((gc_half4*)g)[i4];
+    const half4_t r = ldg<kNT>((gc_half4*)g + i4);
     return f32x4{(float)r.x * us, (float)r.y * us, (float)r.z * us, (float)r.w * us};
   }
   static __device__ __forceinline__ float load1(const void* g, int i, float us) {
@@ -159,15 +192,16 @@ __device__ __forceinline__ void wait_published_n(const double* const (&words)[N]
 
 // A tensor's totals from its chunk partials (kPartialSlots doubles per chunk, N of them starting
 // at `slot`): thread t adds chunks t, t+256, ... in order, then the fixed block tree.  The order
-// depends on nothing but the chunk count.  With kWait the partials are awaited one by one.
+// depends on nothing but the unit count.  A unit is chunks_per_unit chunks (pass A: kChunksPerA)
+// and keeps its partial in its first chunk's slot.  With kWait the partials are awaited.
 template <int N, bool kWait>
-__device__ __forceinline__ void tensor_totals(const double* partials, int slot, int64_t n_chunks,
-                                              double (&tot)[N], double (*red)[kLansWaves],
-                                              SyncHeader* sync) {
+__device__ __forceinline__ void tensor_totals(const double* partials, int slot, int64_t n_units,
+                                              int chunks_per_unit, double (&tot)[N],
+                                              double (*red)[kLansWaves], SyncHeader* sync) {
 #pragma unroll
   for (int j = 0; j < N; ++j) tot[j] = 0.0;
-  for (int64_t i = threadIdx.x; i < n_chunks; i += kLansBlock) {
-    const double* p = partials + kPartialSlots * i + slot;
+  for (int64_t i = threadIdx.x; i < n_units; i += kLansBlock) {
+    const double* p = partials + kPartialSlots * (i * chunks_per_unit) + slot;
     if (kWait) {
       const double* words[N];
       double val[N];
@@ -235,16 +269,17 @@ struct ChunkView {
   int vec_ok;
 };
 
+// `unit` is kChunk for passes B and C and kChunksPerA * kChunk for pass A.
 __device__ __forceinline__ ChunkView chunk_view(const TensorRec& tr, uint32_t chunk,
-                                                int g_elem_bytes) {
-  const int64_t base = (int64_t)chunk * kChunk;
+                                                int g_elem_bytes, int unit = kChunk) {
+  const int64_t base = (int64_t)chunk * unit;
   const int64_t rest = tr.numel - base;
   ChunkView cv;
   cv.g = static_cast<const char*>(tr.g) + base * g_elem_bytes;
   cv.w = tr.w + base;
   cv.m = tr.m + base;
   cv.v = tr.v + base;
-  cv.len = rest < kChunk ? (int)rest : kChunk;
+  cv.len = rest < unit ? (int)rest : unit;
   cv.vec_ok = tr.vec_ok;
   return cv;
 }
@@ -252,7 +287,7 @@ __device__ __forceinline__ ChunkView chunk_view(const TensorRec& tr, uint32_t ch
 // ------------------------------------------------------------------ pass A on one chunk
 // Per-thread contribution to sum g^2 (block reduction is the caller's).  Only the gradient is read:
 // ||w|| is not needed before the trust ratios, so its sum rides along with pass B.
-template <typename G>
+template <typename G, bool kNT>
 __device__ __forceinline__ double chunk_sum_g(const ChunkView& cv, float unscale) {
   constexpr int kW = GradIO<G>::kWide;  // elements per 16-byte lane access
   constexpr int kU = 4;                 // accesses in flight per lane per trip
@@ -265,7 +300,7 @@ __device__ __forceinline__ double chunk_sum_g(const ChunkView& cv, float unscale
       for (int u = 0; u < kU; ++u) {
         const int i = i0 + u * kLansBlock;
         if (i < nw) {
-          GradIO<G>::load_wide(cv.g, i, unscale, x[u]);
+          GradIO<G>::template load_wide<kNT>(cv.g, i, unscale, x[u]);
         } else {
 #pragma unroll
           for (int j = 0; j < kW; ++j) x[u][j] = 0.f;
@@ -296,17 +331,17 @@ struct Batch {
   f32x4 g[kUnroll], w[kUnroll], m[kUnroll], v[kUnroll];
 };
 
-template <typename G>
+template <typename G, bool kGradNT, bool kNT>
 __device__ __forceinline__ void load_batch(Batch& b, const ChunkView& cv, int i0, int n4,
                                            float unscale) {
 #pragma unroll
   for (int u = 0; u < kUnroll; ++u) {
     const int i = i0 + u * kLansBlock;
     if (i < n4) {
-      b.g[u] = GradIO<G>::load4(cv.g, i, unscale);
-      b.w[u] = ((gc_float4*)cv.w)[i];
-      b.m[u] = ((gc_float4*)cv.m)[i];
-      b.v[u] = ((gc_float4*)cv.v)[i];
+      b.g[u] = GradIO<G>::template load4<kGradNT>(cv.g, i, unscale);
+      b.w[u] = ldg<kNT>((gc_float4*)cv.w + i);
+      b.m[u] = ldg<kNT>((gc_float4*)cv.m + i);
+      b.v[u] = ldg<kNT>((gc_float4*)cv.v + i);
     }
   }
 }
@@ -316,7 +351,7 @@ __device__ __forceinline__ void load_batch(Batch& b, const ChunkView& cv, int i0
 // tensor's gradient divisor (the pipelined schedule may have to wait for it).
 // (Issuing trip i+1's loads before evaluating trip i was tried: the extra registers cost a wave of
 // occupancy and the kernels got slower.)
-template <typename G, typename GetInvGdiv>
+template <typename G, bool kGradNT, bool kNT, typename GetInvGdiv>
 __device__ __forceinline__ void chunk_sums_u(const ChunkView& cv, float unscale,
                                              const StepScalars& k, GetInvGdiv&& get_inv_gdiv,
                                              double (&sums)[3]) {
@@ -327,7 +362,7 @@ __device__ __forceinline__ void chunk_sums_u(const ChunkView& cv, float unscale,
     const double inv_gdiv = get_inv_gdiv();
     for (int i0 = threadIdx.x; i0 < n4; i0 += kStride) {
       Batch cur;
-      load_batch<G>(cur, cv, i0, n4, unscale);
+      load_batch<G, kGradNT, kNT>(cur, cv, i0, n4, unscale);
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
         if (i0 + u * kLansBlock < n4) {
@@ -389,7 +424,7 @@ __device__ __forceinline__ Applied apply_one(double g, double w, double m, doubl
 }
 
 // `get_params` supplies the tensor's divisor and trust ratios.
-template <typename G, typename GetParams>
+template <typename G, bool kGradNT, bool kNT, bool kStoreNT, typename GetParams>
 __device__ __forceinline__ void chunk_apply(const ChunkView& cv, float unscale,
                                             const StepScalars& k, GetParams&& get_params) {
   if (cv.vec_ok) {
@@ -398,7 +433,7 @@ __device__ __forceinline__ void chunk_apply(const ChunkView& cv, float unscale,
     const ApplyParams p = get_params();
     for (int i0 = threadIdx.x; i0 < n4; i0 += kStride) {
       Batch cur;
-      load_batch<G>(cur, cv, i0, n4, unscale);
+      load_batch<G, kGradNT, kNT>(cur, cv, i0, n4, unscale);
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
         const int i = i0 + u * kLansBlock;
@@ -407,9 +442,9 @@ __device__ __forceinline__ void chunk_apply(const ChunkView& cv, float unscale,
           const Applied a1 = apply_one(cur.g[u].y, cur.w[u].y, cur.m[u].y, cur.v[u].y, p, k);
           const Applied a2 = apply_one(cur.g[u].z, cur.w[u].z, cur.m[u].z, cur.v[u].z, p, k);
           const Applied a3 = apply_one(cur.g[u].w, cur.w[u].w, cur.m[u].w, cur.v[u].w, p, k);
-          ((g_float4*)cv.w)[i] = f32x4{a0.w, a1.w, a2.w, a3.w};
-          ((g_float4*)cv.m)[i] = f32x4{a0.m, a1.m, a2.m, a3.m};
-          ((g_float4*)cv.v)[i] = f32x4{a0.v, a1.v, a2.v, a3.v};
+          stg<kStoreNT>((g_float4*)cv.w + i, f32x4{a0.w, a1.w, a2.w, a3.w});
+          stg<kStoreNT>((g_float4*)cv.m + i, f32x4{a0.m, a1.m, a2.m, a3.m});
+          stg<kStoreNT>((g_float4*)cv.v + i, f32x4{a0.v, a1.v, a2.v, a3.v});
         }
       }
     }
@@ -465,6 +500,10 @@ __device__ __forceinline__ void stats_after_b(TensorStats* st, const double (&to
 __device__ __forceinline__ int64_t chunks_of(const TensorRec& tr) {
   return (tr.numel + kChunk - 1) / kChunk;
 }
+constexpr int kUnitA = kChunksPerA * kChunk;
+__device__ __forceinline__ int64_t units_a_of(const TensorRec& tr) {
+  return (tr.numel + kUnitA - 1) / kUnitA;
+}
 
 // ------------------------------------------------------------------ set-up launch
 // Host scalars of the reference (lans.cc:94-109), evaluated on the device so that the step tensor
@@ -510,13 +549,15 @@ __global__ __launch_bounds__(kLansBlock) void lans_prepare(LansDeviceArgs a, con
 template <typename G>
 __global__ __launch_bounds__(kLansBlock) void lans_norm_g(LansDeviceArgs a) {
   __shared__ double red[3][kLansWaves];
-  for (int64_t c = blockIdx.x; c < a.n_chunks; c += gridDim.x) {
-    const WorkItem it = a.items[c];
+  for (int64_t i = blockIdx.x; i < a.n_items_a; i += gridDim.x) {
+    const WorkItem it = a.items_a[i];
     const TensorRec tr = a.tensors[it.tensor];
-    const ChunkView cv = chunk_view(tr, it.chunk_phase & kChunkMask, (int)sizeof(G));
-    double s[1] = {chunk_sum_g<G>(cv, a.unscale)};
+    const uint32_t unit = it.chunk_phase & kChunkMask;
+    const ChunkView cv = chunk_view(tr, unit, (int)sizeof(G), kUnitA);
+    double s[1] = {chunk_sum_g<G, kPhasedPolicy.a_g>(cv, a.unscale)};
     block_sum<1>(s, red);
-    if (threadIdx.x == 0) publish(&a.partials[kPartialSlots * c], s[0]);
+    if (threadIdx.x == 0)
+      publish(&a.partials[kPartialSlots * ((int64_t)tr.first_chunk + (int64_t)unit * kChunksPerA)], s[0]);
   }
 }
 
@@ -529,11 +570,11 @@ __global__ __launch_bounds__(kLansBlock) void lans_finish(LansDeviceArgs a, int 
   const StepScalars k = *a.scalars;
   if (after_b) {
     double tot[3], r0, r1;
-    tensor_totals<3, false>(part, 1, chunks_of(tr), tot, red, nullptr);
+    tensor_totals<3, false>(part, 1, chunks_of(tr), 1, tot, red, nullptr);
     if (threadIdx.x == 0) stats_after_b(&a.stats[t], tot, k, r0, r1);
   } else {
     double tot[1];
-    tensor_totals<1, false>(part, 0, chunks_of(tr), tot, red, nullptr);
+    tensor_totals<1, false>(part, 0, units_a_of(tr), kChunksPerA, tot, red, nullptr);
     if (threadIdx.x == 0) stats_after_a(&a.stats[t], tot[0], k);
   }
 }
@@ -542,13 +583,16 @@ template <typename G>
 __global__ __launch_bounds__(kLansBlock) void lans_norm_u(LansDeviceArgs a) {
   __shared__ double red[3][kLansWaves];
   const StepScalars k = *a.scalars;
-  for (int64_t c = blockIdx.x; c < a.n_chunks; c += gridDim.x) {
+  // Back to front: pass A has just streamed the gradients front to back, so the end of the list is
+  // what the Infinity Cache still holds; pass C then starts at the front, where this pass ends.
+  for (int64_t b = blockIdx.x; b < a.n_chunks; b += gridDim.x) {
+    const int64_t c = a.n_chunks - 1 - b;
     const WorkItem it = a.items[c];
     const TensorRec tr = a.tensors[it.tensor];
     const ChunkView cv = chunk_view(tr, it.chunk_phase & kChunkMask, (int)sizeof(G));
     const double inv_gdiv = a.stats[it.tensor].inv_grad_div;
     double s[3];
-    chunk_sums_u<G>(cv, a.unscale, k, [&] { return inv_gdiv; }, s);
+    chunk_sums_u<G, kPhasedPolicy.b_g, kPhasedPolicy.b_wmv>(cv, a.unscale, k, [&] { return inv_gdiv; }, s);
     block_sum<3>(s, red);
     if (threadIdx.x == 0) {
       publish(&a.partials[kPartialSlots * c + 1], s[0]);
@@ -567,7 +611,7 @@ __global__ __launch_bounds__(kLansBlock) void lans_apply(LansDeviceArgs a) {
     const ChunkView cv = chunk_view(tr, it.chunk_phase & kChunkMask, (int)sizeof(G));
     const TensorStats st = a.stats[it.tensor];
     const ApplyParams p{st.inv_grad_div, st.ratio_m, st.ratio_g};
-    chunk_apply<G>(cv, a.unscale, k, [&] { return p; });
+    chunk_apply<G, kPhasedPolicy.c_g, kPhasedPolicy.c_wmv, kPhasedPolicy.c_stores>(cv, a.unscale, k, [&] { return p; });
   }
 }
 
@@ -614,23 +658,25 @@ __global__ __launch_bounds__(kLansBlock) void lans_pipelined(LansDeviceArgs a) {
     const int t = it.tensor;
     const uint32_t phase = it.chunk_phase >> kPhaseShift;
     const uint32_t chunk = it.chunk_phase & kChunkMask;
-    const ChunkView cv = chunk_view(tr, chunk, (int)sizeof(G));
+    const bool unit_a = phase == kPhaseA;  // pass-A items count in units of kChunksPerA chunks
+    const ChunkView cv = chunk_view(tr, chunk, (int)sizeof(G), unit_a ? kUnitA : kChunk);
     const int64_t n_chunks = chunks_of(tr);
-    double* part = a.partials + kPartialSlots * ((int64_t)tr.first_chunk + chunk);
+    double* part = a.partials + kPartialSlots * ((int64_t)tr.first_chunk +
+                                                  (int64_t)chunk * (unit_a ? kChunksPerA : 1));
     const double* tensor_part = a.partials + kPartialSlots * (int64_t)tr.first_chunk;
     TensorStats* st = &a.stats[t];
 
     if (phase == kPhaseA) {
-      double s[1] = {chunk_sum_g<G>(cv, a.unscale)};
+      double s[1] = {chunk_sum_g<G, kPipelinedPolicy.a_g>(cv, a.unscale)};
       block_sum<1>(s, red);
       if (threadIdx.x == 0) publish(part, s[0]);
     } else if (phase == kPhaseFinishA) {
       double tot[1];
-      tensor_totals<1, true>(tensor_part, 0, n_chunks, tot, red, a.sync);
+      tensor_totals<1, true>(tensor_part, 0, units_a_of(tr), kChunksPerA, tot, red, a.sync);
       if (threadIdx.x == 0) stats_after_a(st, tot[0], k);
     } else if (phase == kPhaseB) {
       double s[3];
-      chunk_sums_u<G>(cv, a.unscale, k,
+      chunk_sums_u<G, kPipelinedPolicy.b_g, kPipelinedPolicy.b_wmv>(cv, a.unscale, k,
                       [&] { return wait_published(&st->inv_grad_div, a.sync); }, s);
       block_sum<3>(s, red);
       if (threadIdx.x == 0) {
@@ -640,10 +686,10 @@ __global__ __launch_bounds__(kLansBlock) void lans_pipelined(LansDeviceArgs a) {
       }
     } else if (phase == kPhaseFinishB) {
       double tot[3], r0, r1;
-      tensor_totals<3, true>(tensor_part, 1, n_chunks, tot, red, a.sync);
+      tensor_totals<3, true>(tensor_part, 1, n_chunks, 1, tot, red, a.sync);
       if (threadIdx.x == 0) stats_after_b(st, tot, k, r0, r1);
     } else if (phase == kPhaseC) {
-      chunk_apply<G>(cv, a.unscale, k, [&] {
+      chunk_apply<G, kPipelinedPolicy.c_g, kPipelinedPolicy.c_wmv, kPipelinedPolicy.c_stores>(cv, a.unscale, k, [&] {
         const double* const words[3] = {&st->inv_grad_div, &st->ratio_m, &st->ratio_g};
         double val[3];
         wait_published_n<3>(words, val, a.sync);
@@ -653,18 +699,18 @@ __global__ __launch_bounds__(kLansBlock) void lans_pipelined(LansDeviceArgs a) {
       // A one-chunk tensor: all three passes here, no other workgroup involved.  The totals equal
       // the single chunk partials, exactly as the general path computes them, and travel between
       // the threads through LDS.
-      double s1[1] = {chunk_sum_g<G>(cv, a.unscale)};
+      double s1[1] = {chunk_sum_g<G, false>(cv, a.unscale)};
       block_sum<1>(s1, red);
       if (threadIdx.x == 0) s_bcast[0] = stats_after_a(st, s1[0], k);
       __syncthreads();
       const double inv_gdiv = s_bcast[0];
       double s3[3];
-      chunk_sums_u<G>(cv, a.unscale, k, [&] { return inv_gdiv; }, s3);
+      chunk_sums_u<G, false, false>(cv, a.unscale, k, [&] { return inv_gdiv; }, s3);
       block_sum<3>(s3, red);
       if (threadIdx.x == 0) stats_after_b(st, s3, k, s_bcast[1], s_bcast[2]);
       __syncthreads();
       const ApplyParams p{inv_gdiv, s_bcast[1], s_bcast[2]};
-      chunk_apply<G>(cv, a.unscale, k, [&] { return p; });
+      chunk_apply<G, false, false, true>(cv, a.unscale, k, [&] { return p; });
     }
     if (a.trace && threadIdx.x == 0) {  // diagnostics: when the item was started and finished
       uint64_t* rec = a.trace + 4 * (uint64_t)ticket;
@@ -698,11 +744,12 @@ void launch_phased(int grad_dtype, hipStream_t s, const LansDeviceArgs& a, hipEv
   auto mark = [&](int i) {
     if (marks) (void)hipEventRecord(marks[i], s);
   };
+  const unsigned grid_a = (unsigned)(a.n_items_a < (1 << 20) ? a.n_items_a : (1 << 20));
   mark(0);
   if (f16)
-    hipLaunchKernelGGL(lans_norm_g<_Float16>, dim3(grid), dim3(kLansBlock), 0, s, a);
+    hipLaunchKernelGGL(lans_norm_g<_Float16>, dim3(grid_a), dim3(kLansBlock), 0, s, a);
   else
-    hipLaunchKernelGGL(lans_norm_g<float>, dim3(grid), dim3(kLansBlock), 0, s, a);
+    hipLaunchKernelGGL(lans_norm_g<float>, dim3(grid_a), dim3(kLansBlock), 0, s, a);
   mark(1);
   hipLaunchKernelGGL(lans_finish, dim3((unsigned)a.n_tensors), dim3(kLansBlock), 0, s, a, 0);
   mark(2);

@@ -37,6 +37,9 @@ WorkspaceLayout make_layout(int32_t n_tensors, int64_t n_chunks) {
 }
 
 inline int64_t chunks_of(int64_t numel) { return (numel + kChunk - 1) / kChunk; }
+inline int64_t units_a_of(int64_t numel) {
+  return (numel + (int64_t)kChunksPerA * kChunk - 1) / ((int64_t)kChunksPerA * kChunk);
+}
 
 // Default size of a cache group in elements: the pipelined schedule keeps about three groups'
 // worth of g, w, m, v (14-16 bytes per element) live in the 256 MB Infinity Cache.
@@ -71,8 +74,8 @@ std::vector<WorkItem> build_pipeline(int32_t n, const int64_t* numel, int64_t gr
       g.a.push_back(make_item(t, kPhaseWhole, 0));  // one workgroup does all three passes
       continue;
     }
+    for (int64_t u = 0; u < units_a_of(numel[t]); ++u) g.a.push_back(make_item(t, kPhaseA, u));
     for (int64_t c = 0; c < nc; ++c) {
-      g.a.push_back(make_item(t, kPhaseA, c));
       g.b.push_back(make_item(t, kPhaseB, c));
       g.c.push_back(make_item(t, kPhaseC, c));
     }
@@ -121,10 +124,12 @@ struct rafhip_lans_plan {
   std::vector<int32_t> first_chunk;
   WorkspaceLayout ws{};
 
-  // Device tables in one allocation: [TensorRec x n][phased items x n_chunks][pipeline items].
+  // Device tables in one allocation: [TensorRec x n][chunk items][pipeline items][pass-A items].
   void* d_tables = nullptr;
   TensorRec* d_tensors = nullptr;
   WorkItem* d_items = nullptr;
+  WorkItem* d_items_a = nullptr;
+  int64_t n_items_a = 0;
   WorkItem* d_pipeline = nullptr;
   uint64_t* d_trace = nullptr;  // diagnostics, only with RAFHIP_LANS_TRACE=1
 
@@ -197,6 +202,7 @@ void rafhip_lans_default_hparams(rafhip_lans_hparams* hp) {
 }
 
 int32_t rafhip_lans_chunk_elements(void) { return kChunk; }
+int32_t rafhip_lans_pass_a_unit_elements(void) { return kChunksPerA * kChunk; }
 
 int rafhip_lans_query_layout(int32_t n_tensors, const int64_t* numel, int64_t* n_chunks_out,
                              int64_t* workspace_bytes_out) {
@@ -274,6 +280,10 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
     size_t k = 0;
     for (int32_t t = 0; t < n_tensors; ++t)
       for (int64_t c = 0; c < chunks_of(numel[t]); ++c) phased[k++] = make_item(t, kPhaseA, c);
+    std::vector<WorkItem> phased_a;
+    for (int32_t t = 0; t < n_tensors; ++t)
+      for (int64_t u = 0; u < units_a_of(numel[t]); ++u) phased_a.push_back(make_item(t, kPhaseA, u));
+    p->n_items_a = (int64_t)phased_a.size();
     const std::vector<WorkItem> pipeline = build_pipeline(n_tensors, numel, group_elems_setting());
     p->n_pipeline_items = (uint32_t)pipeline.size();
     // Resident workgroups per CU: never more than fit (every workgroup must be running), and by
@@ -291,7 +301,9 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
     const size_t tensors_bytes = (size_t)align_up((int64_t)sizeof(TensorRec) * n_tensors);
     const size_t phased_bytes = (size_t)align_up((int64_t)sizeof(WorkItem) * (int64_t)phased.size());
     const size_t pipe_bytes = (size_t)align_up((int64_t)sizeof(WorkItem) * (int64_t)pipeline.size());
-    hipError_t e = hipMalloc(&p->d_tables, tensors_bytes + phased_bytes + pipe_bytes + kAlign);
+    const size_t a_bytes = (size_t)align_up((int64_t)sizeof(WorkItem) * (int64_t)phased_a.size());
+    hipError_t e =
+        hipMalloc(&p->d_tables, tensors_bytes + phased_bytes + pipe_bytes + a_bytes + kAlign);
     if (e == hipSuccess)
       e = hipHostMalloc(reinterpret_cast<void**>(&p->h_staging),
                         sizeof(TensorRec) * (size_t)n_tensors, hipHostMallocDefault);
@@ -305,7 +317,11 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
     p->d_tensors = reinterpret_cast<TensorRec*>(base);
     p->d_items = reinterpret_cast<WorkItem*>(base + tensors_bytes);
     p->d_pipeline = reinterpret_cast<WorkItem*>(base + tensors_bytes + phased_bytes);
-    if (!phased.empty())
+    p->d_items_a = reinterpret_cast<WorkItem*>(base + tensors_bytes + phased_bytes + pipe_bytes);
+    if (!phased_a.empty())
+      e = hipMemcpy(p->d_items_a, phased_a.data(), sizeof(WorkItem) * phased_a.size(),
+                    hipMemcpyHostToDevice);
+    if (e == hipSuccess && !phased.empty())
       e = hipMemcpy(p->d_items, phased.data(), sizeof(WorkItem) * phased.size(),
                     hipMemcpyHostToDevice);
     if (e == hipSuccess && !pipeline.empty())
@@ -416,6 +432,8 @@ int rafhip_lans_step(rafhip_lans_plan* plan, const void* const* g, float* const*
   a.n_tensors = n;
   a.items = plan->d_items;
   a.n_chunks = plan->n_chunks;
+  a.items_a = plan->d_items_a;
+  a.n_items_a = plan->n_items_a;
   a.n_items = plan->n_pipeline_items;
   a.pipeline_items = plan->d_pipeline;
   a.unscale = hp->grad_unscale;

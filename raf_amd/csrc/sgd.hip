@@ -9,7 +9,7 @@
 // x86-64, no FMA).  fp32 denormals are kept (no flush-to-zero), as on the CPU.
 //
 // Memory-bound: 12 B read + 8 B written per element.  Each lane moves 16 bytes per access
-// (float4), a wavefront covers 1 KiB per access, and the grid is a fixed multiple of the CU count
+// (four floats), a wavefront covers 1 KiB per access, and the grid is a fixed multiple of the CU count
 // walking the tensor with a grid stride, so consecutive wavefronts touch consecutive 1 KiB lines.
 #include <hip/hip_runtime.h>
 
@@ -21,6 +21,8 @@
 
 namespace rafhip {
 namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));  // native vector (HIP's float4 is a class)
 
 constexpr int kSgdBlock = 256;
 constexpr int kSgdUnroll = 2;  // float4 groups in flight per lane per trip
@@ -35,32 +37,32 @@ __device__ __forceinline__ void sgd_elem(float x0, float dx, float v0, float lr,
 
 // Vector path: all five pointers 16-byte aligned.  n4 = number of whole float4 groups.
 __global__ __launch_bounds__(kSgdBlock) void sgd_vec4_kernel(
-    const float4* x, const float4* dx, const float4* v,
-    float4* v_out, float4* x_out, int64_t n4, float lr, float mu) {
+    const f32x4* x, const f32x4* dx, const f32x4* v, f32x4* v_out, f32x4* x_out, int64_t n4,
+    float lr, float mu) {
   const int64_t stride = (int64_t)gridDim.x * kSgdBlock * kSgdUnroll;
   for (int64_t base = (int64_t)blockIdx.x * kSgdBlock * kSgdUnroll + threadIdx.x; base < n4;
        base += stride) {
-    float4 rx[kSgdUnroll], rd[kSgdUnroll], rv[kSgdUnroll];
+    f32x4 rx[kSgdUnroll], rd[kSgdUnroll], rv[kSgdUnroll];
 #pragma unroll
     for (int u = 0; u < kSgdUnroll; ++u) {
       const int64_t i = base + (int64_t)u * kSgdBlock;
-      if (i < n4) {
-        rx[u] = x[i];
-        rd[u] = dx[i];
-        rv[u] = v[i];
+      if (i < n4) {  // streamed once: non-temporal, so the Infinity Cache does not allocate lines
+        rx[u] = __builtin_nontemporal_load(&x[i]);
+        rd[u] = __builtin_nontemporal_load(&dx[i]);
+        rv[u] = __builtin_nontemporal_load(&v[i]);
       }
     }
 #pragma unroll
     for (int u = 0; u < kSgdUnroll; ++u) {
       const int64_t i = base + (int64_t)u * kSgdBlock;
       if (i < n4) {
-        float4 nv, nx;
-        sgd_elem(rx[u].x, rd[u].x, rv[u].x, lr, mu, nv.x, nx.x);
-        sgd_elem(rx[u].y, rd[u].y, rv[u].y, lr, mu, nv.y, nx.y);
-        sgd_elem(rx[u].z, rd[u].z, rv[u].z, lr, mu, nv.z, nx.z);
-        sgd_elem(rx[u].w, rd[u].w, rv[u].w, lr, mu, nv.w, nx.w);
-        v_out[i] = nv;
-        x_out[i] = nx;
+        float v1[4], x1[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sgd_elem(rx[u][j], rd[u][j], rv[u][j], lr, mu, v1[j], x1[j]);
+        const f32x4 nv = {v1[0], v1[1], v1[2], v1[3]};
+        const f32x4 nx = {x1[0], x1[1], x1[2], x1[3]};
+        __builtin_nontemporal_store(nv, &v_out[i]);
+        __builtin_nontemporal_store(nx, &x_out[i]);
       }
     }
   }
@@ -124,9 +126,9 @@ extern "C" int rafhip_sgd_f32(const float* x, const float* dx, const float* v, f
     int64_t blocks = (n4 + per_block - 1) / per_block;
     if (blocks > cap) blocks = cap;
     hipLaunchKernelGGL(sgd_vec4_kernel, dim3((unsigned)blocks), dim3(kSgdBlock), 0, s,
-                       reinterpret_cast<const float4*>(x), reinterpret_cast<const float4*>(dx),
-                       reinterpret_cast<const float4*>(v), reinterpret_cast<float4*>(v_out),
-                       reinterpret_cast<float4*>(x_out), n4, lr32, mu32);
+                       reinterpret_cast<const f32x4*>(x), reinterpret_cast<const f32x4*>(dx),
+                       reinterpret_cast<const f32x4*>(v), reinterpret_cast<f32x4*>(v_out),
+                       reinterpret_cast<f32x4*>(x_out), n4, lr32, mu32);
     RAFHIP_HIP_TRY(hipGetLastError());
     done = n4 * 4;
   }

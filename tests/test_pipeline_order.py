@@ -5,8 +5,9 @@ import pytest
 KIND_A, KIND_B, KIND_C, KIND_WHOLE, KIND_FIN_A, KIND_FIN_B = range(6)
 
 
-def _check(order, sizes, chunk):
+def _check(order, sizes, chunk, unit_a):
     n_chunks = [-(-n // chunk) for n in sizes]
+    n_units = [-(-n // unit_a) for n in sizes]
     seen = {}
     for pos, (kind, t, c) in enumerate(order):
         assert 0 <= t < len(sizes) and sizes[t] > 0, "empty tensors contribute no work"
@@ -19,13 +20,14 @@ def _check(order, sizes, chunk):
             assert (KIND_WHOLE, t, 0) in seen
             assert not any((k, t, 0) in seen for k in (KIND_A, KIND_B, KIND_C, KIND_FIN_A, KIND_FIN_B))
             continue
-        a = [seen[(KIND_A, t, c)] for c in range(nc)]
+        a = [seen[(KIND_A, t, u)] for u in range(n_units[t])]
+        assert (KIND_A, t, n_units[t]) not in seen
         b = [seen[(KIND_B, t, c)] for c in range(nc)]
         cc = [seen[(KIND_C, t, c)] for c in range(nc)]
         fa, fb = seen[(KIND_FIN_A, t, 0)], seen[(KIND_FIN_B, t, 0)]
         assert max(a) < fa < min(b), f"tensor {t}: finish A must follow its chunks and precede pass B"
         assert max(b) < fb < min(cc), f"tensor {t}: finish B must follow its chunks and precede pass C"
-    expect = sum(1 if nc == 1 else 3 * nc + 2 for nc in n_chunks if nc)
+    expect = sum(1 if nc == 1 else 2 * nc + nu + 2 for nc, nu in zip(n_chunks, n_units) if nc)
     assert len(order) == expect
 
 
@@ -34,15 +36,17 @@ def test_order_invariants(native_libs, group):
     from raf_amd import kernels, shapes
 
     chunk = native_libs.optim().rafhip_lans_chunk_elements()
+    unit_a = native_libs.optim().rafhip_lans_pass_a_unit_elements()
+    assert unit_a % chunk == 0
     lists = [
-        [1, 3, 0, chunk - 1, chunk, chunk + 1, 5 * chunk + 7, 0, 2 * chunk, 17],
+        [1, 3, 0, chunk - 1, chunk, chunk + 1, 5 * chunk + 7, 0, 2 * chunk, 17, unit_a, unit_a + 1, 3 * unit_a - 1],
         shapes.log_uniform_numels(300, seed=7),
         shapes.numels(shapes.bert_base_shapes()),
         [],
         [0, 0],
     ]
     for sizes in lists:
-        _check(kernels.pipeline_order(sizes, group), sizes, chunk)
+        _check(kernels.pipeline_order(sizes, group), sizes, chunk, unit_a)
 
 
 def test_groups_bound_the_reuse_distance(native_libs):
@@ -55,7 +59,7 @@ def test_groups_bound_the_reuse_distance(native_libs):
     order = kernels.pipeline_order(sizes, 16 * chunk)
     first_a = {t: min(i for i, (k, tt, _) in enumerate(order) if k == KIND_A and tt == t) for t in range(40)}
     last_c = {t: max(i for i, (k, tt, _) in enumerate(order) if k == KIND_C and tt == t) for t in range(40)}
-    per_group = 2 * (3 * 8 + 2)
+    per_group = 2 * (2 * 8 + 1 + 2)
     for t in range(40):
         assert last_c[t] - first_a[t] <= 3 * per_group
     # one giant group degenerates into pass-major order: all of A, then all of B, then all of C
@@ -71,5 +75,5 @@ def test_bert_large_group_structure(native_libs):
     sizes = shapes.numels(shapes.bert_large_shapes())
     order = kernels.pipeline_order(sizes)
     chunk = native_libs.optim().rafhip_lans_chunk_elements()
-    _check(order, sizes, chunk)
+    _check(order, sizes, chunk, native_libs.optim().rafhip_lans_pass_a_unit_elements())
     assert sum(1 for k, _, _ in order if k == KIND_WHOLE) == sum(1 for n in sizes if 0 < n <= chunk)
