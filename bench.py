@@ -149,7 +149,9 @@ def bench_lans(name, wl, args):
     total = sum(sizes)
     g, w, m, v = gen_lans(sizes, g16, wl["zero_state"], dev)
     plan = kernels.LansPlan(sizes, torch.float16 if g16 else torch.float32, dev)
-    plan.set_schedule(args.schedule)
+    if args.schedule != "auto":
+        plan.set_schedule(args.schedule)
+    schedule = plan.schedule
     hp = kernels.make_hparams(grad_unscale=(1.0 / 1024 if g16 else 1.0))
     plan.bind(g, w, m, v, hp)
     step_t = torch.full((), float(wl["step0"]), dtype=torch.float32, device=dev)
@@ -185,12 +187,12 @@ def bench_lans(name, wl, args):
                    "bytes_per_element": a + b + c, "bytes_per_step": bytes_step,
                    "kernel_bytes_per_element": ka + kb + kc,
                    "pct_of_hbm_peak": round(100 * bytes_step / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
-                   "schedule": args.schedule, "launches_per_step": 6 if args.schedule == "phased" else 2},
+                   "schedule": schedule, "launches_per_step": 6 if schedule == "phased" else 2},
     }
     if not args.no_kernel_events:
         ts = np.array([plan.timing_read(i) for i in range(args.steps)], dtype=np.float64)
         avg = ts.mean(axis=0)
-        if args.schedule == "phased":
+        if schedule == "phased":
             # dominant kernel: lans_apply (reads g,w,m,v, writes w,m,v)
             apply_ms = float(avg[4])
             achieved = total * c / (apply_ms * 1e-3) / 1e9
@@ -306,8 +308,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="lans_bert_large_fp16grad")
-    ap.add_argument("--schedule", default="phased", choices=["phased", "pipelined"],
-                    help="LANS launch schedule (bit-identical results)")
+    ap.add_argument("--schedule", default="auto", choices=["auto", "phased", "pipelined"],
+                    help="LANS launch schedule (bit-identical results); auto = the library's choice")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline leg")
     ap.add_argument("--no-kernel-events", action="store_true", help="do not record per-kernel HIP events")
     args = ap.parse_args()

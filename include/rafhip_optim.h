@@ -112,7 +112,9 @@ int32_t rafhip_lans_pass_a_unit_elements(void);
  *   PIPELINED  set-up + ONE persistent launch whose work list interleaves the three passes of
  *              neighbouring cache-sized tensor groups, so that a group's second and third reads
  *              come from the 256 MB Infinity Cache instead of HBM.
- * The default can be overridden per process with RAFHIP_LANS_SCHEDULE=phased|pipelined.
+ * A plan picks PIPELINED for lists of 128 Mi elements or more and PHASED below (short lists are
+ * launch- and latency-bound); RAFHIP_LANS_SCHEDULE=phased|pipelined overrides that per process and
+ * rafhip_lans_plan_set_schedule per plan.
  */
 typedef enum rafhip_lans_schedule {
   RAFHIP_LANS_PHASED = 0,
@@ -136,6 +138,7 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
                             rafhip_lans_plan** out_plan);
 int rafhip_lans_plan_destroy(rafhip_lans_plan* plan);
 int rafhip_lans_plan_set_schedule(rafhip_lans_plan* plan, int32_t schedule);
+int32_t rafhip_lans_plan_schedule(const rafhip_lans_plan* plan); /* the schedule in force; -1 on NULL */
 
 /* Bytes of caller-provided scratch a step needs (partial sums, per-tensor norms, flags); 256-byte
  * alignment required.  Returns a negative value on a NULL plan. */

@@ -68,6 +68,7 @@ OPTIM_SYMBOLS = {
     "rafhip_lans_pipeline_order": (c_int, [c_int32, POINTER(c_int64), c_int64, POINTER(c_int32), c_int64,
                                            POINTER(c_int64)]),
     "rafhip_lans_plan_set_schedule": (c_int, [c_void_p, c_int32]),
+    "rafhip_lans_plan_schedule": (c_int32, [c_void_p]),
     "rafhip_lans_query_layout": (c_int, [c_int32, POINTER(c_int64), POINTER(c_int64),
                                          POINTER(c_int64)]),
     "rafhip_lans_plan_create": (c_int, [c_int32, POINTER(c_int64), c_int32, POINTER(c_void_p)]),

@@ -30,12 +30,16 @@ typedef RAFHIP_GLOBAL const _Float16 gc_half;
 // stream worth caching is the gradient in passes B and C: it is the smallest array, pass B walks
 // the list back to front and pass C front to back, so pass C finds the gradients of the front
 // third of the list still cached.  Measured best of nine combinations on the BERT-large list.
-// The pipelined schedule keeps passes A and B temporal because it WANTS their lines to stay.
 struct CachePolicy {  // true = non-temporal
   bool a_g, b_g, b_wmv, c_g, c_wmv, c_stores;
 };
 constexpr CachePolicy kPhasedPolicy = {true, false, true, false, true, true};
-constexpr CachePolicy kPipelinedPolicy = {false, false, false, true, true, true};
+// Pipelined: pass B loads w, m, v temporally so that they are cached when pass C of the same group
+// reads them a round later; pass C reads non-temporally (a hit is consumed, not kept) and writes
+// non-temporally; the gradient is not worth cache space there.  Measured best of seven combinations.
+constexpr CachePolicy kPipelinedPolicy = {true, true, false, true, true, true};
+// Lists whose whole working set fits in the cache (a few million elements) are better off cached.
+constexpr CachePolicy kResidentPolicy = {false, false, false, false, false, false};
 
 template <bool kNT, typename T>
 __device__ __forceinline__ T ldg(const RAFHIP_GLOBAL T* p) {
@@ -546,15 +550,16 @@ __global__ __launch_bounds__(kLansBlock) void lans_prepare(LansDeviceArgs a, con
 }
 
 // ------------------------------------------------------------------ phased schedule
-template <typename G>
+template <typename G, bool kStream>
 __global__ __launch_bounds__(kLansBlock) void lans_norm_g(LansDeviceArgs a) {
+  constexpr CachePolicy kP = kStream ? kPhasedPolicy : kResidentPolicy;
   __shared__ double red[3][kLansWaves];
   for (int64_t i = blockIdx.x; i < a.n_items_a; i += gridDim.x) {
     const WorkItem it = a.items_a[i];
     const TensorRec tr = a.tensors[it.tensor];
     const uint32_t unit = it.chunk_phase & kChunkMask;
     const ChunkView cv = chunk_view(tr, unit, (int)sizeof(G), kUnitA);
-    double s[1] = {chunk_sum_g<G, kPhasedPolicy.a_g>(cv, a.unscale)};
+    double s[1] = {chunk_sum_g<G, kP.a_g>(cv, a.unscale)};
     block_sum<1>(s, red);
     if (threadIdx.x == 0)
       publish(&a.partials[kPartialSlots * ((int64_t)tr.first_chunk + (int64_t)unit * kChunksPerA)], s[0]);
@@ -579,8 +584,9 @@ __global__ __launch_bounds__(kLansBlock) void lans_finish(LansDeviceArgs a, int 
   }
 }
 
-template <typename G>
+template <typename G, bool kStream>
 __global__ __launch_bounds__(kLansBlock) void lans_norm_u(LansDeviceArgs a) {
+  constexpr CachePolicy kP = kStream ? kPhasedPolicy : kResidentPolicy;
   __shared__ double red[3][kLansWaves];
   const StepScalars k = *a.scalars;
   // Back to front: pass A has just streamed the gradients front to back, so the end of the list is
@@ -592,7 +598,7 @@ __global__ __launch_bounds__(kLansBlock) void lans_norm_u(LansDeviceArgs a) {
     const ChunkView cv = chunk_view(tr, it.chunk_phase & kChunkMask, (int)sizeof(G));
     const double inv_gdiv = a.stats[it.tensor].inv_grad_div;
     double s[3];
-    chunk_sums_u<G, kPhasedPolicy.b_g, kPhasedPolicy.b_wmv>(cv, a.unscale, k, [&] { return inv_gdiv; }, s);
+    chunk_sums_u<G, kP.b_g, kP.b_wmv>(cv, a.unscale, k, [&] { return inv_gdiv; }, s);
     block_sum<3>(s, red);
     if (threadIdx.x == 0) {
       publish(&a.partials[kPartialSlots * c + 1], s[0]);
@@ -602,8 +608,9 @@ __global__ __launch_bounds__(kLansBlock) void lans_norm_u(LansDeviceArgs a) {
   }
 }
 
-template <typename G>
+template <typename G, bool kStream>
 __global__ __launch_bounds__(kLansBlock) void lans_apply(LansDeviceArgs a) {
+  constexpr CachePolicy kP = kStream ? kPhasedPolicy : kResidentPolicy;
   const StepScalars k = *a.scalars;
   for (int64_t c = blockIdx.x; c < a.n_chunks; c += gridDim.x) {
     const WorkItem it = a.items[c];
@@ -611,7 +618,7 @@ __global__ __launch_bounds__(kLansBlock) void lans_apply(LansDeviceArgs a) {
     const ChunkView cv = chunk_view(tr, it.chunk_phase & kChunkMask, (int)sizeof(G));
     const TensorStats st = a.stats[it.tensor];
     const ApplyParams p{st.inv_grad_div, st.ratio_m, st.ratio_g};
-    chunk_apply<G, kPhasedPolicy.c_g, kPhasedPolicy.c_wmv, kPhasedPolicy.c_stores>(cv, a.unscale, k, [&] { return p; });
+    chunk_apply<G, kP.c_g, kP.c_wmv, kP.c_stores>(cv, a.unscale, k, [&] { return p; });
   }
 }
 
@@ -738,33 +745,41 @@ void launch_prepare(hipStream_t s, const LansDeviceArgs& a, const float* step_de
                      step_host, hp);
 }
 
-void launch_phased(int grad_dtype, hipStream_t s, const LansDeviceArgs& a, hipEvent_t* marks) {
+namespace {
+template <typename G, bool kStream>
+void launch_phased_t(hipStream_t s, const LansDeviceArgs& a, hipEvent_t* marks) {
   const unsigned grid = (unsigned)(a.n_chunks < (1 << 20) ? a.n_chunks : (1 << 20));
-  const bool f16 = grad_dtype == RAFHIP_F16;
+  const unsigned grid_a = (unsigned)(a.n_items_a < (1 << 20) ? a.n_items_a : (1 << 20));
   auto mark = [&](int i) {
     if (marks) (void)hipEventRecord(marks[i], s);
   };
-  const unsigned grid_a = (unsigned)(a.n_items_a < (1 << 20) ? a.n_items_a : (1 << 20));
   mark(0);
-  if (f16)
-    hipLaunchKernelGGL(lans_norm_g<_Float16>, dim3(grid_a), dim3(kLansBlock), 0, s, a);
-  else
-    hipLaunchKernelGGL(lans_norm_g<float>, dim3(grid_a), dim3(kLansBlock), 0, s, a);
+  hipLaunchKernelGGL((lans_norm_g<G, kStream>), dim3(grid_a), dim3(kLansBlock), 0, s, a);
   mark(1);
   hipLaunchKernelGGL(lans_finish, dim3((unsigned)a.n_tensors), dim3(kLansBlock), 0, s, a, 0);
   mark(2);
-  if (f16)
-    hipLaunchKernelGGL(lans_norm_u<_Float16>, dim3(grid), dim3(kLansBlock), 0, s, a);
-  else
-    hipLaunchKernelGGL(lans_norm_u<float>, dim3(grid), dim3(kLansBlock), 0, s, a);
+  hipLaunchKernelGGL((lans_norm_u<G, kStream>), dim3(grid), dim3(kLansBlock), 0, s, a);
   mark(3);
   hipLaunchKernelGGL(lans_finish, dim3((unsigned)a.n_tensors), dim3(kLansBlock), 0, s, a, 1);
   mark(4);
-  if (f16)
-    hipLaunchKernelGGL(lans_apply<_Float16>, dim3(grid), dim3(kLansBlock), 0, s, a);
-  else
-    hipLaunchKernelGGL(lans_apply<float>, dim3(grid), dim3(kLansBlock), 0, s, a);
+  hipLaunchKernelGGL((lans_apply<G, kStream>), dim3(grid), dim3(kLansBlock), 0, s, a);
   mark(5);
+}
+}  // namespace
+
+void launch_phased(int grad_dtype, bool streaming, hipStream_t s, const LansDeviceArgs& a,
+                   hipEvent_t* marks) {
+  if (grad_dtype == RAFHIP_F16) {
+    if (streaming)
+      launch_phased_t<_Float16, true>(s, a, marks);
+    else
+      launch_phased_t<_Float16, false>(s, a, marks);
+  } else {
+    if (streaming)
+      launch_phased_t<float, true>(s, a, marks);
+    else
+      launch_phased_t<float, false>(s, a, marks);
+  }
 }
 
 void launch_pipelined(int grad_dtype, unsigned grid, hipStream_t s, const LansDeviceArgs& a) {

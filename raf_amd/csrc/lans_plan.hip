@@ -41,9 +41,15 @@ inline int64_t units_a_of(int64_t numel) {
   return (numel + (int64_t)kChunksPerA * kChunk - 1) / ((int64_t)kChunksPerA * kChunk);
 }
 
-// Default size of a cache group in elements: the pipelined schedule keeps about three groups'
-// worth of g, w, m, v (14-16 bytes per element) live in the 256 MB Infinity Cache.
-constexpr int64_t kDefaultGroupElems = 4608 * 1024;
+// Default size of a cache group in elements (measured optimum on MI355X for BERT-large and
+// GPT-2-1.5B lists): pass C of a group finds the 12 bytes per element of w, m, v that pass B of the
+// same group left in the 256 MB Infinity Cache one round earlier.
+constexpr int64_t kDefaultGroupElems = 13 * 1000 * 1000;
+// Lists at least this long run pipelined by default; shorter ones are launch- and latency-bound
+// and do better with one launch per pass.
+constexpr int64_t kPipelinedFromElems = 128 * 1024 * 1024;
+// Lists whose g, w, m, v together stay under this many bytes fit in the cache: temporal accesses.
+constexpr int64_t kResidentBytes = 192LL << 20;
 
 inline WorkItem make_item(int32_t tensor, uint32_t phase, int64_t chunk) {
   return WorkItem{tensor, (phase << kPhaseShift) | (uint32_t)chunk};
@@ -100,12 +106,12 @@ int64_t group_elems_setting() {
   return kDefaultGroupElems;
 }
 
-int schedule_setting() {
+int schedule_setting(int64_t total_elements) {
   if (const char* e = std::getenv("RAFHIP_LANS_SCHEDULE")) {
     if (!std::strcmp(e, "phased")) return RAFHIP_LANS_PHASED;
     if (!std::strcmp(e, "pipelined")) return RAFHIP_LANS_PIPELINED;
   }
-  return RAFHIP_LANS_PHASED;
+  return total_elements >= kPipelinedFromElems ? RAFHIP_LANS_PIPELINED : RAFHIP_LANS_PHASED;
 }
 
 }  // namespace
@@ -252,7 +258,6 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
   if (!p) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_plan_create: out of host memory");
   p->n_tensors = n_tensors;
   p->grad_dtype = grad_dtype;
-  p->schedule = schedule_setting();
   p->numel.assign(numel, numel + n_tensors);
   p->first_chunk.resize(n_tensors);
   int64_t chunks = 0, total = 0;
@@ -263,6 +268,7 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
   }
   p->n_chunks = chunks;
   p->total_elements = total;
+  p->schedule = schedule_setting(total);
   p->ws = make_layout(n_tensors, chunks);
 
   if (hipGetDevice(&p->device) != hipSuccess) {
@@ -353,6 +359,8 @@ int rafhip_lans_plan_set_schedule(rafhip_lans_plan* plan, int32_t schedule) {
   plan->schedule = schedule;
   return RAFHIP_OK;
 }
+
+int32_t rafhip_lans_plan_schedule(const rafhip_lans_plan* plan) { return plan ? plan->schedule : -1; }
 
 int64_t rafhip_lans_workspace_bytes(const rafhip_lans_plan* plan) {
   return plan ? plan->ws.total : -1;
@@ -467,7 +475,9 @@ int rafhip_lans_step(rafhip_lans_plan* plan, const void* const* g, float* const*
       for (int i = 2; i < 6; ++i) RAFHIP_HIP_TRY(hipEventRecord(marks[i], s));
   } else {
     launch_prepare(s, a, step_dev, step_host, pod);
-    launch_phased(plan->grad_dtype, s, a, marks);
+    const int64_t bytes_per_elt = plan->grad_dtype == RAFHIP_F16 ? 14 : 16;
+    launch_phased(plan->grad_dtype, plan->total_elements * bytes_per_elt > kResidentBytes, s, a,
+                  marks);
   }
   RAFHIP_HIP_TRY(hipGetLastError());
   plan->steps_done++;

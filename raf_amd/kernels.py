@@ -103,6 +103,10 @@ class LansPlan:
         code = {"phased": _lib.RAFHIP_LANS_PHASED, "pipelined": _lib.RAFHIP_LANS_PIPELINED}[schedule]
         check(self.lib.rafhip_lans_plan_set_schedule(self._h, code))
 
+    @property
+    def schedule(self) -> str:
+        return {0: "phased", 1: "pipelined"}[self.lib.rafhip_lans_plan_schedule(self._h)]
+
     def close(self):
         if self._h:
             self.lib.rafhip_lans_plan_destroy(self._h)
