@@ -41,9 +41,11 @@ SGD_BYTES_PER_ELT = 20  # read x, dx, v; write v1, x1
 
 # Memory traffic per launch of the dominant kernel (bytes), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs scaled by a plain 1 GiB copy (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); figures and commands are in
-# profiles/lans_phased_bert_large_fp16grad.md.  Workloads not listed were not measured (null).
+# profiles/.  Workloads not listed were not measured (null).
 MEASURED_TRAFFIC = {
-    ("lans_bert_large_fp16grad", "lans_apply"): 8_717_300_000,
+    ("lans_bert_large_fp16grad", "lans_pipelined"): 14_088_400_000,
+    ("lans_bert_large_fp16grad", "lans_apply"): 8_716_600_000,
+    ("sgd_4m_fp32", "sgd_vec4_kernel"): 83_925_600,
 }
 
 
@@ -213,7 +215,11 @@ def bench_lans(name, wl, args):
             out["roofline"] = {"bound": "hbm", "kernel": "lans_pipelined", "achieved": round(achieved, 1),
                                "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                                "traffic": MEASURED_TRAFFIC.get((name, "lans_pipelined")),
-                               "bytes_per_launch": bytes_step, "avg_launch_ms": round(k_ms, 4)}
+                               "bytes_per_launch": bytes_step, "avg_launch_ms": round(k_ms, 4),
+                               # the same launch priced by the bytes the kernel requests (the norm of w
+                               # rides on pass B) and by the compulsory read-once/write-once bytes
+                               "achieved_by_requested_bytes": round(total * (ka + kb + kc) / (k_ms * 1e-3) / 1e9, 1),
+                               "achieved_by_compulsory_bytes": round(total * c / (k_ms * 1e-3) / 1e9, 1)}
             out["kernels_ms"] = {"lans_prepare": round(float(avg[0]), 4), "lans_pipelined": round(k_ms, 4)}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline_lans(sizes, g16)

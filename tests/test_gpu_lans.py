@@ -240,13 +240,34 @@ def test_workspace_and_argument_errors(native_libs):
 
 
 # ------------------------------------------------------------------ the two schedules
+def test_default_schedule_follows_list_length(native_libs, monkeypatch):
+    """Lists of 128 Mi elements or more run pipelined, shorter ones phased; the environment variable
+    and the per-plan setter override that."""
+    from raf_amd import kernels
+
+    monkeypatch.delenv("RAFHIP_LANS_SCHEDULE", raising=False)
+    for sizes, want in (([1000, 5], "phased"), ([(1 << 27) - 1], "phased"), ([1 << 26, 1 << 26], "pipelined")):
+        plan = kernels.LansPlan(sizes, torch.float32, DEV)
+        assert plan.schedule == want, sizes
+        plan.set_schedule("pipelined" if want == "phased" else "phased")
+        assert plan.schedule != want
+        plan.close()
+    monkeypatch.setenv("RAFHIP_LANS_SCHEDULE", "pipelined")
+    plan = kernels.LansPlan([1000, 5], torch.float32, DEV)
+    assert plan.schedule == "pipelined"
+    plan.close()
+
+
+@pytest.mark.parametrize("group_elems", [None, 1 << 20])
 @pytest.mark.parametrize("g16", [False, True])
-def test_pipelined_schedule_is_bitwise_equal_to_phased(native_libs, g16):
+def test_pipelined_schedule_is_bitwise_equal_to_phased(native_libs, monkeypatch, g16, group_elems):
     """The persistent, cache-aware schedule runs the same per-chunk code and adds the same partials
     in the same order as the five-launch schedule: every output bit must agree, and both must
     match the oracle."""
     from raf_amd import kernels, shapes
 
+    if group_elems is not None:  # small cache groups: many rounds, three passes in flight at once
+        monkeypatch.setenv("RAFHIP_LANS_GROUP_ELEMS", str(group_elems))
     cases = {
         "edge": [1, 3, 4, 5, 0, 255, 1023, 8191, 8192, 8193, 16385, 65537, 100003],
         "many small": shapes.log_uniform_numels(400, seed=3),
