@@ -55,6 +55,9 @@ def workloads():
     return {
         "lans_bert_large_fp16grad": dict(kind="lans", sizes=shapes.numels(shapes.bert_large_shapes()), g16=True,
                                          zero_state=True, step0=1),
+        # half-precision model with fp32 master weights: fp16 gradients in, fp16 weight copies out
+        "lans_bert_large_mixed_fp16": dict(kind="lans", sizes=shapes.numels(shapes.bert_large_shapes()), g16=True,
+                                           zero_state=True, step0=1, copy16=True),
         "lans_bert_large_fp32grad": dict(kind="lans", sizes=shapes.numels(shapes.bert_large_shapes()), g16=False,
                                          zero_state=True, step0=1),
         "lans_bert_base_fp32": dict(kind="lans", sizes=shapes.numels(shapes.bert_base_shapes()), g16=False,
@@ -155,7 +158,9 @@ def bench_lans(name, wl, args):
         plan.set_schedule(args.schedule)
     schedule = plan.schedule
     hp = kernels.make_hparams(grad_unscale=(1.0 / 1024 if g16 else 1.0))
-    plan.bind(g, w, m, v, hp)
+    copy16 = bool(wl.get("copy16"))
+    p16 = [torch.empty(n, dtype=torch.float16, device=dev) for n in sizes] if copy16 else None
+    plan.bind(g, w, m, v, hp, p=p16)
     step_t = torch.full((), float(wl["step0"]), dtype=torch.float32, device=dev)
 
     for _ in range(args.warmup):
@@ -174,6 +179,8 @@ def bench_lans(name, wl, args):
 
     a, b, c = lans_bytes_per_elt(2 if g16 else 4)
     ka, kb, kc = lans_kernel_bytes_per_elt(2 if g16 else 4)
+    if copy16:  # the third pass also writes the 2-byte copy of the new weight
+        c, kc = c + 2, kc + 2
     bytes_step = total * (a + b + c)
     out = {
         "metric": "LANS optimizer-step achieved HBM bandwidth (algorithmic bytes / step time); "
@@ -185,7 +192,8 @@ def bench_lans(name, wl, args):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f64", "data": "synthetic",
         "config": {"workload": name, "tensors": len(sizes), "elements": total,
-                   "storage": "fp32 w/m/v, " + ("fp16 g (x1024, unscaled in kernel)" if g16 else "fp32 g"),
+                   "storage": "fp32 w/m/v, " + ("fp16 g (x1024, unscaled in kernel)" if g16 else "fp32 g") +
+                              (", fp16 copy of the new weights written" if copy16 else ""),
                    "bytes_per_element": a + b + c, "bytes_per_step": bytes_step,
                    "kernel_bytes_per_element": ka + kb + kc,
                    "pct_of_hbm_peak": round(100 * bytes_step / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),

@@ -25,7 +25,7 @@ typedef struct rafhip_tensor_desc {
   void* data;
   int32_t device_type; /* 1 cpu, 2 cuda, 10 rocm (include/raf/device.h:37-50) */
   int32_t device_id;
-  int32_t dtype_code;  /* DLPack: 0 int, 1 uint, 2 float */
+  int32_t dtype_code;  /* DLPack: 0 int, 1 uint, 2 float, 4 bfloat */
   int32_t dtype_bits;
   int32_t ndim;
   const int64_t* shape;
@@ -63,6 +63,16 @@ int rafhip_raf_lans_make(int32_t list_len, const rafhip_tensor_desc* tensor_list
                          float beta2, float eps, int32_t bias_correction, float weight_decay,
                          int32_t grad_averaging, int32_t mode, int32_t normalize_grad,
                          rafhip_raf_env** env_out);
+/* Extension op raf.op.lans_mixed (no counterpart in the reference's op set): the same arguments
+ * with a tensor_list of 5n descriptors g..., w..., m..., v..., p..., where p are the model's
+ * float16 / bfloat16 parameters; they receive the new fp32 weights narrowed to 16 bits, which the
+ * reference's traced optimizer does with a cast and a copy after raf.op.lans
+ * (python/raf/optim/lans.py:289-291, :303-305).  Execute with rafhip_raf_lans_execute. */
+int rafhip_raf_lans_mixed_make(int32_t list_len, const rafhip_tensor_desc* tensor_list,
+                               const rafhip_tensor_desc* step, float learning_rate, float beta1,
+                               float beta2, float eps, int32_t bias_correction, float weight_decay,
+                               int32_t grad_averaging, int32_t mode, int32_t normalize_grad,
+                               rafhip_raf_env** env_out);
 int rafhip_raf_lans_execute(rafhip_raf_env* env, int32_t list_len,
                             const rafhip_tensor_desc* tensor_list, const rafhip_tensor_desc* step,
                             void* workspace, int64_t workspace_bytes, void* stream);

@@ -42,7 +42,8 @@ typedef enum rafhip_status {
 
 typedef enum rafhip_dtype {
   RAFHIP_F32 = 0,
-  RAFHIP_F16 = 1 /* IEEE binary16; accepted for LANS gradients only */
+  RAFHIP_F16 = 1, /* IEEE binary16; LANS gradients and 16-bit weight copies only */
+  RAFHIP_BF16 = 2 /* bfloat16; LANS gradients and 16-bit weight copies only      */
 } rafhip_dtype;
 
 /* ABI version of the loaded library (== RAFHIP_ABI_VERSION it was built with). */
@@ -166,6 +167,23 @@ int rafhip_lans_step(rafhip_lans_plan* plan, const void* const* g, float* const*
                      float* const* m, float* const* v, const float* step_dev, int32_t step_host,
                      const rafhip_lans_hparams* hp, void* workspace, int64_t workspace_bytes,
                      void* stream);
+
+/*
+ * The same step for a half-precision model with fp32 master weights, i.e. what the reference's
+ * traced optimizer builds around raf.op.lans out of three more ops (python/raf/optim/lans.py):
+ *   - gradients of the plan's dtype (binary16 / bfloat16) are widened on load, replacing
+ *     `_op.group_cast(g_list, "float32")` (:261-265) and the fp32 gradient copies it materialises;
+ *   - p[i], when p is not NULL, receives the NEW fp32 weight narrowed to p_dtype (RAFHIP_F16 or
+ *     RAFHIP_BF16) with round to nearest even, replacing `_op.cast(new_w, dtype)` and the copy into
+ *     the model's parameter `_op.add(new_w, zero, out=p)` (:289-291, :303-305).
+ * p is a host array of n_tensors device pointers (2-byte elements, numel[i] each; an entry may be
+ * NULL to skip that tensor).  With p == NULL this is rafhip_lans_step.
+ */
+int rafhip_lans_step_mixed(rafhip_lans_plan* plan, const void* const* g, float* const* w,
+                           float* const* m, float* const* v, void* const* p, int32_t p_dtype,
+                           const float* step_dev, int32_t step_host,
+                           const rafhip_lans_hparams* hp, void* workspace,
+                           int64_t workspace_bytes, void* stream);
 
 /* Copies the per-tensor norms left in the workspace by the last step on `stream`
  * (4 doubles per tensor: ||g||, ||w||, ||u_m||, ||u_g||) to host memory; synchronises `stream`. */

@@ -44,7 +44,11 @@ def lib():
         l.oracle_lans_step.restype = None
         l.oracle_lans_step.argtypes = [c_int32, POINTER(c_int64), POINTER(c_void_p), c_int,
                                        POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
-                                       c_float, POINTER(OracleHParams), POINTER(c_double), c_int]
+                                       c_float, POINTER(OracleHParams), POINTER(c_double), c_int,
+                                       POINTER(c_void_p), c_int]
+        for fn in (l.oracle_f32_to_f16_bits, l.oracle_f32_to_bf16_bits):
+            fn.restype = None
+            fn.argtypes = [c_void_p, c_void_p, c_int64]
         l.oracle_max_threads.restype = c_int
         _lib = l
     return _lib
@@ -72,14 +76,32 @@ def hparams_from(hp) -> OracleHParams:
                          int(bool(hp.normalize_grad)), hp.grad_unscale)
 
 
-def lans_step_inplace(g_list, w_list, m_list, v_list, step, hp, threads: int = 0):
-    """In place on the fp32 arrays of w/m/v; g may be fp32 or fp16 arrays.  Returns [n,4] norms."""
+_DTYPE_CODE = {np.dtype(np.float32): 0, np.dtype(np.float16): 1, np.dtype(np.uint16): 2}
+
+
+def narrow_bits(x, dtype: str):
+    """fp32 -> float16 / bfloat16 bit patterns (uint16) with the C oracle's own conversions."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(x.shape, dtype=np.uint16)
+    fn = lib().oracle_f32_to_bf16_bits if dtype == "bfloat16" else lib().oracle_f32_to_f16_bits
+    fn(x.ctypes.data, out.ctypes.data, x.size)
+    return out
+
+
+def lans_step_inplace(g_list, w_list, m_list, v_list, step, hp, threads: int = 0, p_list=None,
+                      model_dtype: str = "float16"):
+    """In place on the fp32 arrays of w/m/v; g may be fp32, fp16 or uint16 (bfloat16 bit patterns)
+    arrays.  ``p_list``: optional uint16/float16 arrays that receive the new weights narrowed to
+    ``model_dtype``.  Returns [n,4] norms."""
     n = len(w_list)
-    g_is_f16 = int(n > 0 and g_list[0].dtype == np.float16)
-    for arrs, dt in ((g_list, np.float16 if g_is_f16 else np.float32), (w_list, np.float32),
-                     (m_list, np.float32), (v_list, np.float32)):
+    gdt = g_list[0].dtype if n > 0 else np.dtype(np.float32)
+    g_dtype = _DTYPE_CODE[np.dtype(gdt)]
+    for arrs, dt in ((g_list, gdt), (w_list, np.float32), (m_list, np.float32), (v_list, np.float32)):
         for a in arrs:
             assert a.dtype == dt and a.flags.c_contiguous, (a.dtype, dt)
+    if p_list is not None:
+        for a, w in zip(p_list, w_list):
+            assert a.dtype.itemsize == 2 and a.flags.c_contiguous and a.size == w.size
     numel = (c_int64 * max(n, 1))(*[int(a.size) for a in w_list])
 
     def ptrs(arrs):
@@ -87,7 +109,9 @@ def lans_step_inplace(g_list, w_list, m_list, v_list, step, hp, threads: int = 0
 
     norms = np.zeros((n, 4), dtype=np.float64)
     ohp = hparams_from(hp)
-    lib().oracle_lans_step(n, numel, ptrs(g_list), g_is_f16, ptrs(w_list), ptrs(m_list),
+    lib().oracle_lans_step(n, numel, ptrs(g_list), g_dtype, ptrs(w_list), ptrs(m_list),
                            ptrs(v_list), float(np.float32(step)), ctypes.byref(ohp),
-                           norms.ctypes.data_as(POINTER(c_double)), int(threads))
+                           norms.ctypes.data_as(POINTER(c_double)), int(threads),
+                           ptrs(p_list) if p_list is not None else None,
+                           2 if model_dtype == "bfloat16" else 1)
     return norms

@@ -43,6 +43,8 @@ from typing import List, Sequence, Tuple
 
 import numpy as np
 
+from oracle.halfs import narrow_weight, widen_grad
+
 
 def f32(x) -> float:
     """Round a Python number to fp32 and return it as a Python float."""
@@ -100,9 +102,11 @@ def lans_scalars(hp: LansHParams, step) -> LansScalars:
 
 
 def grad_to_f64(g: np.ndarray, hp: LansHParams) -> np.ndarray:
-    """Gradient ingest: any float dtype -> fp32, times the fp32 unscale
-    factor (one fp32 rounding; exact for powers of two), then float64."""
-    g32 = np.asarray(g).astype(np.float32) * np.float32(hp.grad_unscale)
+    """Gradient ingest: float32, float16 or bfloat16 (uint16 bit patterns) ->
+    fp32 exactly as ``group_cast`` widens it (python/raf/optim/lans.py:261-265),
+    times the fp32 unscale factor (one fp32 rounding; exact for powers of
+    two), then float64."""
+    g32 = widen_grad(g) * np.float32(hp.grad_unscale)
     return g32.astype(np.float64)
 
 
@@ -177,6 +181,18 @@ def lans_step(
         vs.append(v1.astype(state_dtype).reshape(shape))
         norms[t] = nr
     return ws, ms, vs, norms
+
+
+def lans_mixed_step(g_list, w_list, m_list, v_list, step, hp: LansHParams = LansHParams(),
+                    model_dtype: str = "float16"):
+    """The mixed-precision step of the reference's wrapper: ``lans_step`` on
+    the fp32 master weights, then the model's half-precision parameters as
+    ``cast(new_w, dtype)`` of the *stored fp32* weight (python/raf/optim/
+    lans.py:289-291, :303-305).  Returns ``(ws, ms, vs, ps, norms)``; ``ps``
+    are float16 arrays or bfloat16 bit patterns (uint16)."""
+    ws, ms, vs, norms = lans_step(g_list, w_list, m_list, v_list, step, hp, np.float32)
+    ps = [narrow_weight(w, model_dtype) for w in ws]
+    return ws, ms, vs, ps, norms
 
 
 def lans_flat_list_step(tensor_list, step, hp: LansHParams = LansHParams(), state_dtype=np.float32):

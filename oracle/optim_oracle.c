@@ -82,8 +82,60 @@ static float half_to_float(uint16_t h) {
   return f;
 }
 
-static inline double load_grad(const void* g, int g_is_f16, int64_t i, float unscale) {
-  float g32 = g_is_f16 ? half_to_float(((const uint16_t*)g)[i]) : ((const float*)g)[i];
+/* bfloat16 -> float: the pattern is the upper half of the fp32 word. */
+static float bf16_to_float(uint16_t h) {
+  uint32_t bits = (uint32_t)h << 16;
+  float f;
+  memcpy(&f, &bits, 4);
+  return f;
+}
+
+/* float -> IEEE binary16, round to nearest even, bit-level.  This is the `cast(new_w, "float16")`
+ * of the mixed-precision wrapper (python/raf/optim/lans.py:289-291). */
+static uint16_t float_to_half(float f) {
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  const uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+  const uint32_t ax = x & 0x7fffffffu;
+  if (ax > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);  /* NaN */
+  if (ax >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u); /* >= 65520 rounds to infinity */
+  if (ax <= 0x33000000u) return sign;                       /* <= 2^-25 rounds to zero */
+  const uint32_t exp = ax >> 23;
+  if (exp < 113) { /* below 2^-14: a binary16 subnormal, unit 2^-24 */
+    const uint32_t man = (ax & 0x7fffffu) | 0x800000u;
+    const uint32_t shift = 126 - exp; /* 14 .. 24 */
+    uint32_t h = man >> shift;
+    const uint32_t rem = man & ((1u << shift) - 1u), half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (h & 1u))) ++h;
+    return (uint16_t)(sign | h);
+  }
+  uint32_t h = ((exp - 112u) << 10) | ((ax & 0x7fffffu) >> 13);
+  const uint32_t rem = ax & 0x1fffu;
+  if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) ++h; /* a carry moves into the exponent */
+  return (uint16_t)(sign | h);
+}
+
+/* float -> bfloat16, round to nearest even (add-and-shift); NaN stays a quiet NaN. */
+static uint16_t float_to_bf16(float f) {
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x0040u);
+  return (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);
+}
+
+void oracle_f32_to_f16_bits(const float* x, uint16_t* out, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) out[i] = float_to_half(x[i]);
+}
+void oracle_f32_to_bf16_bits(const float* x, uint16_t* out, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) out[i] = float_to_bf16(x[i]);
+}
+
+/* Gradient dtypes: 0 = fp32, 1 = binary16, 2 = bfloat16; widening is exact, as group_cast's is
+ * (python/raf/optim/lans.py:261-265). */
+static inline double load_grad(const void* g, int g_dtype, int64_t i, float unscale) {
+  float g32 = g_dtype == 1   ? half_to_float(((const uint16_t*)g)[i])
+              : g_dtype == 2 ? bf16_to_float(((const uint16_t*)g)[i])
+                             : ((const float*)g)[i];
   float scaled = g32 * unscale; /* one fp32 rounding, exact for powers of two */
   return (double)scaled;
 }
@@ -98,14 +150,14 @@ static double ordered_total(const double* part, int64_t nb) {
   return total;
 }
 
-static double sumsq_grad(const void* g, int g_is_f16, int64_t n, float unscale, double* part) {
+static double sumsq_grad(const void* g, int g_dtype, int64_t n, float unscale, double* part) {
   int64_t nb = (n + ORACLE_BLOCK - 1) / ORACLE_BLOCK;
 #pragma omp parallel for schedule(static) if (n > (1 << 16))
   for (int64_t b = 0; b < nb; ++b) {
     int64_t lo = b * ORACLE_BLOCK, hi = lo + ORACLE_BLOCK < n ? lo + ORACLE_BLOCK : n;
     double s = 0.0;
     for (int64_t i = lo; i < hi; ++i) {
-      double x = load_grad(g, g_is_f16, i, unscale);
+      double x = load_grad(g, g_dtype, i, unscale);
       s += x * x;
     }
     part[b] = s;
@@ -178,12 +230,15 @@ static inline void directions(double g, double w, double m, double v, const scal
 
 /*
  * One LANS step over n tensors, in place on w/m/v (fp32 storage, float64 arithmetic).
- * g[t] points at numel[t] gradients (fp32, or binary16 when g_is_f16); g is not modified.
+ * g[t] points at numel[t] gradients of dtype g_dtype (0 fp32, 1 binary16, 2 bfloat16); g is not
+ * modified.  If p is not NULL, p[t] receives the stored fp32 weight narrowed to p_dtype (1 binary16,
+ * 2 bfloat16): the model's half-precision parameter (python/raf/optim/lans.py:289-291, :303-305).
  * norms_out, if not NULL, receives 4 doubles per tensor: ||g||, ||w||, ||u_m||, ||u_g||.
  */
-void oracle_lans_step(int32_t n_tensors, const int64_t* numel, const void* const* g, int g_is_f16,
+void oracle_lans_step(int32_t n_tensors, const int64_t* numel, const void* const* g, int g_dtype,
                       float* const* w, float* const* m, float* const* v, float step_value,
-                      const oracle_lans_hparams* hp, double* norms_out, int threads) {
+                      const oracle_lans_hparams* hp, double* norms_out, int threads,
+                      uint16_t* const* p, int p_dtype) {
   scalars_t s = make_scalars(hp, step_value);
 #ifdef _OPENMP
   if (threads > 0) omp_set_num_threads(threads);
@@ -198,7 +253,7 @@ void oracle_lans_step(int32_t n_tensors, const int64_t* numel, const void* const
     int64_t nb = (n + ORACLE_BLOCK - 1) / ORACLE_BLOCK;
     double* part = (double*)malloc((size_t)(2 * nb + 2) * sizeof(double));
     double* part2 = part + nb + 1;
-    const double gn = sqrt(sumsq_grad(gt, g_is_f16, n, us, part));
+    const double gn = sqrt(sumsq_grad(gt, g_dtype, n, us, part));
     const double pn = sqrt(sumsq_f32(wt, n, part));
 
 #pragma omp parallel for schedule(static) if (n > (1 << 16))
@@ -207,7 +262,7 @@ void oracle_lans_step(int32_t n_tensors, const int64_t* numel, const void* const
       double a = 0.0, c = 0.0;
       for (int64_t i = lo; i < hi; ++i) {
         double m1, v1, um, ug;
-        directions(load_grad(gt, g_is_f16, i, us), wt[i], mt[i], vt[i], &s, hp->normalize_grad, gn,
+        directions(load_grad(gt, g_dtype, i, us), wt[i], mt[i], vt[i], &s, hp->normalize_grad, gn,
                    hp->mode, &m1, &v1, &um, &ug);
         a += um * um;
         c += ug * ug;
@@ -225,9 +280,10 @@ void oracle_lans_step(int32_t n_tensors, const int64_t* numel, const void* const
     for (int64_t i = 0; i < n; ++i) {
       double m1, v1, um, ug;
       double w0 = wt[i];
-      directions(load_grad(gt, g_is_f16, i, us), w0, mt[i], vt[i], &s, hp->normalize_grad, gn,
+      directions(load_grad(gt, g_dtype, i, us), w0, mt[i], vt[i], &s, hp->normalize_grad, gn,
                  hp->mode, &m1, &v1, &um, &ug);
       wt[i] = (float)(w0 - rm * um - rg * ug);
+      if (p) p[t][i] = p_dtype == 2 ? float_to_bf16(wt[i]) : float_to_half(wt[i]);
       mt[i] = (float)m1;
       vt[i] = (float)v1;
     }

@@ -23,6 +23,7 @@ RAFHIP_ERR_NO_DEVICE = 5
 
 RAFHIP_F32 = 0
 RAFHIP_F16 = 1
+RAFHIP_BF16 = 2
 
 RAFHIP_LANS_PHASED = 0
 RAFHIP_LANS_PIPELINED = 1
@@ -80,6 +81,9 @@ OPTIM_SYMBOLS = {
     "rafhip_lans_step": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
                                  POINTER(c_void_p), c_void_p, c_int32, POINTER(LansHParams),
                                  c_void_p, c_int64, c_void_p]),
+    "rafhip_lans_step_mixed": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
+                                       POINTER(c_void_p), POINTER(c_void_p), c_int32, c_void_p, c_int32,
+                                       POINTER(LansHParams), c_void_p, c_int64, c_void_p]),
     "rafhip_lans_read_norms": (c_int, [c_void_p, c_void_p, POINTER(c_double), c_void_p]),
     "rafhip_lans_debug_trace": (c_int, [c_void_p, POINTER(ctypes.c_uint64), c_int64, POINTER(c_int64)]),
     "rafhip_lans_timing_enable": (c_int, [c_void_p, c_int32]),
@@ -109,6 +113,9 @@ DIALECT_SYMBOLS = {
                                     c_double, c_double, POINTER(c_void_p)]),
     "rafhip_raf_sgd_execute": (c_int, [c_void_p] + [POINTER(TensorDesc)] * 5 + [c_void_p]),
     "rafhip_raf_lans_make": (c_int, [c_int32, POINTER(TensorDesc), POINTER(TensorDesc), c_float,
+                                     c_float, c_float, c_float, c_int32, c_float, c_int32, c_int32,
+                                     c_int32, POINTER(c_void_p)]),
+    "rafhip_raf_lans_mixed_make": (c_int, [c_int32, POINTER(TensorDesc), POINTER(TensorDesc), c_float,
                                      c_float, c_float, c_float, c_int32, c_float, c_int32, c_int32,
                                      c_int32, POINTER(c_void_p)]),
     "rafhip_raf_lans_execute": (c_int, [c_void_p, c_int32, POINTER(TensorDesc),

@@ -155,11 +155,11 @@ int rafhip_raf_sgd_execute(rafhip_raf_env* env, const rafhip_tensor_desc* x,
   });
 }
 
-int rafhip_raf_lans_make(int32_t list_len, const rafhip_tensor_desc* tensor_list,
-                         const rafhip_tensor_desc* step, float learning_rate, float beta1,
-                         float beta2, float eps, int32_t bias_correction, float weight_decay,
-                         int32_t grad_averaging, int32_t mode, int32_t normalize_grad,
-                         rafhip_raf_env** env_out) {
+namespace {
+int LansMake(const char* op_name, int32_t list_len, const rafhip_tensor_desc* tensor_list,
+             const rafhip_tensor_desc* step, float learning_rate, float beta1, float beta2,
+             float eps, int32_t bias_correction, float weight_decay, int32_t grad_averaging,
+             int32_t mode, int32_t normalize_grad, rafhip_raf_env** env_out) {
   return Guard([&] {
     if (!env_out) throw Error("rafhip_raf_lans_make: env_out is NULL");
     *env_out = nullptr;
@@ -178,8 +178,27 @@ int rafhip_raf_lans_make(int32_t list_len, const rafhip_tensor_desc* tensor_list
     args->grad_averaging = grad_averaging;
     args->mode = mode;
     args->normalize_grad = normalize_grad != 0;
-    *env_out = Finish(MakeCall("raf.op.lans", args));
+    *env_out = Finish(MakeCall(op_name, args));
   });
+}
+}  // namespace
+
+int rafhip_raf_lans_make(int32_t list_len, const rafhip_tensor_desc* tensor_list,
+                         const rafhip_tensor_desc* step, float learning_rate, float beta1,
+                         float beta2, float eps, int32_t bias_correction, float weight_decay,
+                         int32_t grad_averaging, int32_t mode, int32_t normalize_grad,
+                         rafhip_raf_env** env_out) {
+  return LansMake("raf.op.lans", list_len, tensor_list, step, learning_rate, beta1, beta2, eps,
+                  bias_correction, weight_decay, grad_averaging, mode, normalize_grad, env_out);
+}
+
+int rafhip_raf_lans_mixed_make(int32_t list_len, const rafhip_tensor_desc* tensor_list,
+                               const rafhip_tensor_desc* step, float learning_rate, float beta1,
+                               float beta2, float eps, int32_t bias_correction, float weight_decay,
+                               int32_t grad_averaging, int32_t mode, int32_t normalize_grad,
+                               rafhip_raf_env** env_out) {
+  return LansMake("raf.op.lans_mixed", list_len, tensor_list, step, learning_rate, beta1, beta2,
+                  eps, bias_correction, weight_decay, grad_averaging, mode, normalize_grad, env_out);
 }
 
 int rafhip_raf_lans_execute(rafhip_raf_env* env, int32_t list_len,

@@ -39,6 +39,10 @@ std::string KernelError(const char* what, int status) {
 
 bool IsF32(const DType& t) { return t.code == kDLFloat && t.bits == 32; }
 bool IsF16(const DType& t) { return t.code == kDLFloat && t.bits == 16; }
+bool IsBF16(const DType& t) { return t.code == kDLBfloat && t.bits == 16; }
+int32_t KernelDType(const DType& t) {
+  return IsF32(t) ? RAFHIP_F32 : IsF16(t) ? RAFHIP_F16 : IsBF16(t) ? RAFHIP_BF16 : -1;
+}
 
 }  // namespace
 
@@ -103,12 +107,20 @@ class SgdHipEnv : public OpEnv {
 };
 
 // ---------------------------------------------------------------------------------------- LANS
+// One class serves raf.op.lans (tensor_list = g, w, m, v blocks) and the extension op
+// raf.op.lans_mixed (a fifth block p: the model's float16 / bfloat16 parameters, which receive the
+// new weights narrowed to 16 bits -- what the reference's traced optimizer does with a cast and a
+// copy after the op, python/raf/optim/lans.py:289-291, :303-305).  Half gradients are accepted by
+// both and widened in the kernel, replacing the group_cast in front of the op (lans.py:261-265).
 class LansHipEnv : public OpEnv {
  public:
-  explicit LansHipEnv(const CallValues& cv) {
+  LansHipEnv(const CallValues& cv, bool mixed)
+      : blocks_(mixed ? 5 : 4),
+        op_(mixed ? "raf.op.hip.lans_mixed" : "raf.op.hip.lans"),
+        name_(TruncateName(GetUniqueName(op_))) {
     const auto* args = cv->args_as<schema::LansArgs>();
     if (!args) {
-      error_msgs.push_back("raf.op.hip.lans: call does not carry LansArgs");
+      error_msgs.push_back(op_ + ": call does not carry LansArgs");
       return;
     }
     arg_indices = {args->FieldIndex("tensor_list"), args->FieldIndex("step")};  // lans.cc:32-35
@@ -125,37 +137,48 @@ class LansHipEnv : public OpEnv {
     hp_.grad_unscale = GetLansGradUnscale();
 
     const size_t total = args->tensor_list.size();
-    if (total % 4 != 0) {  // lans.cc:53
-      error_msgs.push_back("raf.op.hip.lans: tensor_list must hold 4n tensors");
+    if (total % (size_t)blocks_ != 0) {  // lans.cc:53
+      error_msgs.push_back(op_ + ": tensor_list must hold " + std::to_string(blocks_) + "n tensors");
       return;
     }
-    n_ = (int32_t)(total / 4);
+    n_ = (int32_t)(total / (size_t)blocks_);
     if (cv->device.device_type() != DevType::kROCM())
-      error_msgs.push_back("raf.op.hip.lans: device is not rocm");
+      error_msgs.push_back(op_ + ": device is not rocm");
     if (hp_.mode != 0 && hp_.mode != 1)
-      error_msgs.push_back("raf.op.hip.lans: mode must be 0 (L2) or 1 (decoupled weight decay)");
+      error_msgs.push_back(op_ + ": mode must be 0 (L2) or 1 (decoupled weight decay)");
     int32_t grad_dtype = RAFHIP_F32;
     std::vector<int64_t> numels;
     for (int32_t i = 0; i < n_; ++i) {
       const TensorView& g = args->tensor_list[i]->tensor;
-      const int32_t gd = IsF32(g.dtype) ? RAFHIP_F32 : IsF16(g.dtype) ? RAFHIP_F16 : -1;
+      const int32_t gd = KernelDType(g.dtype);
       if (gd < 0 || (i > 0 && gd != grad_dtype)) {
-        error_msgs.push_back("raf.op.hip.lans: gradients must all be float32 or all float16");
+        error_msgs.push_back(op_ + ": gradients must all be float32, all float16 or all bfloat16");
         break;
       }
       grad_dtype = gd;
       numels.push_back(g.numel());
       for (int q = 1; q < 4; ++q) {  // w, m, v: fp32 (lans.cc:37-40) and as large as g
         const TensorView& t = args->tensor_list[q * n_ + i]->tensor;
-        if (!IsF32(t.dtype)) error_msgs.push_back("raf.op.hip.lans: LANS only takes FP32 weights and state");
+        if (!IsF32(t.dtype)) error_msgs.push_back(op_ + ": LANS only takes FP32 weights and state");
         if (t.numel() != g.numel())
-          error_msgs.push_back("raf.op.hip.lans: g, w, m, v of one parameter differ in size");
+          error_msgs.push_back(op_ + ": g, w, m, v of one parameter differ in size");
+      }
+      if (blocks_ == 5) {  // p: 16-bit, one dtype for the whole list, as large as g
+        const TensorView& t = args->tensor_list[4 * n_ + i]->tensor;
+        const int32_t pd = KernelDType(t.dtype);
+        if (pd != RAFHIP_F16 && pd != RAFHIP_BF16)
+          error_msgs.push_back(op_ + ": model parameters must be float16 or bfloat16");
+        else if (i > 0 && pd != copy_dtype_)
+          error_msgs.push_back(op_ + ": model parameters must share one dtype");
+        copy_dtype_ = pd;
+        if (t.numel() != g.numel())
+          error_msgs.push_back(op_ + ": model parameter and gradient differ in size");
       }
       if (!error_msgs.empty()) break;
     }
     if (!error_msgs.empty()) return;
     if (rafhip_device_count() <= 0) {
-      error_msgs.push_back("raf.op.hip.lans: no HIP device is visible");
+      error_msgs.push_back(op_ + ": no HIP device is visible");
       return;
     }
     int st = rafhip_lans_plan_create(n_, numels.data(), grad_dtype, &plan_);
@@ -184,8 +207,8 @@ class LansHipEnv : public OpEnv {
     (void)output;  // aliases the inputs (declare/optimizer.cc:53-57); the update is in place
     RAF_CHECK(inputs.size() == 2, "raf.op.hip.lans takes (tensor_list, step)");
     auto tuple = AsTuple(inputs[0]);
-    RAF_CHECK((int64_t)tuple->fields.size() == 4 * (int64_t)n_,
-              "raf.op.hip.lans: tensor_list length changed since the OpEnv was made");
+    RAF_CHECK((int64_t)tuple->fields.size() == (int64_t)blocks_ * (int64_t)n_,
+              op_ + ": tensor_list length changed since the OpEnv was made");
     const TensorView& step = AsTensor(inputs[1])->tensor;
     RAF_CHECK(step.ndim() == 0, "step must be a 0-d tensor");  // lans.cc:96
     RAF_CHECK(IsF32(step.dtype), "step must be float32");
@@ -195,30 +218,37 @@ class LansHipEnv : public OpEnv {
     for (size_t i = 0; i < ptrs.size(); ++i) ptrs[i] = AsTensor(tuple->fields[i])->tensor.data;
     void** p = ptrs.data();
     void* stream = DeviceAPI::Get(DevType::kROCM())->GetStream();
-    int st = rafhip_lans_step(plan_, reinterpret_cast<const void* const*>(p),
-                              reinterpret_cast<float* const*>(p + n_),
-                              reinterpret_cast<float* const*>(p + 2 * n_),
-                              reinterpret_cast<float* const*>(p + 3 * n_),
-                              static_cast<const float*>(step.data), 0, &hp_, workspace_,
-                              workspace_bytes_, stream);
-    if (st != RAFHIP_OK) throw Error(KernelError("rafhip_lans_step", st));
+    int st = rafhip_lans_step_mixed(plan_, reinterpret_cast<const void* const*>(p),
+                                    reinterpret_cast<float* const*>(p + n_),
+                                    reinterpret_cast<float* const*>(p + 2 * n_),
+                                    reinterpret_cast<float* const*>(p + 3 * n_),
+                                    blocks_ == 5 ? p + 4 * n_ : nullptr, copy_dtype_,
+                                    static_cast<const float*>(step.data), 0, &hp_, workspace_,
+                                    workspace_bytes_, stream);
+    if (st != RAFHIP_OK) throw Error(KernelError("rafhip_lans_step_mixed", st));
   }
 
-  static OpEnv* make(const CallValues& cv) { return new LansHipEnv(cv); }
+  static OpEnv* make(const CallValues& cv) { return new LansHipEnv(cv, false); }
+  static OpEnv* make_mixed(const CallValues& cv) { return new LansHipEnv(cv, true); }
 
  private:
+  int blocks_;  // 4: g, w, m, v; 5: and the 16-bit model parameters
+  std::string op_;
+  std::string name_;
   rafhip_lans_hparams hp_{};
   int32_t n_ = 0;
+  int32_t copy_dtype_ = RAFHIP_F16;
   rafhip_lans_plan* plan_ = nullptr;
   void* workspace_ = nullptr;  // bound by the executor around each Execute
   int64_t workspace_bytes_ = 0;
-  std::string name_ = TruncateName(GetUniqueName("raf.op.hip.lans"));
 };
 
 RAF_REGISTER_DIALECT("hip").set_enable(DevType::kROCM());
 // plevels above the reference's own backends (cuda lans = 20, tvm sgd = 10).
 RAF_REGISTER_DIALECT_OP(hip, lans, 30);
 RAF_OP_ENV_MAKER("raf.op.hip.lans", LansHipEnv::make);
+RAF_REGISTER_DIALECT_OP(hip, lans_mixed, 30);
+RAF_OP_ENV_MAKER("raf.op.hip.lans_mixed", LansHipEnv::make_mixed);
 RAF_REGISTER_DIALECT_OP(hip, sgd, 30);
 RAF_OP_ENV_MAKER("raf.op.hip.sgd", SgdHipEnv::make);
 

@@ -66,8 +66,9 @@ struct Device {
   int device_id() const { return device_id_; }
 };
 
-// DLPack-style dtype codes (kDLInt = 0, kDLUInt = 1, kDLFloat = 2).
+// DLPack-style dtype codes (kDLInt = 0, kDLUInt = 1, kDLFloat = 2, kDLBfloat = 4).
 constexpr int kDLFloat = 2;
+constexpr int kDLBfloat = 4;
 struct DType {
   int code = kDLFloat;
   int bits = 32;

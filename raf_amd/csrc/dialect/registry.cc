@@ -134,6 +134,22 @@ void LansDecl(const CallValues& call) {
   call->out = value::MakeTuple(std::move(out));
 }
 
+// Extension op raf.op.lans_mixed: LansArgs with a fifth block of tensors, the model's 16-bit
+// parameters, that receive the narrowed new weights; declared like raf.op.lans (output = inputs).
+void LansMixedDecl(const CallValues& call) {
+  const auto* args = call->args_as<schema::LansArgs>();
+  RAF_CHECK(args != nullptr, "raf.op.lans_mixed expects LansArgs");
+  RAF_CHECK(args->tensor_list.size() % 5 == 0,
+            "tensor_list must hold 5n tensors (g, w, m, v, p)");
+  std::vector<value::Value> out;
+  for (const auto& t : args->tensor_list) {
+    RAF_CHECK(t != nullptr, "tensor_list holds a null tensor");
+    out.push_back(t);
+  }
+  if (!args->tensor_list.empty()) call->device = args->tensor_list[0]->tensor.device;
+  call->out = value::MakeTuple(std::move(out));
+}
+
 }  // namespace
 
 void RunDeclare(const CallValues& call) {
@@ -141,6 +157,7 @@ void RunDeclare(const CallValues& call) {
   if (IsDialectOp(op)) op = GetBaseOp(op);
   if (op == "raf.op.sgd") return SgdDecl(call);
   if (op == "raf.op.lans") return LansDecl(call);
+  if (op == "raf.op.lans_mixed") return LansMixedDecl(call);
   throw Error("no declare function registered for op " + op);
 }
 

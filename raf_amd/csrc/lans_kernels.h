@@ -32,7 +32,12 @@
 // Results are bit-identical from run to run, across grid sizes and across the two schedules.
 // Atomics are used for tickets, counters and flags only, never to accumulate values.
 //
-// Arithmetic.  Loads and stores are fp32 (fp16 for the optional half gradients); every
+// Mixed precision.  Gradients may arrive as binary16 or bfloat16 (widened exactly on load, which
+// replaces the reference's group_cast, python/raf/optim/lans.py:261-265), and pass C can write,
+// next to the fp32 weight, its round-to-nearest-even 16-bit copy (replacing the cast + copy into
+// the model's parameter, lans.py:289-291, :303-305).
+//
+// Arithmetic.  Loads and stores are fp32 (16-bit for the optional half gradients); every
 // per-element operation and every accumulation is float64, rounded once on store.  The weight
 // update subtracts a ~1e-5-sized step from the weight, so an fp32 evaluation of the step (or of the
 // norms behind the trust ratio) would leave errors far above 1e-5 *relative* on the weights that
@@ -53,14 +58,16 @@ constexpr int kChunksPerA = 8;   // pass A reads 2-4 bytes per element, so its u
 constexpr int kUnroll = 2;       // 4-element groups in flight per lane per trip
 constexpr int kPartialSlots = 4; // doubles per chunk: [0] sum g^2 | [1] sum u_m^2 [2] sum u_g^2 [3] sum w^2
 
-struct TensorRec {  // 48 bytes, one per tensor
+struct TensorRec {  // 64 bytes, one per tensor
   const void* g;
   float* w;
   float* m;
   float* v;
+  void* p;  // optional 16-bit copy of the new weight (the model's half-precision parameter) or null
   int64_t numel;
   int32_t first_chunk;
-  int32_t vec_ok;  // 1: every base pointer is 16-byte aligned: 128-bit lane accesses
+  int32_t vec_ok;  // 1: every base pointer is aligned for 4-element lane accesses
+  int64_t reserved;
 };
 
 // One unit of work: kind in the top three bits of `chunk_phase`, chunk number within the tensor
@@ -122,6 +129,7 @@ struct LansDeviceArgs {
   uint32_t n_items;       // pipelined work-list length
   const WorkItem* pipeline_items;
   float unscale;
+  int32_t p_is_bf16;      // dtype of the optional 16-bit weight copies: 0 binary16, 1 bfloat16
   StepScalars* scalars;
   TensorStats* stats;
   double* partials;       // kPartialSlots doubles per chunk

@@ -22,6 +22,18 @@ typedef RAFHIP_GLOBAL const half4_t gc_half4;
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef RAFHIP_GLOBAL const half8_t gc_half8;
 typedef RAFHIP_GLOBAL const _Float16 gc_half;
+typedef unsigned short u16x4 __attribute__((ext_vector_type(4)));
+typedef unsigned short u16x8 __attribute__((ext_vector_type(8)));
+typedef RAFHIP_GLOBAL const u16x4 gc_u16x4;
+typedef RAFHIP_GLOBAL const u16x8 gc_u16x8;
+typedef RAFHIP_GLOBAL u16x4 g_u16x4;
+typedef RAFHIP_GLOBAL const unsigned short gc_u16;
+typedef RAFHIP_GLOBAL unsigned short g_u16;
+
+// Gradient element type tag for bfloat16 (two bytes, like the data).
+struct Bf16 {
+  unsigned short bits;
+};
 
 // ------------------------------------------------------------------ cache policy
 // Every pass streams far more data than the 256 MB Infinity Cache holds.  Loads and stores that
@@ -104,6 +116,43 @@ struct GradIO<_Float16> {
     return (float)((gc_half*)g)[i] * us;
   }
 };
+
+template <>
+struct GradIO<Bf16> {
+  static constexpr int kWide = 8;
+  // bfloat16 is the upper half of the fp32 word: widening is a shift.
+  static __device__ __forceinline__ float widen(unsigned short b) {
+    return __uint_as_float((unsigned)b << 16);
+  }
+  template <bool kNT>
+  static __device__ __forceinline__ void load_wide(const void* g, int iw, float us,
+                                                   float (&out)[kWide]) {
+    const u16x8 r = ldg<kNT>((gc_u16x8*)g + iw);
+#pragma unroll
+    for (int j = 0; j < kWide; ++j) out[j] = widen(r[j]) * us;
+  }
+  template <bool kNT>
+  static __device__ __forceinline__ f32x4 load4(const void* g, int i4, float us) {
+    const u16x4 r = ldg<kNT>((gc_u16x4*)g + i4);
+    return f32x4{widen(r.x) * us, widen(r.y) * us, widen(r.z) * us, widen(r.w) * us};
+  }
+  static __device__ __forceinline__ float load1(const void* g, int i, float us) {
+    return widen(((gc_u16*)g)[i]) * us;
+  }
+};
+
+// ------------------------------------------------------------------ 16-bit weight copy
+// The stored fp32 weight narrowed with round to nearest even: binary16 by the hardware conversion,
+// bfloat16 by add-and-shift on the bit pattern (NaN stays a quiet NaN).
+__device__ __forceinline__ unsigned short narrow16(float x, bool bf16) {
+  if (bf16) {
+    const unsigned u = __float_as_uint(x);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x0040u);
+    return (unsigned short)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+  }
+  const _Float16 h = (_Float16)x;
+  return __builtin_bit_cast(unsigned short, h);
+}
 
 // ------------------------------------------------------------------ reductions
 // Sum over the 64 lanes of a wavefront; the total is valid in lane 0.  Fixed butterfly order.
@@ -269,7 +318,8 @@ struct ChunkView {
   float* w;
   float* m;
   float* v;
-  int len;  // elements in this chunk
+  unsigned short* p;  // 16-bit weight copy or null
+  int len;            // elements in this chunk
   int vec_ok;
 };
 
@@ -283,6 +333,7 @@ __device__ __forceinline__ ChunkView chunk_view(const TensorRec& tr, uint32_t ch
   cv.w = tr.w + base;
   cv.m = tr.m + base;
   cv.v = tr.v + base;
+  cv.p = tr.p ? static_cast<unsigned short*>(tr.p) + base : nullptr;
   cv.len = rest < unit ? (int)rest : unit;
   cv.vec_ok = tr.vec_ok;
   return cv;
@@ -429,7 +480,7 @@ __device__ __forceinline__ Applied apply_one(double g, double w, double m, doubl
 
 // `get_params` supplies the tensor's divisor and trust ratios.
 template <typename G, bool kGradNT, bool kNT, bool kStoreNT, typename GetParams>
-__device__ __forceinline__ void chunk_apply(const ChunkView& cv, float unscale,
+__device__ __forceinline__ void chunk_apply(const ChunkView& cv, float unscale, bool p_is_bf16,
                                             const StepScalars& k, GetParams&& get_params) {
   if (cv.vec_ok) {
     const int n4 = cv.len >> 2;
@@ -449,6 +500,10 @@ __device__ __forceinline__ void chunk_apply(const ChunkView& cv, float unscale,
           stg<kStoreNT>((g_float4*)cv.w + i, f32x4{a0.w, a1.w, a2.w, a3.w});
           stg<kStoreNT>((g_float4*)cv.m + i, f32x4{a0.m, a1.m, a2.m, a3.m});
           stg<kStoreNT>((g_float4*)cv.v + i, f32x4{a0.v, a1.v, a2.v, a3.v});
+          if (cv.p)  // uniform over the workgroup
+            stg<kStoreNT>((g_u16x4*)cv.p + i,
+                          u16x4{narrow16(a0.w, p_is_bf16), narrow16(a1.w, p_is_bf16),
+                                narrow16(a2.w, p_is_bf16), narrow16(a3.w, p_is_bf16)});
         }
       }
     }
@@ -459,6 +514,7 @@ __device__ __forceinline__ void chunk_apply(const ChunkView& cv, float unscale,
       ((g_float*)cv.w)[tail] = o.w;
       ((g_float*)cv.m)[tail] = o.m;
       ((g_float*)cv.v)[tail] = o.v;
+      if (cv.p) ((g_u16*)cv.p)[tail] = narrow16(o.w, p_is_bf16);
     }
   } else {
     const ApplyParams p = get_params();
@@ -468,6 +524,7 @@ __device__ __forceinline__ void chunk_apply(const ChunkView& cv, float unscale,
       ((g_float*)cv.w)[i] = o.w;
       ((g_float*)cv.m)[i] = o.m;
       ((g_float*)cv.v)[i] = o.v;
+      if (cv.p) ((g_u16*)cv.p)[i] = narrow16(o.w, p_is_bf16);
     }
   }
 }
@@ -618,7 +675,7 @@ __global__ __launch_bounds__(kLansBlock) void lans_apply(LansDeviceArgs a) {
     const ChunkView cv = chunk_view(tr, it.chunk_phase & kChunkMask, (int)sizeof(G));
     const TensorStats st = a.stats[it.tensor];
     const ApplyParams p{st.inv_grad_div, st.ratio_m, st.ratio_g};
-    chunk_apply<G, kP.c_g, kP.c_wmv, kP.c_stores>(cv, a.unscale, k, [&] { return p; });
+    chunk_apply<G, kP.c_g, kP.c_wmv, kP.c_stores>(cv, a.unscale, a.p_is_bf16 != 0, k, [&] { return p; });
   }
 }
 
@@ -696,7 +753,8 @@ __global__ __launch_bounds__(kLansBlock) void lans_pipelined(LansDeviceArgs a) {
       tensor_totals<3, true>(tensor_part, 1, n_chunks, 1, tot, red, a.sync);
       if (threadIdx.x == 0) stats_after_b(st, tot, k, r0, r1);
     } else if (phase == kPhaseC) {
-      chunk_apply<G, kPipelinedPolicy.c_g, kPipelinedPolicy.c_wmv, kPipelinedPolicy.c_stores>(cv, a.unscale, k, [&] {
+      chunk_apply<G, kPipelinedPolicy.c_g, kPipelinedPolicy.c_wmv, kPipelinedPolicy.c_stores>(
+          cv, a.unscale, a.p_is_bf16 != 0, k, [&] {
         const double* const words[3] = {&st->inv_grad_div, &st->ratio_m, &st->ratio_g};
         double val[3];
         wait_published_n<3>(words, val, a.sync);
@@ -717,7 +775,7 @@ __global__ __launch_bounds__(kLansBlock) void lans_pipelined(LansDeviceArgs a) {
       if (threadIdx.x == 0) stats_after_b(st, s3, k, s_bcast[1], s_bcast[2]);
       __syncthreads();
       const ApplyParams p{inv_gdiv, s_bcast[1], s_bcast[2]};
-      chunk_apply<G, false, false, true>(cv, a.unscale, k, [&] { return p; });
+      chunk_apply<G, false, false, true>(cv, a.unscale, a.p_is_bf16 != 0, k, [&] { return p; });
     }
     if (a.trace && threadIdx.x == 0) {  // diagnostics: when the item was started and finished
       uint64_t* rec = a.trace + 4 * (uint64_t)ticket;
@@ -769,33 +827,39 @@ void launch_phased_t(hipStream_t s, const LansDeviceArgs& a, hipEvent_t* marks) 
 
 void launch_phased(int grad_dtype, bool streaming, hipStream_t s, const LansDeviceArgs& a,
                    hipEvent_t* marks) {
-  if (grad_dtype == RAFHIP_F16) {
+  auto go = [&](auto tag) {
+    using G = decltype(tag);
     if (streaming)
-      launch_phased_t<_Float16, true>(s, a, marks);
+      launch_phased_t<G, true>(s, a, marks);
     else
-      launch_phased_t<_Float16, false>(s, a, marks);
-  } else {
-    if (streaming)
-      launch_phased_t<float, true>(s, a, marks);
-    else
-      launch_phased_t<float, false>(s, a, marks);
-  }
+      launch_phased_t<G, false>(s, a, marks);
+  };
+  if (grad_dtype == RAFHIP_F16)
+    go(_Float16{});
+  else if (grad_dtype == RAFHIP_BF16)
+    go(Bf16{});
+  else
+    go(float{});
 }
 
 void launch_pipelined(int grad_dtype, unsigned grid, hipStream_t s, const LansDeviceArgs& a) {
   if (grad_dtype == RAFHIP_F16)
     hipLaunchKernelGGL(lans_pipelined<_Float16>, dim3(grid), dim3(kLansBlock), 0, s, a);
+  else if (grad_dtype == RAFHIP_BF16)
+    hipLaunchKernelGGL(lans_pipelined<Bf16>, dim3(grid), dim3(kLansBlock), 0, s, a);
   else
     hipLaunchKernelGGL(lans_pipelined<float>, dim3(grid), dim3(kLansBlock), 0, s, a);
 }
 
 int pipelined_blocks_per_cu(int grad_dtype) {
   int n = 0;
-  hipError_t e = grad_dtype == RAFHIP_F16
-                     ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, lans_pipelined<_Float16>,
-                                                                    kLansBlock, 0)
-                     : hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, lans_pipelined<float>,
-                                                                    kLansBlock, 0);
+  hipError_t e;
+  if (grad_dtype == RAFHIP_F16)
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, lans_pipelined<_Float16>, kLansBlock, 0);
+  else if (grad_dtype == RAFHIP_BF16)
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, lans_pipelined<Bf16>, kLansBlock, 0);
+  else
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, lans_pipelined<float>, kLansBlock, 0);
   if (e != hipSuccess) {
     (void)hipGetLastError();
     return 0;

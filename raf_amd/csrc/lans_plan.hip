@@ -248,10 +248,10 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
   if (!out_plan) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_plan_create: out_plan is NULL");
   *out_plan = nullptr;
   if (int st = validate_list("rafhip_lans_plan_create", n_tensors, numel)) return st;
-  if (grad_dtype != RAFHIP_F32 && grad_dtype != RAFHIP_F16)
+  if (grad_dtype != RAFHIP_F32 && grad_dtype != RAFHIP_F16 && grad_dtype != RAFHIP_BF16)
     return fail(RAFHIP_ERR_UNSUPPORTED,
                 "rafhip_lans_plan_create: gradient dtype %d (LANS takes fp32 weights and state; "
-                "gradients may be fp32 or fp16)",
+                "gradients may be fp32, fp16 or bf16)",
                 grad_dtype);
 
   rafhip_lans_plan* p = new (std::nothrow) rafhip_lans_plan();
@@ -379,8 +379,20 @@ int rafhip_lans_step(rafhip_lans_plan* plan, const void* const* g, float* const*
                      float* const* m, float* const* v, const float* step_dev, int32_t step_host,
                      const rafhip_lans_hparams* hp, void* workspace, int64_t workspace_bytes,
                      void* stream) {
+  return rafhip_lans_step_mixed(plan, g, w, m, v, nullptr, RAFHIP_F16, step_dev, step_host, hp,
+                                workspace, workspace_bytes, stream);
+}
+
+int rafhip_lans_step_mixed(rafhip_lans_plan* plan, const void* const* g, float* const* w,
+                           float* const* m, float* const* v, void* const* p, int32_t p_dtype,
+                           const float* step_dev, int32_t step_host,
+                           const rafhip_lans_hparams* hp, void* workspace,
+                           int64_t workspace_bytes, void* stream) {
   clear_error();
   if (!plan) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_step: plan is NULL");
+  if (p && p_dtype != RAFHIP_F16 && p_dtype != RAFHIP_BF16)
+    return fail(RAFHIP_ERR_UNSUPPORTED,
+                "rafhip_lans_step: weight-copy dtype %d (binary16 or bfloat16)", p_dtype);
   if (!hp) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_step: hparams is NULL");
   if (hp->mode != 0 && hp->mode != 1)
     return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_step: mode = %d (0 = L2, 1 = decoupled)",
@@ -398,7 +410,7 @@ int rafhip_lans_step(rafhip_lans_plan* plan, const void* const* g, float* const*
 
   // Build this call's tensor table; 4-byte (fp16 g: 2-byte) alignment is the hard requirement,
   // 16-byte alignment of all four selects the vector path.
-  const uintptr_t g_elem = plan->grad_dtype == RAFHIP_F16 ? 2 : 4;
+  const uintptr_t g_elem = plan->grad_dtype == RAFHIP_F32 ? 4 : 2;
   const uintptr_t g_vec = 16;  // pass A reads the gradient with 16-byte lane accesses
   std::vector<TensorRec> recs((size_t)n);
   for (int32_t t = 0; t < n; ++t) {
@@ -407,17 +419,19 @@ int rafhip_lans_step(rafhip_lans_plan* plan, const void* const* g, float* const*
     r.w = w[t];
     r.m = m[t];
     r.v = v[t];
+    r.p = p ? p[t] : nullptr;
     r.numel = plan->numel[t];
     r.first_chunk = plan->first_chunk[t];
     r.vec_ok = 0;
+    r.reserved = 0;
     if (r.numel == 0) continue;
     if (!r.g || !r.w || !r.m || !r.v)
       return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_step: tensor %d has a null data pointer", t);
     if (!aligned_to(r.g, g_elem) || !aligned_to(r.w, 4) || !aligned_to(r.m, 4) ||
-        !aligned_to(r.v, 4))
+        !aligned_to(r.v, 4) || !aligned_to(r.p, 2))
       return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_step: tensor %d is not element-aligned", t);
     r.vec_ok = aligned_to(r.g, g_vec) && aligned_to(r.w, 16) && aligned_to(r.m, 16) &&
-               aligned_to(r.v, 16);
+               aligned_to(r.v, 16) && aligned_to(r.p, 8);
   }
 
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -445,6 +459,7 @@ int rafhip_lans_step(rafhip_lans_plan* plan, const void* const* g, float* const*
   a.n_items = plan->n_pipeline_items;
   a.pipeline_items = plan->d_pipeline;
   a.unscale = hp->grad_unscale;
+  a.p_is_bf16 = p_dtype == RAFHIP_BF16 ? 1 : 0;
   a.scalars = reinterpret_cast<StepScalars*>(ws + plan->ws.scalars_off);
   a.stats = reinterpret_cast<TensorStats*>(ws + plan->ws.stats_off);
   a.partials = reinterpret_cast<double*>(ws + plan->ws.partials_off);
@@ -475,7 +490,7 @@ int rafhip_lans_step(rafhip_lans_plan* plan, const void* const* g, float* const*
       for (int i = 2; i < 6; ++i) RAFHIP_HIP_TRY(hipEventRecord(marks[i], s));
   } else {
     launch_prepare(s, a, step_dev, step_host, pod);
-    const int64_t bytes_per_elt = plan->grad_dtype == RAFHIP_F16 ? 14 : 16;
+    const int64_t bytes_per_elt = plan->grad_dtype == RAFHIP_F32 ? 16 : 14;
     launch_phased(plan->grad_dtype, plan->total_elements * bytes_per_elt > kResidentBytes, s, a,
                   marks);
   }

@@ -12,7 +12,7 @@ from typing import List, Optional, Sequence
 import torch
 
 from . import _lib
-from ._lib import LansHParams, RAFHIP_F16, RAFHIP_F32, check
+from ._lib import LansHParams, RAFHIP_BF16, RAFHIP_F16, RAFHIP_F32, check
 
 
 def _current_stream(device) -> int:
@@ -73,6 +73,9 @@ def pipeline_order(numels: Sequence[int], group_elements: int = 0):
     return [(buf[3 * i], buf[3 * i + 1], buf[3 * i + 2]) for i in range(count.value)]
 
 
+_DTYPE_CODE = {torch.float32: RAFHIP_F32, torch.float16: RAFHIP_F16, torch.bfloat16: RAFHIP_BF16}
+
+
 class LansPlan:
     """Owns a ``rafhip_lans_plan`` and a workspace tensor sized for it."""
 
@@ -82,12 +85,9 @@ class LansPlan:
         self.device = torch.device(device)
         self.numels = [int(n) for n in numels]
         self.n = len(self.numels)
-        if grad_dtype == torch.float32:
-            code = RAFHIP_F32
-        elif grad_dtype == torch.float16:
-            code = RAFHIP_F16
-        else:
-            raise TypeError(f"LANS gradients must be float32 or float16, got {grad_dtype}")
+        if grad_dtype not in _DTYPE_CODE:
+            raise TypeError(f"LANS gradients must be float32, float16 or bfloat16, got {grad_dtype}")
+        code = _DTYPE_CODE[grad_dtype]
         self.grad_dtype = grad_dtype
         arr = (c_int64 * max(self.n, 1))(*self.numels)
         with torch.cuda.device(self.device):
@@ -131,11 +131,32 @@ class LansPlan:
             arr[i] = t.data_ptr()
         return arr
 
+    def _model_ptrs(self, p):
+        """Pointer list and dtype code of the optional 16-bit weight copies."""
+        if p is None:
+            return None, RAFHIP_F16
+        dt = next((t.dtype for t in p if t is not None), torch.float16)
+        if dt not in (torch.float16, torch.bfloat16):
+            raise TypeError(f"16-bit weight copies must be float16 or bfloat16, got {dt}")
+        if len(p) != self.n:
+            raise ValueError(f"p: expected {self.n} tensors, got {len(p)}")
+        arr = (c_void_p * max(self.n, 1))()
+        for i, t in enumerate(p):
+            if t is None:
+                continue
+            if not t.is_cuda or t.dtype != dt or not t.is_contiguous() or t.numel() != self.numels[i]:
+                raise TypeError(f"p[{i}]: need a contiguous {dt} GPU tensor of {self.numels[i]} elements")
+            arr[i] = t.data_ptr()
+        return arr, _DTYPE_CODE[dt]
+
     def step(self, g: Sequence[torch.Tensor], w: Sequence[torch.Tensor],
              m: Sequence[torch.Tensor], v: Sequence[torch.Tensor], step, hp: LansHParams,
-             workspace: Optional[torch.Tensor] = None):
-        """``step`` is a 0-d fp32 GPU tensor (read on the device) or a Python int."""
+             workspace: Optional[torch.Tensor] = None, p: Optional[Sequence] = None):
+        """``step`` is a 0-d fp32 GPU tensor (read on the device) or a Python int.  ``p``: optional
+        float16 / bfloat16 tensors (entries may be None) that receive the new weights narrowed to
+        16 bits: the half-precision model parameters of a mixed-precision run."""
         ws = self.workspace if workspace is None else workspace
+        pp, p_code = self._model_ptrs(p)
         gp = self._ptrs(g, self.grad_dtype, "g")
         wp = self._ptrs(w, torch.float32, "w")
         mp = self._ptrs(m, torch.float32, "m")
@@ -146,24 +167,25 @@ class LansPlan:
             step_dev, step_host = step.data_ptr(), 0
         else:
             step_dev, step_host = None, int(step)
-        check(self.lib.rafhip_lans_step(self._h, gp, wp, mp, vp, step_dev, step_host,
-                                        ctypes.byref(hp), ws.data_ptr(), ws.numel(),
-                                        _current_stream(self.device)))
+        check(self.lib.rafhip_lans_step_mixed(self._h, gp, wp, mp, vp, pp, p_code, step_dev, step_host,
+                                              ctypes.byref(hp), ws.data_ptr(), ws.numel(),
+                                              _current_stream(self.device)))
 
-    def bind(self, g, w, m, v, hp: LansHParams, workspace: Optional[torch.Tensor] = None):
+    def bind(self, g, w, m, v, hp: LansHParams, workspace: Optional[torch.Tensor] = None, p=None):
         """Marshal the pointer lists once for tensors that stay where they are; ``step_bound`` then
         costs one foreign call per step (a training loop updates the same buffers every step)."""
         ws = self.workspace if workspace is None else workspace
+        pp, p_code = self._model_ptrs(p)
         self._bound = (self._ptrs(g, self.grad_dtype, "g"), self._ptrs(w, torch.float32, "w"),
                        self._ptrs(m, torch.float32, "m"), self._ptrs(v, torch.float32, "v"),
-                       hp, ws, (list(g), list(w), list(m), list(v)))
+                       pp, p_code, hp, ws, (list(g), list(w), list(m), list(v), p))
 
     def step_bound(self, step: torch.Tensor):
         """One step on the tensors given to ``bind``; ``step`` is the 0-d fp32 GPU step tensor."""
-        gp, wp, mp, vp, hp, ws, _ = self._bound
-        check(self.lib.rafhip_lans_step(self._h, gp, wp, mp, vp, step.data_ptr(), 0,
-                                        ctypes.byref(hp), ws.data_ptr(), ws.numel(),
-                                        _current_stream(self.device)))
+        gp, wp, mp, vp, pp, p_code, hp, ws, _ = self._bound
+        check(self.lib.rafhip_lans_step_mixed(self._h, gp, wp, mp, vp, pp, p_code, step.data_ptr(), 0,
+                                              ctypes.byref(hp), ws.data_ptr(), ws.numel(),
+                                              _current_stream(self.device)))
 
     def read_norms(self, workspace: Optional[torch.Tensor] = None):
         """[n, 4] float64: ||g||, ||w||, ||u_m||, ||u_g|| of the last step."""

@@ -98,6 +98,23 @@ def lans(tensor_list: Sequence[torch.Tensor], step: torch.Tensor, learning_rate,
     """``raf._op.imp.lans(...)``: updates the w, m, v quarters of ``tensor_list`` in place and
     returns the list (the op's output aliases its input, declare/optimizer.cc:53-57).  Booleans
     become ints as the schema's ``int`` fields receive them (python/raf/optim/lans.py:51-54)."""
+    return _lans("lans", tensor_list, step, learning_rate, beta1, beta2, eps, bias_correction,
+                 weight_decay, grad_averaging, mode, normalize_grad)
+
+
+def lans_mixed(tensor_list: Sequence[torch.Tensor], step: torch.Tensor, learning_rate, beta1, beta2,
+               eps, bias_correction, weight_decay, grad_averaging, mode, normalize_grad):
+    """Extension op for half-precision models with fp32 master weights: ``tensor_list`` holds five
+    blocks ``[g..., w..., m..., v..., p...]``; ``p`` are the model's float16 / bfloat16 parameters
+    and receive the new weights narrowed to 16 bits.  One call does what the reference's traced
+    optimizer builds from ``group_cast`` + ``lans`` + ``cast`` + ``add(out=p)``
+    (python/raf/optim/lans.py:261-265, :289-291, :303-305)."""
+    return _lans("lans_mixed", tensor_list, step, learning_rate, beta1, beta2, eps, bias_correction,
+                 weight_decay, grad_averaging, mode, normalize_grad)
+
+
+def _lans(op_name, tensor_list, step, learning_rate, beta1, beta2, eps, bias_correction,
+          weight_decay, grad_averaging, mode, normalize_grad):
     lib = _lib.dialect()
     tensor_list = list(tensor_list)
     keep: list = []
@@ -106,11 +123,12 @@ def lans(tensor_list: Sequence[torch.Tensor], step: torch.Tensor, learning_rate,
     dstep = _desc(step, keep)
     hp = (float(learning_rate), float(beta1), float(beta2), float(eps), int(bias_correction),
           float(weight_decay), int(grad_averaging), int(mode), int(bool(normalize_grad)))
-    key = ("lans", tuple(_sig(t) for t in tensor_list), _sig(step), hp, get_lans_grad_unscale())
+    key = (op_name, tuple(_sig(t) for t in tensor_list), _sig(step), hp, get_lans_grad_unscale())
     env = _env_cache.get(key)
     if env is None:
         h = c_void_p(None)
-        check_raf(lib.rafhip_raf_lans_make(n4, descs, dstep, *hp, ctypes.byref(h)))
+        make = lib.rafhip_raf_lans_make if op_name == "lans" else lib.rafhip_raf_lans_mixed_make
+        check_raf(make(n4, descs, dstep, *hp, ctypes.byref(h)))
         env = _env_cache[key] = _Env(h)
     ws = None
     ws_ptr = None

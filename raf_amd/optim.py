@@ -38,7 +38,13 @@ class SGD:
 
 
 class LANS:
-    """LANS (http://arxiv.org/abs/2006.13484): one multi-tensor ``raf.op.lans`` call per step."""
+    """LANS (http://arxiv.org/abs/2006.13484): one multi-tensor ``raf.op.lans`` call per step.
+
+    float16 / bfloat16 parameters are trained the way the reference's traced optimizer trains
+    them (python/raf/optim/lans.py:213-227, :261-305): an fp32 master copy of every weight holds
+    the state, the half gradients feed the op directly and the parameter receives the new master
+    weight narrowed to its dtype -- here in one ``lans_mixed`` call instead of
+    ``group_cast`` + ``lans`` + ``cast`` + ``add(out=p)``."""
 
     def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), eps=1e-6, weight_decay=0.01,
                  bias_correction=True, grad_averaging=True, mode=True, normalize_grad=True):
@@ -53,25 +59,37 @@ class LANS:
         self.normalize_grad = normalize_grad
         self.params = []
         self._step = 1  # lans.py:66
+        params = list(params)
+        halves = {x.dtype for x in params if isinstance(x, torch.Tensor)} & {torch.float16, torch.bfloat16}
+        self.mixed = bool(halves)
+        if self.mixed and (len(halves) > 1 or any(x.dtype not in halves for x in params)):
+            raise TypeError("a half-precision model must use one 16-bit dtype for all parameters")
         for x in params:
             assert isinstance(x, torch.Tensor), "Only tensors can be optimized!"
-            self.params.append((x, torch.zeros_like(x), torch.zeros_like(x)))
+            # the fp32 master weight: the parameter itself, or its widened copy (lans.py:217-219)
+            w = x.data.float() if self.mixed else x.data
+            self.params.append((x, w, torch.zeros_like(w), torch.zeros_like(w)))
 
     def step(self):
         """Update the parameters with gradients."""
-        g_list, x_list, m_list, v_list = [], [], [], []
-        for x, m, v in self.params:
+        g_list, x_list, m_list, v_list, p_list = [], [], [], [], []
+        for x, w, m, v in self.params:
             if x.grad is None:
                 continue
             g_list.append(x.grad)
-            x_list.append(x.data)
+            x_list.append(w)
             m_list.append(m)
             v_list.append(v)
+            p_list.append(x.data)
         if not x_list:
             self._step += 1
             return
         step = torch.tensor(float(self._step), dtype=torch.float32, device=x_list[0].device)
         tensor_list = g_list + x_list + m_list + v_list  # lans.py:89
-        _op.lans(tensor_list, step, self.lr, self.beta1, self.beta2, self.eps, self.bias_correction,
-                 self.weight_decay, self.grad_averaging, self.mode, self.normalize_grad)
+        hyper = (self.lr, self.beta1, self.beta2, self.eps, self.bias_correction, self.weight_decay,
+                 self.grad_averaging, self.mode, self.normalize_grad)
+        if self.mixed:
+            _op.lans_mixed(tensor_list + p_list, step, *hyper)
+        else:
+            _op.lans(tensor_list, step, *hyper)
         self._step += 1

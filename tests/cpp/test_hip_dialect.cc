@@ -165,6 +165,24 @@ int main() {
     for (int i = 0; i < 6; ++i) l->tensor_list.push_back(T({8}, DevType::kROCM()));
     l->step = T({}, DevType::kROCM());
     EXPECT(Raises([&] { RunDeclare(MakeCall("raf.op.lans", l)); }).find("4n tensors") != std::string::npos);
+    EXPECT(Raises([&] { RunDeclare(MakeCall("raf.op.lans_mixed", l)); }).find("5n tensors") != std::string::npos);
+  }
+
+  std::puts("extension op lans_mixed: five blocks, 16-bit parameters");
+  {
+    auto mixed = OpDialect::GetDispatchList("raf.op.lans_mixed", DevType::kROCM());
+    EXPECT(mixed.size() == 1 && mixed.front().dialect_op == "raf.op.hip.lans_mixed");
+    auto l = std::make_shared<schema::LansArgs>();
+    for (int i = 0; i < 5; ++i) l->tensor_list.push_back(T({8}, DevType::kROCM(), 32));  // p is fp32: refused
+    l->step = T({}, DevType::kROCM());
+    l->mode = 1;
+    auto lc = MakeCall("raf.op.lans_mixed", l);
+    RunDeclare(lc);
+    EXPECT(value::AsTuple(lc->out)->fields.size() == 5);
+    EXPECT(value::AsTuple(lc->out)->fields[4] == l->tensor_list[4]);
+    OpEnvPtr le((*OpEnvMaker::Get("raf.op.hip.lans_mixed"))(lc));
+    EXPECT(le->HasError() && le->error_msgs[0].find("float16 or bfloat16") != std::string::npos);
+    EXPECT(le->name().find("raf_op_hip_lans_mixed") == 0);
   }
 
   std::puts("unique and truncated OpEnv names");

@@ -15,10 +15,17 @@ def rng_for(cfg: int, tensor: int, field: int) -> np.random.Generator:
 
 
 def lans_inputs(sizes, cfg=0, g16=False, zero_state=False, loss_scale=1024.0):
+    """``g16``: False -> fp32 gradients; True or "float16" -> loss-scaled float16; "bfloat16" ->
+    loss-scaled bfloat16 carried as uint16 bit patterns."""
     g, w, m, v = [], [], [], []
     for t, n in enumerate(sizes):
         gt = rng_for(cfg, t, 0).normal(0.0, 1e-3, n)
-        g.append((gt * loss_scale).astype(np.float16) if g16 else gt.astype(np.float32))
+        if g16 == "bfloat16":
+            from oracle.halfs import f32_to_bf16_bits
+
+            g.append(f32_to_bf16_bits((gt * loss_scale).astype(np.float32)))
+        else:
+            g.append((gt * loss_scale).astype(np.float16) if g16 else gt.astype(np.float32))
         w.append(rng_for(cfg, t, 1).normal(0.0, 0.02, n).astype(np.float32))
         if zero_state:
             m.append(np.zeros(n, np.float32))

@@ -184,7 +184,7 @@ def test_optim_classes_follow_reference_semantics(native_libs):
     assert lans._step == 5
     for p, a in zip(params, hw):
         assert p.shape == a.shape and max_rel_err(p.cpu().numpy(), a) <= 1e-5
-    for (_, m, v), a, b in zip(lans.params, hm, hvv):
+    for (_, _, m, v), a, b in zip(lans.params, hm, hvv):
         assert max_rel_err(m.cpu().numpy(), a) <= 1e-5 and max_rel_err(v.cpu().numpy(), b) <= 1e-5
 
 
@@ -208,3 +208,43 @@ def test_op_lans_fp16_gradients_with_unscale(native_libs):
         assert max_rel_err(tl[4 + t].cpu().numpy(), om[t]) <= 1e-5
         assert max_rel_err(tl[6 + t].cpu().numpy(), ov[t]) <= 1e-5
         assert np.array_equal(tl[t].cpu().numpy(), g[t])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_op_lans_mixed_and_half_precision_optimizer(native_libs, dtype):
+    """The extension op through dialect dispatch, and raf_amd.optim.LANS on a half-precision model:
+    fp32 master weights follow the oracle, the model's parameters are their 16-bit narrowing."""
+    from oracle import halfs, lans_f64
+    from raf_amd import op, optim
+    from tests.helpers import lans_inputs
+
+    name = "float16" if dtype == torch.float16 else "bfloat16"
+    sizes = [100, 4097, 20000]
+    _, w, m, v = lans_inputs(sizes, cfg=91)
+    params = [torch.from_numpy(a).to(DEV).to(dtype).requires_grad_() for a in w]
+    masters = [p.detach().float().cpu().numpy() for p in params]  # what the optimizer starts from
+    grads = [(torch.randn(n, device=DEV, generator=torch.Generator(DEV).manual_seed(7 + i)) * 1e-3).to(dtype)
+             for i, n in enumerate(sizes)]
+    opt = optim.LANS(params)
+    assert opt.mixed
+    g_np = [(halfs.f32_to_bf16_bits(g.float().cpu().numpy()) if name == "bfloat16" else g.cpu().numpy())
+            for g in grads]
+    ow, om, ov = masters, [np.zeros_like(a) for a in masters], [np.zeros_like(a) for a in masters]
+    for step in (1, 2, 3):
+        for p, g in zip(params, grads):
+            p.grad = g
+        opt.step()
+        ow, om, ov, op16, _ = lans_f64.lans_mixed_step(g_np, ow, om, ov, step, lans_f64.LansHParams(), name)
+    for (p, wm, mm, vm), a, b, c in zip(opt.params, ow, om, ov):
+        assert max_rel_err(wm.cpu().numpy(), a) <= 1e-5
+        assert max_rel_err(mm.cpu().numpy(), b) <= 1e-5 and max_rel_err(vm.cpu().numpy(), c) <= 1e-5
+        bits = p.detach().view(torch.int16).cpu().numpy().view(np.uint16)
+        assert np.array_equal(bits, halfs.narrow_weight(wm.cpu().numpy(), name).view(np.uint16))
+    # the op itself: picked by dispatch, output list is the input list
+    tl = grads + [t[1] for t in opt.params] + [t[2] for t in opt.params] + [t[3] for t in opt.params] + \
+        [p.data for p in params]
+    out = op.lans_mixed(tl, torch.tensor(4.0, device=DEV), 1e-3, 0.9, 0.999, 1e-6, True, 0.01, True, True, True)
+    assert out[7] is tl[7] and len(out) == 15
+    with pytest.raises(native_libs.RafError, match="float16 or bfloat16"):
+        op.lans_mixed(tl[:12] + [t.float() for t in tl[12:]], torch.tensor(4.0, device=DEV), 1e-3, 0.9, 0.999,
+                      1e-6, True, 0.01, True, True, True)

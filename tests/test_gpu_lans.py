@@ -236,7 +236,7 @@ def test_workspace_and_argument_errors(native_libs):
     with pytest.raises(TypeError):
         plan.step([t[0].half()], t, t, t, 1, hp)
     with pytest.raises(TypeError):
-        kernels.LansPlan([8], torch.bfloat16, DEV)
+        kernels.LansPlan([8], torch.float64, DEV)
 
 
 # ------------------------------------------------------------------ the two schedules

@@ -281,7 +281,7 @@ def test_state_dtype_and_shapes():
 
 
 # ------------------------------------------------------------------ the C restatement
-@pytest.mark.parametrize("g16", [False, True])
+@pytest.mark.parametrize("g16", [False, True, "bfloat16"])
 @pytest.mark.parametrize("mode", [0, 1])
 def test_c_restatement_matches_numpy_oracle(c_oracle, g16, mode):
     sizes = [1, 3, 4, 5, 511, 513, 4097, 70000, 0]
@@ -296,6 +296,51 @@ def test_c_restatement_matches_numpy_oracle(c_oracle, g16, mode):
         mism = sum(int((a != b).sum()) for a, b in zip(ws + ms + vs, wc + mc + vc))
         assert mism <= 2  # a rounding-boundary flip is possible, nothing more
         np.testing.assert_allclose(nc, norms, rtol=1e-13)
+
+
+# ------------------------------------------------------------------ mixed precision
+def test_bf16_gradient_equals_its_widened_float32(c_oracle):
+    """group_cast widens exactly (python/raf/optim/lans.py:261-265): a bfloat16 gradient and the
+    fp32 array holding the same values give identical results in both oracles."""
+    from oracle import halfs
+
+    g, w, m, v = lans_inputs([5000, 7], cfg=52, g16="bfloat16")
+    g32 = [halfs.bf16_bits_to_f32(x) for x in g]
+    # the widened values really are on the bfloat16 grid and scaled as generated (~1e-3 * 1024)
+    assert all((x.view(np.uint32) & 0xFFFF == 0).all() for x in g32)
+    assert 0.5 < np.std(g32[0]) < 2.0
+    hp = LansHParams(grad_unscale=1 / 1024)
+    a = lans_f64.lans_step(g, w, m, v, 2, hp)
+    b = lans_f64.lans_step(g32, w, m, v, 2, hp)
+    for x, y in zip(a[0] + a[1] + a[2], b[0] + b[1] + b[2]):
+        assert np.array_equal(x, y)
+    wc, mc, vc = [x.copy() for x in w], [x.copy() for x in m], [x.copy() for x in v]
+    wd, md, vd = [x.copy() for x in w], [x.copy() for x in m], [x.copy() for x in v]
+    c_oracle.lans_step_inplace(g, wc, mc, vc, 2, hp)
+    c_oracle.lans_step_inplace(g32, wd, md, vd, 2, hp)
+    for x, y in zip(wc + mc + vc, wd + md + vd):
+        assert np.array_equal(x, y)
+
+
+@pytest.mark.parametrize("model_dtype", ["float16", "bfloat16"])
+def test_mixed_step_copies_are_the_narrowed_stored_weights(c_oracle, model_dtype):
+    """cast(new_w, dtype) acts on the fp32 weight that was stored (lans.py:289-291), not on the
+    float64 value behind it; both oracles must agree on that, bit for bit given equal weights."""
+    import torch
+    from oracle import halfs
+
+    g, w, m, v = lans_inputs([4097, 3, 70000], cfg=53, g16=True)
+    hp = LansHParams(grad_unscale=1 / 1024)
+    ws, ms, vs, ps, _ = lans_f64.lans_mixed_step(g, w, m, v, 2, hp, model_dtype)
+    tdt = torch.float16 if model_dtype == "float16" else torch.bfloat16
+    for w32, p in zip(ws, ps):
+        t = torch.from_numpy(w32).to(tdt).view(torch.int16).numpy().view(np.uint16)
+        assert np.array_equal(p.view(np.uint16), t)
+    wc, mc, vc = [x.copy() for x in w], [x.copy() for x in m], [x.copy() for x in v]
+    pc = [np.zeros(x.size, np.uint16) for x in w]
+    c_oracle.lans_step_inplace(g, wc, mc, vc, 2, hp, p_list=pc, model_dtype=model_dtype)
+    for w32, p in zip(wc, pc):
+        assert np.array_equal(p, halfs.narrow_weight(w32, model_dtype).view(np.uint16))
 
 
 def test_c_restatement_thread_count_independent(c_oracle):
