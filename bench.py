@@ -67,6 +67,10 @@ def workloads():
         "lans_gpt2_1p5b_fp32": dict(kind="lans", sizes=shapes.numels(shapes.gpt2_shapes()), g16=False,
                                     zero_state=True, step0=1),
         "sgd_4m_fp32": dict(kind="sgd", n=4_194_304),
+        # neighbours of the optimizer step that reuse its machinery
+        "l2norm_bert_large_flat_fp32": dict(kind="l2norm", n=sum(shapes.numels(shapes.bert_large_shapes()))),
+        "fuse_bert_large_fp32": dict(kind="fuse", sizes=shapes.numels(shapes.bert_large_shapes()), gather=True),
+        "defuse_bert_large_fp32": dict(kind="fuse", sizes=shapes.numels(shapes.bert_large_shapes()), gather=False),
         # a plain device-to-device copy of known size: the yardstick that rocprofv3's FETCH_SIZE /
         # WRITE_SIZE counters are scaled by when HBM traffic is measured
         "copy_1gib": dict(kind="copy", nbytes=1 << 30),
@@ -286,6 +290,107 @@ def bench_sgd(name, wl, args):
     return out
 
 
+def _timed(fn, args):
+    """Warm-up, then `steps` calls of fn between events on torch's current stream (the one the
+    kernels are launched on); returns (wall ms per step, device ms per step)."""
+    import torch
+
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for i in range(args.warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(args.steps):
+        fn(i)
+    stop.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    return wall_ms, start.elapsed_time(stop) / args.steps
+
+
+def _line(metric, name, dtype, bytes_step, wall_ms, dev_ms, kernel, args, config):
+    achieved = bytes_step / (dev_ms * 1e-3) / 1e9
+    return {
+        "metric": metric, "value": round(bytes_step / (wall_ms * 1e-3) / 1e9, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
+        "config": dict(workload=name, **config),
+        "roofline": {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC.get((name, kernel)), "bytes_per_launch": bytes_step,
+                     "avg_launch_ms": round(dev_ms, 5)},
+    }
+
+
+def bench_l2norm(name, wl, args):
+    import torch
+
+    from oracle import tensor_ops
+    from raf_amd import kernels
+
+    dev = torch.device("cuda:0")
+    n = wl["n"]
+    x = torch.randn(n, device=dev, generator=torch.Generator(dev).manual_seed(2024)) * 0.02
+    out = torch.empty((), device=dev)
+    ws = torch.empty(max(_libs().rafhip_l2norm_workspace_bytes(n), 8), dtype=torch.uint8, device=dev)
+    wall_ms, dev_ms = _timed(lambda i: kernels.l2norm(x, out=out, workspace=ws), args)
+    res = _line("L2 norm achieved HBM bandwidth (algorithmic bytes / time)", name, "f64", 4 * n, wall_ms, dev_ms,
+                "l2norm_partials", args, {"elements": n, "bytes_per_element": 4, "storage": "fp32"})
+    if not args.no_cpu_baseline:
+        sample = x[:1 << 26].cpu().numpy()
+        best = None
+        for _ in range(5):
+            t0 = time.perf_counter()
+            tensor_ops.l2norm(sample)
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        res["cpu_baseline"] = {"value": round(sample.size * 4 / best / 1e9, 2), "unit": "GB/s", "cores": 1,
+                               "kind": "port", "sample": f"first {sample.size} elements, best of 5, NumPy float64 oracle"}
+    return res
+
+
+def bench_fuse(name, wl, args):
+    import torch
+
+    from oracle import tensor_ops
+    from raf_amd import kernels
+
+    dev = torch.device("cuda:0")
+    sizes = wl["sizes"]
+    gen = torch.Generator(dev).manual_seed(2024)
+    parts = [torch.randn(n, device=dev, generator=gen) for n in sizes]
+    flat = torch.randn(sum(sizes), device=dev, generator=gen)
+    plan = kernels.FusePlan([4 * n for n in sizes], dev)
+    if wl["gather"]:
+        step, kernel, what = (lambda i: plan.fuse(parts, flat)), "fuse_copy", "fuse_tensor"
+    else:
+        step, kernel, what = (lambda i: plan.defuse(flat, parts)), "fuse_copy", "defuse_tensor"
+    wall_ms, dev_ms = _timed(step, args)
+    moved = 2 * plan.total_bytes
+    res = _line(f"{what} achieved HBM bandwidth (bytes read + written / time)", name, "u8", moved, wall_ms, dev_ms,
+                kernel, args, {"tensors": len(sizes), "bytes_read_per_step": plan.total_bytes,
+                               "bytes_written_per_step": plan.total_bytes, "launches_per_step": 1})
+    if not args.no_cpu_baseline:
+        host = [p.cpu().numpy() for p in parts[:48]]
+        best = None
+        for _ in range(5):
+            t0 = time.perf_counter()
+            tensor_ops.fuse_tensor(host)
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        nb = sum(a.nbytes for a in host)
+        res["cpu_baseline"] = {"value": round(2 * nb / best / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": f"first {len(host)} tensors ({nb} bytes), best of 5, NumPy oracle (fuse direction)"}
+    return res
+
+
+def _libs():
+    from raf_amd import _lib
+
+    return _lib.optim()
+
+
 def bench_copy(name, wl, args):
     import torch
 
@@ -343,7 +448,8 @@ def main():
 
     _lib.optim()  # fails loudly if the HIP library is not built
     wl = table[args.workload]
-    fn = {"lans": bench_lans, "sgd": bench_sgd, "copy": bench_copy}[wl["kind"]]
+    fn = {"lans": bench_lans, "sgd": bench_sgd, "copy": bench_copy, "l2norm": bench_l2norm,
+          "fuse": bench_fuse}[wl["kind"]]
     out = fn(args.workload, wl, args)
     print(json.dumps(out), flush=True)
 

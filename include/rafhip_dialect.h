@@ -77,6 +77,38 @@ int rafhip_raf_lans_execute(rafhip_raf_env* env, int32_t list_len,
                             const rafhip_tensor_desc* tensor_list, const rafhip_tensor_desc* step,
                             void* workspace, int64_t workspace_bytes, void* stream);
 
+/* raf.op.l2norm(x) -> 0-d tensor of x's dtype; scripts/src_codegen/def_schema.py:425-427,
+ * src/op/declare/reduce.cc:118-126. */
+int rafhip_raf_l2norm_make(const rafhip_tensor_desc* x, rafhip_raf_env** env_out);
+int rafhip_raf_l2norm_execute(rafhip_raf_env* env, const rafhip_tensor_desc* x,
+                              const rafhip_tensor_desc* out, void* workspace,
+                              int64_t workspace_bytes, void* stream);
+
+/* raf.op.fuse_tensor(data) -> 1-d tensor holding every tensor's elements back to back
+ * (def_schema.py:829-835, src/op/declare/memory.cc:43-63).  An empty list declares no output:
+ * make succeeds, the env has no outputs and execute does nothing. */
+int rafhip_raf_fuse_tensor_make(int32_t n, const rafhip_tensor_desc* data,
+                                rafhip_raf_env** env_out);
+int rafhip_raf_fuse_tensor_execute(rafhip_raf_env* env, int32_t n, const rafhip_tensor_desc* data,
+                                   const rafhip_tensor_desc* out, void* stream);
+
+/* raf.op.defuse_tensor(data, sizes, shapes, shape_indices) -> tuple of tensors
+ * (def_schema.py:836-841, src/op/declare/memory.cc:65-93). */
+int rafhip_raf_defuse_tensor_make(const rafhip_tensor_desc* data, int32_t n_sizes,
+                                  const int64_t* sizes, int32_t n_shapes, const int64_t* shapes,
+                                  int32_t n_indices, const int64_t* shape_indices,
+                                  rafhip_raf_env** env_out);
+int rafhip_raf_defuse_tensor_execute(rafhip_raf_env* env, const rafhip_tensor_desc* data,
+                                     int32_t n_out, const rafhip_tensor_desc* outs, void* stream);
+
+/* What the op's declare function produced (call->out): number of output tensors (a tuple counts
+ * its fields; -1 on NULL) and each one's dtype and shape, so that the caller can allocate them the
+ * way an executor does (src/impl/interpreter.cc:397-426).  shape_out may be NULL to query ndim. */
+int32_t rafhip_raf_env_num_outputs(const rafhip_raf_env* env);
+int rafhip_raf_env_output(const rafhip_raf_env* env, int32_t index, int32_t* dtype_code,
+                          int32_t* dtype_bits, int32_t* ndim, int64_t* shape_out,
+                          int32_t shape_capacity);
+
 /* Total bytes of the OpEnv's workspace requests (each rounded up to 256). */
 int64_t rafhip_raf_env_workspace_bytes(const rafhip_raf_env* env);
 /* OpEnv::name() and the dialect op the dispatcher picked; pointers stay valid until destroy. */

@@ -12,6 +12,10 @@
  *                           python/raf/_tvm_op/sgd.py:13-30, registered at
  *                           src/op/dialect/tvm/optimizer.cc:44-45 and invoked with
  *                           [x, dx, v, v1, x1] at src/op/dialect/tvm/tvm_utils.cc:92-133.
+ *   rafhip_l2norm           cublasSnrm2 / cublasDnrm2 in device-pointer mode behind
+ *                           `raf.op.cublas.l2norm`, src/op/dialect/cublas/l2_norm.cc:52-75.
+ *   rafhip_fuse_* / defuse  the per-tensor cudaMemcpyAsync loops of `raf.op.cuda.fuse_tensor` and
+ *                           `raf.op.cuda.defuse_tensor`, src/op/dialect/cuda/memory.cc:55-68, :120-134.
  *   rafhip_lans_*           multi_tensor_lans_cuda<float>(...) declared at
  *                           src/op/dialect/cuda/kernels/kernel_util.cuh:25-34 and called from
  *                           LansImpl::Execute, src/op/dialect/cuda/lans.cc:124-130; the plan object
@@ -43,7 +47,8 @@ typedef enum rafhip_status {
 typedef enum rafhip_dtype {
   RAFHIP_F32 = 0,
   RAFHIP_F16 = 1, /* IEEE binary16; LANS gradients and 16-bit weight copies only */
-  RAFHIP_BF16 = 2 /* bfloat16; LANS gradients and 16-bit weight copies only      */
+  RAFHIP_BF16 = 2, /* bfloat16; LANS gradients and 16-bit weight copies only      */
+  RAFHIP_F64 = 3   /* IEEE binary64; rafhip_l2norm only                            */
 } rafhip_dtype;
 
 /* ABI version of the loaded library (== RAFHIP_ABI_VERSION it was built with). */
@@ -209,6 +214,38 @@ int rafhip_lans_timing_read(rafhip_lans_plan* plan, int32_t slot, float* ms_out5
  */
 int rafhip_lans_debug_trace(rafhip_lans_plan* plan, uint64_t* words_out, int64_t capacity_items,
                             int64_t* n_items_out);
+
+/* --------------------------------------------------------------------------------------- l2norm
+ * `raf.op.l2norm(x)`: out = sqrt(sum x_i^2) as ONE element of x's dtype on the device
+ * (src/op/declare/reduce.cc:118-124).  dtype: RAFHIP_F32, RAFHIP_F64 (the two the reference's
+ * cuBLAS backend takes, l2_norm.cc:57-71), RAFHIP_F16, RAFHIP_BF16.  Squares are accumulated in
+ * float64 in a fixed order (the result is bit-identical from run to run and device to device) and
+ * rounded once to the output dtype.  n == 0 gives 0.  workspace: device scratch of at least
+ * rafhip_l2norm_workspace_bytes(n) bytes, 8-byte aligned, no initialisation needed (0 bytes, and
+ * workspace may be NULL, for tensors of at most 16384 elements).
+ */
+int64_t rafhip_l2norm_workspace_bytes(int64_t n);
+int rafhip_l2norm(const void* x, int32_t dtype, int64_t n, void* out, void* workspace,
+                  int64_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------- fuse / defuse tensor
+ * `raf.op.fuse_tensor(data)` packs a list of tensors back to back into one flat buffer and
+ * `raf.op.defuse_tensor(data, sizes, ...)` unpacks it (src/op/declare/memory.cc:43-93); offsets are
+ * the running sums of the tensors' byte sizes (memory.cc:61-66).  A plan fixes the byte sizes, as
+ * the reference's OpEnv constructors do (memory.cc:33-43, :95-103), and owns a small device
+ * table; each call is ONE kernel launch whatever the number of tensors, and allocates nothing.
+ * nbytes[i] >= 0; empty tensors and empty lists are valid.  Pointers need no alignment (16-byte
+ * lane accesses are used when source and destination agree modulo 4).  One call at a time per plan.
+ */
+typedef struct rafhip_fuse_plan rafhip_fuse_plan;
+int rafhip_fuse_plan_create(int32_t n_tensors, const int64_t* nbytes, rafhip_fuse_plan** out_plan);
+int rafhip_fuse_plan_destroy(rafhip_fuse_plan* plan);
+int64_t rafhip_fuse_plan_total_bytes(const rafhip_fuse_plan* plan); /* -1 on NULL */
+/* parts: host array of n_tensors device pointers; fused: device buffer of total_bytes. */
+int rafhip_fuse_tensors(rafhip_fuse_plan* plan, const void* const* parts, void* fused,
+                        void* stream);
+int rafhip_defuse_tensor(rafhip_fuse_plan* plan, const void* fused, void* const* parts,
+                         void* stream);
 
 #ifdef __cplusplus
 }

@@ -24,6 +24,7 @@ RAFHIP_ERR_NO_DEVICE = 5
 RAFHIP_F32 = 0
 RAFHIP_F16 = 1
 RAFHIP_BF16 = 2
+RAFHIP_F64 = 3
 
 RAFHIP_LANS_PHASED = 0
 RAFHIP_LANS_PIPELINED = 1
@@ -84,6 +85,13 @@ OPTIM_SYMBOLS = {
     "rafhip_lans_step_mixed": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
                                        POINTER(c_void_p), POINTER(c_void_p), c_int32, c_void_p, c_int32,
                                        POINTER(LansHParams), c_void_p, c_int64, c_void_p]),
+    "rafhip_l2norm_workspace_bytes": (c_int64, [c_int64]),
+    "rafhip_l2norm": (c_int, [c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_int64, c_void_p]),
+    "rafhip_fuse_plan_create": (c_int, [c_int32, POINTER(c_int64), POINTER(c_void_p)]),
+    "rafhip_fuse_plan_destroy": (c_int, [c_void_p]),
+    "rafhip_fuse_plan_total_bytes": (c_int64, [c_void_p]),
+    "rafhip_fuse_tensors": (c_int, [c_void_p, POINTER(c_void_p), c_void_p, c_void_p]),
+    "rafhip_defuse_tensor": (c_int, [c_void_p, c_void_p, POINTER(c_void_p), c_void_p]),
     "rafhip_lans_read_norms": (c_int, [c_void_p, c_void_p, POINTER(c_double), c_void_p]),
     "rafhip_lans_debug_trace": (c_int, [c_void_p, POINTER(ctypes.c_uint64), c_int64, POINTER(c_int64)]),
     "rafhip_lans_timing_enable": (c_int, [c_void_p, c_int32]),
@@ -120,6 +128,19 @@ DIALECT_SYMBOLS = {
                                      c_int32, POINTER(c_void_p)]),
     "rafhip_raf_lans_execute": (c_int, [c_void_p, c_int32, POINTER(TensorDesc),
                                         POINTER(TensorDesc), c_void_p, c_int64, c_void_p]),
+    "rafhip_raf_l2norm_make": (c_int, [POINTER(TensorDesc), POINTER(c_void_p)]),
+    "rafhip_raf_l2norm_execute": (c_int, [c_void_p, POINTER(TensorDesc), POINTER(TensorDesc), c_void_p,
+                                          c_int64, c_void_p]),
+    "rafhip_raf_fuse_tensor_make": (c_int, [c_int32, POINTER(TensorDesc), POINTER(c_void_p)]),
+    "rafhip_raf_fuse_tensor_execute": (c_int, [c_void_p, c_int32, POINTER(TensorDesc), POINTER(TensorDesc),
+                                               c_void_p]),
+    "rafhip_raf_defuse_tensor_make": (c_int, [POINTER(TensorDesc), c_int32, POINTER(c_int64), c_int32,
+                                              POINTER(c_int64), c_int32, POINTER(c_int64), POINTER(c_void_p)]),
+    "rafhip_raf_defuse_tensor_execute": (c_int, [c_void_p, POINTER(TensorDesc), c_int32, POINTER(TensorDesc),
+                                                 c_void_p]),
+    "rafhip_raf_env_num_outputs": (c_int32, [c_void_p]),
+    "rafhip_raf_env_output": (c_int, [c_void_p, c_int32, POINTER(c_int32), POINTER(c_int32), POINTER(c_int32),
+                                      POINTER(c_int64), c_int32]),
     "rafhip_raf_env_workspace_bytes": (c_int64, [c_void_p]),
     "rafhip_raf_env_name": (c_char_p, [c_void_p]),
     "rafhip_raf_env_op": (c_char_p, [c_void_p]),

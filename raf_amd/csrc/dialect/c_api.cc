@@ -76,14 +76,33 @@ struct WorkspaceBinding {
 
 rafhip_raf_env* Finish(const CallValues& call) {
   RunDeclare(call);
-  std::string picked;
-  OpEnvPtr env = DispatchSingleOp(call, &picked);
   auto* h = new rafhip_raf_env();
-  h->env = env;
   h->call = call;
+  if (call->callee.empty()) return h;  // declared as a no-op (an empty tensor list): nothing to dispatch
+  std::string picked;
+  std::unique_ptr<rafhip_raf_env> guard(h);
+  OpEnvPtr env = DispatchSingleOp(call, &picked);
+  h->env = env;
   h->name = env->name();
   h->op = picked;
-  return h;
+  return guard.release();
+}
+
+std::vector<int64_t> ToVector(const int64_t* p, int32_t n, const char* what) {
+  if (n < 0 || (n > 0 && !p)) throw Error(std::string(what) + ": bad integer list");
+  return std::vector<int64_t>(p, p + n);
+}
+
+// The declared outputs, flattened: a tensor is one output, a tuple its fields.
+std::vector<value::TensorValue> Outputs(const rafhip_raf_env* env) {
+  std::vector<value::TensorValue> outs;
+  if (!env->call->out) return outs;
+  if (auto t = std::dynamic_pointer_cast<value::TensorValueObj>(env->call->out)) {
+    outs.push_back(t);
+  } else {
+    for (const auto& f : value::AsTuple(env->call->out)->fields) outs.push_back(value::AsTensor(f));
+  }
+  return outs;
 }
 
 }  // namespace
@@ -219,8 +238,114 @@ int rafhip_raf_lans_execute(rafhip_raf_env* env, int32_t list_len,
   });
 }
 
+int rafhip_raf_l2norm_make(const rafhip_tensor_desc* x, rafhip_raf_env** env_out) {
+  return Guard([&] {
+    if (!env_out) throw Error("rafhip_raf_l2norm_make: env_out is NULL");
+    *env_out = nullptr;
+    auto args = std::make_shared<schema::L2NormArgs>();
+    args->x = FromDesc(x, "x");
+    *env_out = Finish(MakeCall("raf.op.l2norm", args));
+  });
+}
+
+int rafhip_raf_l2norm_execute(rafhip_raf_env* env, const rafhip_tensor_desc* x,
+                              const rafhip_tensor_desc* out, void* workspace,
+                              int64_t workspace_bytes, void* stream) {
+  return Guard([&] {
+    if (!env || !env->env) throw Error("rafhip_raf_l2norm_execute: env is NULL");
+    std::vector<value::Value> inputs = {FromDesc(x, "x")};
+    OpEnv::SetStreamForAllBackends(env->call->device, stream);
+    WorkspaceBinding bind(env->env.get(), workspace, workspace_bytes);
+    env->env->Execute(inputs, FromDesc(out, "out"));
+  });
+}
+
+int rafhip_raf_fuse_tensor_make(int32_t n, const rafhip_tensor_desc* data,
+                                rafhip_raf_env** env_out) {
+  return Guard([&] {
+    if (!env_out) throw Error("rafhip_raf_fuse_tensor_make: env_out is NULL");
+    *env_out = nullptr;
+    if (n < 0 || (n > 0 && !data)) throw Error("rafhip_raf_fuse_tensor_make: bad tensor list");
+    auto args = std::make_shared<schema::FuseTensorArgs>();
+    for (int32_t i = 0; i < n; ++i) args->data.push_back(FromDesc(&data[i], "data"));
+    *env_out = Finish(MakeCall("raf.op.fuse_tensor", args));
+  });
+}
+
+int rafhip_raf_fuse_tensor_execute(rafhip_raf_env* env, int32_t n, const rafhip_tensor_desc* data,
+                                   const rafhip_tensor_desc* out, void* stream) {
+  return Guard([&] {
+    if (!env) throw Error("rafhip_raf_fuse_tensor_execute: env is NULL");
+    if (!env->env) return;  // declared as a no-op
+    if (n < 0 || (n > 0 && !data)) throw Error("rafhip_raf_fuse_tensor_execute: bad tensor list");
+    std::vector<value::Value> fields;
+    for (int32_t i = 0; i < n; ++i) fields.push_back(FromDesc(&data[i], "data"));
+    std::vector<value::Value> inputs = {value::MakeTuple(std::move(fields))};
+    OpEnv::SetStreamForAllBackends(env->call->device, stream);
+    WorkspaceBinding bind(env->env.get(), nullptr, 0);
+    env->env->Execute(inputs, FromDesc(out, "out"));
+  });
+}
+
+int rafhip_raf_defuse_tensor_make(const rafhip_tensor_desc* data, int32_t n_sizes,
+                                  const int64_t* sizes, int32_t n_shapes, const int64_t* shapes,
+                                  int32_t n_indices, const int64_t* shape_indices,
+                                  rafhip_raf_env** env_out) {
+  return Guard([&] {
+    if (!env_out) throw Error("rafhip_raf_defuse_tensor_make: env_out is NULL");
+    *env_out = nullptr;
+    auto args = std::make_shared<schema::DefuseTensorArgs>();
+    args->data = FromDesc(data, "data");
+    args->sizes = ToVector(sizes, n_sizes, "sizes");
+    args->shapes = ToVector(shapes, n_shapes, "shapes");
+    args->shape_indices = ToVector(shape_indices, n_indices, "shape_indices");
+    *env_out = Finish(MakeCall("raf.op.defuse_tensor", args));
+  });
+}
+
+int rafhip_raf_defuse_tensor_execute(rafhip_raf_env* env, const rafhip_tensor_desc* data,
+                                     int32_t n_out, const rafhip_tensor_desc* outs, void* stream) {
+  return Guard([&] {
+    if (!env) throw Error("rafhip_raf_defuse_tensor_execute: env is NULL");
+    if (!env->env) return;  // declared as a no-op
+    if (n_out < 0 || (n_out > 0 && !outs)) throw Error("rafhip_raf_defuse_tensor_execute: bad output list");
+    std::vector<value::Value> fields;
+    for (int32_t i = 0; i < n_out; ++i) fields.push_back(FromDesc(&outs[i], "out"));
+    std::vector<value::Value> inputs = {FromDesc(data, "data")};
+    OpEnv::SetStreamForAllBackends(env->call->device, stream);
+    WorkspaceBinding bind(env->env.get(), nullptr, 0);
+    env->env->Execute(inputs, value::MakeTuple(std::move(fields)));
+  });
+}
+
+int32_t rafhip_raf_env_num_outputs(const rafhip_raf_env* env) {
+  if (!env) return -1;
+  int32_t n = -1;
+  Guard([&] { n = (int32_t)Outputs(env).size(); });
+  return n;
+}
+
+int rafhip_raf_env_output(const rafhip_raf_env* env, int32_t index, int32_t* dtype_code,
+                          int32_t* dtype_bits, int32_t* ndim, int64_t* shape_out,
+                          int32_t shape_capacity) {
+  return Guard([&] {
+    if (!env || !dtype_code || !dtype_bits || !ndim) throw Error("rafhip_raf_env_output: null argument");
+    auto outs = Outputs(env);
+    if (index < 0 || (size_t)index >= outs.size()) throw Error("rafhip_raf_env_output: no such output");
+    const TensorView& t = outs[(size_t)index]->tensor;
+    *dtype_code = t.dtype.code;
+    *dtype_bits = t.dtype.bits;
+    *ndim = t.ndim();
+    if (shape_out) {
+      if (shape_capacity < t.ndim()) throw Error("rafhip_raf_env_output: shape buffer too small");
+      for (int i = 0; i < t.ndim(); ++i) shape_out[i] = t.shape[(size_t)i];
+    }
+  });
+}
+
 int64_t rafhip_raf_env_workspace_bytes(const rafhip_raf_env* env) {
   if (!env) return -1;
+  if (!env->env) return 0;
   int64_t need = 0;
   for (const auto& r : env->env->workspace_requests()) need += RoundUp(r.nbytes);
   return need;

@@ -4,6 +4,9 @@
 //
 // Counterparts in the reference tree:
 //   LansHipEnv   LansImpl, src/op/dialect/cuda/lans.cc:25-165 (registration :164-165)
+//   L2NormHipEnv       L2NormImpl, src/op/dialect/cublas/l2_norm.cc:26-86
+//   FuseTensorHipEnv   CudaFuseTensor, src/op/dialect/cuda/memory.cc:27-77
+//   DefuseTensorHipEnv CudaDefuseTensor, src/op/dialect/cuda/memory.cc:82-143
 //   SgdHipEnv    the RAF_TVM(sgd, ...) backend, src/op/dialect/tvm/optimizer.cc:22-45, whose
 //                Execute packs [x, dx, v, v1, x1] (src/op/dialect/tvm/tvm_utils.cc:92-133)
 // Differences on purpose: the stream is looked up at Execute time (the reference caches it in the
@@ -243,6 +246,151 @@ class LansHipEnv : public OpEnv {
   int64_t workspace_bytes_ = 0;
 };
 
+// -------------------------------------------------------------------------------------- l2norm
+class L2NormHipEnv : public OpEnv {
+ public:
+  explicit L2NormHipEnv(const CallValues& cv) {
+    const auto* args = cv->args_as<schema::L2NormArgs>();
+    if (!args) {
+      error_msgs.push_back("raf.op.hip.l2norm: call does not carry L2NormArgs");
+      return;
+    }
+    arg_indices = {args->FieldIndex("x")};  // l2_norm.cc:38-40
+    const TensorView& x = args->x->tensor;
+    n_ = x.numel();
+    dtype_ = x.dtype.code == kDLFloat && x.dtype.bits == 64 ? (int32_t)RAFHIP_F64 : KernelDType(x.dtype);
+    if (cv->device.device_type() != DevType::kROCM())
+      error_msgs.push_back("raf.op.hip.l2norm: device is not rocm");
+    if (dtype_ < 0) error_msgs.push_back("raf.op.hip.l2norm: Unsupported output dtype");  // l2_norm.cc:73
+    if (error_msgs.empty() && rafhip_device_count() <= 0)
+      error_msgs.push_back("raf.op.hip.l2norm: no HIP device is visible");
+    if (!error_msgs.empty()) return;
+    workspace_bytes_ = rafhip_l2norm_workspace_bytes(n_);
+    if (workspace_bytes_ > 0) RequestWorkspace(&workspace_, cv->device, workspace_bytes_);
+  }
+
+  std::string name() const override { return name_; }
+
+  void Execute(const CallValues& cv) override {
+    const auto* args = cv->args_as<schema::L2NormArgs>();
+    RAF_CHECK(args != nullptr, "raf.op.hip.l2norm expects L2NormArgs");
+    Execute(std::vector<Value>{args->x}, cv->out);
+  }
+
+  void Execute(const std::vector<Value>& inputs, Value output) override {
+    RAF_CHECK(inputs.size() == 1, "raf.op.hip.l2norm takes x");
+    const TensorView& x = AsTensor(inputs[0])->tensor;
+    const TensorView& out = AsTensor(output)->tensor;
+    RAF_CHECK(x.numel() == n_, "raf.op.hip.l2norm: element count changed since the OpEnv was made");
+    void* stream = DeviceAPI::Get(DevType::kROCM())->GetStream();
+    int st = rafhip_l2norm(x.data, dtype_, n_, out.data, workspace_, workspace_bytes_, stream);
+    if (st != RAFHIP_OK) throw Error(KernelError("rafhip_l2norm", st));
+  }
+
+  static OpEnv* make(const CallValues& cv) { return new L2NormHipEnv(cv); }
+
+ private:
+  int64_t n_ = 0;
+  int32_t dtype_ = -1;
+  void* workspace_ = nullptr;
+  int64_t workspace_bytes_ = 0;
+  std::string name_ = TruncateName(GetUniqueName("raf.op.hip.l2norm"));
+};
+
+// ------------------------------------------------------------------------- fuse / defuse tensor
+// Both hold a plan made from the tensors' byte sizes, which the reference's constructors record
+// too (memory.cc:37-43, :99-103).  The reference issues its copies on a dedicated copy stream
+// (RequestStream, memory.cc:32, :93); here the single launch goes to the current compute stream.
+class FuseBase : public OpEnv {
+ public:
+  ~FuseBase() override {
+    if (plan_) rafhip_fuse_plan_destroy(plan_);
+  }
+  std::string name() const override { return name_; }
+
+ protected:
+  FuseBase(const char* op, const CallValues& cv) : op_(op), name_(TruncateName(GetUniqueName(op))) {
+    if (cv->device.device_type() != DevType::kROCM()) error_msgs.push_back(op_ + ": device is not rocm");
+  }
+  void MakePlan(const std::vector<int64_t>& nbytes) {
+    if (!error_msgs.empty()) return;
+    if (rafhip_device_count() <= 0) {
+      error_msgs.push_back(op_ + ": no HIP device is visible");
+      return;
+    }
+    int st = rafhip_fuse_plan_create((int32_t)nbytes.size(), nbytes.data(), &plan_);
+    if (st != RAFHIP_OK) error_msgs.push_back(KernelError("rafhip_fuse_plan_create", st));
+    n_ = nbytes.size();
+  }
+  std::vector<void*> Pointers(const value::TupleValue& tuple) const {
+    RAF_CHECK(tuple->fields.size() == n_, op_ + ": tensor count changed since the OpEnv was made");
+    std::vector<void*> ptrs(n_);
+    for (size_t i = 0; i < n_; ++i) ptrs[i] = AsTensor(tuple->fields[i])->tensor.data;
+    return ptrs;
+  }
+  std::string op_, name_;
+  rafhip_fuse_plan* plan_ = nullptr;
+  size_t n_ = 0;
+};
+
+class FuseTensorHipEnv : public FuseBase {
+ public:
+  explicit FuseTensorHipEnv(const CallValues& cv) : FuseBase("raf.op.hip.fuse_tensor", cv) {
+    const auto* args = cv->args_as<schema::FuseTensorArgs>();
+    if (!args) {
+      error_msgs.push_back(op_ + ": call does not carry FuseTensorArgs");
+      return;
+    }
+    arg_indices = {args->FieldIndex("data")};  // memory.cc:31
+    std::vector<int64_t> nbytes;
+    for (const auto& t : args->data) nbytes.push_back(t->tensor.numel() * ((t->tensor.dtype.bits + 7) / 8));
+    MakePlan(nbytes);
+  }
+  void Execute(const CallValues& cv) override {
+    const auto* args = cv->args_as<schema::FuseTensorArgs>();
+    RAF_CHECK(args != nullptr, op_ + " expects FuseTensorArgs");
+    std::vector<Value> fields(args->data.begin(), args->data.end());
+    Execute(std::vector<Value>{value::MakeTuple(std::move(fields))}, cv->out);
+  }
+  void Execute(const std::vector<Value>& inputs, Value output) override {
+    RAF_CHECK(inputs.size() == 1, op_ + " takes (data)");
+    std::vector<void*> ptrs = Pointers(AsTuple(inputs[0]));
+    void* stream = DeviceAPI::Get(DevType::kROCM())->GetStream();
+    int st = rafhip_fuse_tensors(plan_, ptrs.data(), AsTensor(output)->tensor.data, stream);
+    if (st != RAFHIP_OK) throw Error(KernelError("rafhip_fuse_tensors", st));
+  }
+  static OpEnv* make(const CallValues& cv) { return new FuseTensorHipEnv(cv); }
+};
+
+class DefuseTensorHipEnv : public FuseBase {
+ public:
+  explicit DefuseTensorHipEnv(const CallValues& cv) : FuseBase("raf.op.hip.defuse_tensor", cv) {
+    const auto* args = cv->args_as<schema::DefuseTensorArgs>();
+    if (!args) {
+      error_msgs.push_back(op_ + ": call does not carry DefuseTensorArgs");
+      return;
+    }
+    arg_indices = {args->FieldIndex("data")};  // memory.cc:92
+    const int64_t eb = (args->data->tensor.dtype.bits + 7) / 8;  // memory.cc:97-102
+    std::vector<int64_t> nbytes;
+    for (int64_t s : args->sizes) nbytes.push_back(s * eb);
+    MakePlan(nbytes);
+  }
+  void Execute(const CallValues& cv) override {
+    const auto* args = cv->args_as<schema::DefuseTensorArgs>();
+    RAF_CHECK(args != nullptr, op_ + " expects DefuseTensorArgs");
+    Execute(std::vector<Value>{args->data}, cv->out);
+  }
+  void Execute(const std::vector<Value>& inputs, Value output) override {
+    RAF_CHECK(inputs.size() == 1, op_ + " takes (data)");
+    std::vector<void*> ptrs = Pointers(AsTuple(output));
+    void* stream = DeviceAPI::Get(DevType::kROCM())->GetStream();
+    int st = rafhip_defuse_tensor(plan_, AsTensor(inputs[0])->tensor.data, ptrs.data(), stream);
+    if (st != RAFHIP_OK) throw Error(KernelError("rafhip_defuse_tensor", st));
+  }
+  static OpEnv* make(const CallValues& cv) { return new DefuseTensorHipEnv(cv); }
+};
+
 RAF_REGISTER_DIALECT("hip").set_enable(DevType::kROCM());
 // plevels above the reference's own backends (cuda lans = 20, tvm sgd = 10).
 RAF_REGISTER_DIALECT_OP(hip, lans, 30);
@@ -251,6 +399,13 @@ RAF_REGISTER_DIALECT_OP(hip, lans_mixed, 30);
 RAF_OP_ENV_MAKER("raf.op.hip.lans_mixed", LansHipEnv::make_mixed);
 RAF_REGISTER_DIALECT_OP(hip, sgd, 30);
 RAF_OP_ENV_MAKER("raf.op.hip.sgd", SgdHipEnv::make);
+// cublas l2norm is plevel 15, tvm 10; cuda fuse_tensor / defuse_tensor are plevel 10.
+RAF_REGISTER_DIALECT_OP(hip, l2norm, 30);
+RAF_OP_ENV_MAKER("raf.op.hip.l2norm", L2NormHipEnv::make);
+RAF_REGISTER_DIALECT_OP(hip, fuse_tensor, 30);
+RAF_OP_ENV_MAKER("raf.op.hip.fuse_tensor", FuseTensorHipEnv::make);
+RAF_REGISTER_DIALECT_OP(hip, defuse_tensor, 30);
+RAF_OP_ENV_MAKER("raf.op.hip.defuse_tensor", DefuseTensorHipEnv::make);
 
 }  // namespace hip
 }  // namespace op

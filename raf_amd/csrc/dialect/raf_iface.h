@@ -164,6 +164,24 @@ struct LansArgs : ArgsBase {  // def_schema.py:678-694
   int FieldIndex(const std::string& name) const override;
 };
 
+struct L2NormArgs : ArgsBase {  // def_schema.py:425-427
+  value::TensorValue x;
+  int FieldIndex(const std::string& name) const override;
+};
+
+struct FuseTensorArgs : ArgsBase {  // def_schema.py:829-835
+  std::vector<value::TensorValue> data;
+  int FieldIndex(const std::string& name) const override;
+};
+
+struct DefuseTensorArgs : ArgsBase {  // def_schema.py:836-841
+  value::TensorValue data;
+  std::vector<int64_t> sizes;          // element count of every output
+  std::vector<int64_t> shapes;         // all outputs' dimensions, concatenated
+  std::vector<int64_t> shape_indices;  // end of every output's dimensions in `shapes`
+  int FieldIndex(const std::string& name) const override;
+};
+
 }  // namespace schema
 
 // ---------------------------------------------------------------------------------- CallValues

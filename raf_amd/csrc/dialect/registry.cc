@@ -84,6 +84,21 @@ int LansArgs::FieldIndex(const std::string& name) const {
   return IndexIn(kNames, 11, name);
 }
 
+int L2NormArgs::FieldIndex(const std::string& name) const {
+  static const char* const kNames[] = {"x"};
+  return IndexIn(kNames, 1, name);
+}
+
+int FuseTensorArgs::FieldIndex(const std::string& name) const {
+  static const char* const kNames[] = {"data"};
+  return IndexIn(kNames, 1, name);
+}
+
+int DefuseTensorArgs::FieldIndex(const std::string& name) const {
+  static const char* const kNames[] = {"data", "sizes", "shapes", "shape_indices"};
+  return IndexIn(kNames, 4, name);
+}
+
 }  // namespace schema
 
 CallValues MakeCall(const std::string& op_name, std::shared_ptr<schema::ArgsBase> args) {
@@ -150,6 +165,69 @@ void LansMixedDecl(const CallValues& call) {
   call->out = value::MakeTuple(std::move(out));
 }
 
+// src/op/declare/reduce.cc:118-124: a 0-d output of x's dtype on x's device.
+void L2NormDecl(const CallValues& call) {
+  const auto* args = call->args_as<schema::L2NormArgs>();
+  RAF_CHECK(args != nullptr && args->x, "raf.op.l2norm expects a tensor");
+  TensorView out;
+  out.device = args->x->tensor.device;
+  out.dtype = args->x->tensor.dtype;
+  call->out = value::MakeTensor(out);
+  call->device = out.device;
+}
+
+// src/op/declare/memory.cc:43-63: a 1-d output with the total element count, dtype and device of
+// the first tensor; an empty list has no output and no callee.
+void FuseTensorDecl(const CallValues& call) {
+  const auto* args = call->args_as<schema::FuseTensorArgs>();
+  RAF_CHECK(args != nullptr, "raf.op.fuse_tensor expects FuseTensorArgs");
+  if (args->data.empty()) {
+    call->callee.clear();
+    return;
+  }
+  int64_t total = 0;
+  for (const auto& t : args->data) {
+    RAF_CHECK(t != nullptr, "data holds a null tensor");
+    total += t->tensor.numel();
+  }
+  const TensorView& x = args->data[0]->tensor;
+  TensorView out;
+  out.device = x.device;
+  out.dtype = x.dtype;
+  out.shape = {total};
+  call->out = value::MakeTensor(out);
+  call->device = x.device;
+}
+
+// src/op/declare/memory.cc:65-93: the sizes must add up to the input's element count; one output
+// per entry of shape_indices, shaped by its slice of `shapes`.
+void DefuseTensorDecl(const CallValues& call) {
+  const auto* args = call->args_as<schema::DefuseTensorArgs>();
+  RAF_CHECK(args != nullptr && args->data, "raf.op.defuse_tensor expects DefuseTensorArgs");
+  const TensorView& x = args->data->tensor;
+  call->device = x.device;
+  int64_t total = 0;
+  for (int64_t s : args->sizes) total += s;
+  RAF_CHECK(total == x.numel(), "Input tensor size should be " + std::to_string(total) + ", got " +
+                                    std::to_string(x.numel()) + ".");
+  std::vector<value::Value> outs;
+  int64_t start = 0;
+  for (int64_t end : args->shape_indices) {
+    RAF_CHECK(start <= end && end <= (int64_t)args->shapes.size(), "shape_indices out of range");
+    TensorView t;
+    t.device = x.device;
+    t.dtype = x.dtype;
+    t.shape.assign(args->shapes.begin() + start, args->shapes.begin() + end);
+    outs.push_back(value::MakeTensor(t));
+    start = end;
+  }
+  if (outs.empty()) {
+    call->callee.clear();
+    return;
+  }
+  call->out = value::MakeTuple(std::move(outs));
+}
+
 }  // namespace
 
 void RunDeclare(const CallValues& call) {
@@ -158,6 +236,9 @@ void RunDeclare(const CallValues& call) {
   if (op == "raf.op.sgd") return SgdDecl(call);
   if (op == "raf.op.lans") return LansDecl(call);
   if (op == "raf.op.lans_mixed") return LansMixedDecl(call);
+  if (op == "raf.op.l2norm") return L2NormDecl(call);
+  if (op == "raf.op.fuse_tensor") return FuseTensorDecl(call);
+  if (op == "raf.op.defuse_tensor") return DefuseTensorDecl(call);
   throw Error("no declare function registered for op " + op);
 }
 

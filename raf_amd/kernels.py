@@ -12,7 +12,7 @@ from typing import List, Optional, Sequence
 import torch
 
 from . import _lib
-from ._lib import LansHParams, RAFHIP_BF16, RAFHIP_F16, RAFHIP_F32, check
+from ._lib import LansHParams, RAFHIP_BF16, RAFHIP_F16, RAFHIP_F32, RAFHIP_F64, check
 
 
 def _current_stream(device) -> int:
@@ -41,6 +41,87 @@ def sgd_f32(x: torch.Tensor, dx: torch.Tensor, v: torch.Tensor, learning_rate: f
                                       x1.data_ptr(), x.numel(), float(learning_rate), float(mu),
                                       _current_stream(x.device)))
     return v1, x1
+
+
+_NORM_DTYPES = {torch.float32: RAFHIP_F32, torch.float64: RAFHIP_F64, torch.float16: RAFHIP_F16,
+                torch.bfloat16: RAFHIP_BF16}
+
+
+def l2norm(x: torch.Tensor, out: Optional[torch.Tensor] = None,
+           workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``rafhip_l2norm``: sqrt(sum x^2) as a 0-d tensor of x's dtype, left on the device."""
+    if not x.is_cuda or not x.is_contiguous():
+        raise ValueError("l2norm: expected a contiguous tensor on the GPU")
+    if x.dtype not in _NORM_DTYPES:
+        raise TypeError(f"l2norm: unsupported dtype {x.dtype}")
+    lib = _lib.optim()
+    if out is None:
+        out = torch.empty((), dtype=x.dtype, device=x.device)
+    elif out.dtype != x.dtype or out.numel() != 1 or not out.is_cuda:
+        raise TypeError("l2norm: out must be a one-element GPU tensor of x's dtype")
+    need = lib.rafhip_l2norm_workspace_bytes(x.numel())
+    if workspace is None and need > 0:
+        workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+    check(lib.rafhip_l2norm(x.data_ptr(), _NORM_DTYPES[x.dtype], x.numel(), out.data_ptr(),
+                            workspace.data_ptr() if workspace is not None else None,
+                            workspace.numel() if workspace is not None else 0,
+                            _current_stream(x.device)))
+    return out
+
+
+class FusePlan:
+    """Owns a ``rafhip_fuse_plan`` for a list of tensors of fixed byte sizes: ``fuse`` packs them
+    back to back into one flat buffer, ``defuse`` unpacks it, one kernel launch each."""
+
+    def __init__(self, nbytes: Sequence[int], device="cuda:0"):
+        self._h = c_void_p(None)
+        self.lib = _lib.optim()
+        self.device = torch.device(device)
+        self.nbytes = [int(b) for b in nbytes]
+        self.n = len(self.nbytes)
+        arr = (c_int64 * max(self.n, 1))(*self.nbytes)
+        with torch.cuda.device(self.device):
+            check(self.lib.rafhip_fuse_plan_create(self.n, arr, ctypes.byref(self._h)))
+        self.total_bytes = self.lib.rafhip_fuse_plan_total_bytes(self._h)
+
+    def close(self):
+        if self._h:
+            self.lib.rafhip_fuse_plan_destroy(self._h)
+            self._h = c_void_p(None)
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:  # interpreter shutdown
+            pass
+
+    def _ptrs(self, parts: Sequence[torch.Tensor]):
+        if len(parts) != self.n:
+            raise ValueError(f"expected {self.n} tensors, got {len(parts)}")
+        arr = (c_void_p * max(self.n, 1))()
+        for i, t in enumerate(parts):
+            if not t.is_cuda or not t.is_contiguous():
+                raise ValueError(f"parts[{i}]: need a contiguous GPU tensor")
+            if t.numel() * t.element_size() != self.nbytes[i]:
+                raise ValueError(f"parts[{i}]: {t.numel() * t.element_size()} bytes, plan has {self.nbytes[i]}")
+            arr[i] = t.data_ptr()
+        return arr
+
+    def _check_flat(self, flat: torch.Tensor):
+        if not flat.is_cuda or not flat.is_contiguous() or flat.numel() * flat.element_size() != self.total_bytes:
+            raise ValueError(f"flat buffer: need a contiguous GPU tensor of {self.total_bytes} bytes")
+
+    def fuse(self, parts: Sequence[torch.Tensor], flat: torch.Tensor) -> torch.Tensor:
+        self._check_flat(flat)
+        check(self.lib.rafhip_fuse_tensors(self._h, self._ptrs(parts), flat.data_ptr(),
+                                           _current_stream(self.device)))
+        return flat
+
+    def defuse(self, flat: torch.Tensor, parts: Sequence[torch.Tensor]):
+        self._check_flat(flat)
+        check(self.lib.rafhip_defuse_tensor(self._h, flat.data_ptr(), self._ptrs(parts),
+                                            _current_stream(self.device)))
+        return parts
 
 
 def make_hparams(learning_rate=1e-3, beta1=0.9, beta2=0.999, eps=1e-6, bias_correction=1,

@@ -24,7 +24,8 @@ DEV_CPU, DEV_CUDA, DEV_ROCM = 1, 2, 10  # include/raf/device.h:37-50
 
 _DTYPES = {
     torch.float32: (2, 32), torch.float16: (2, 16), torch.float64: (2, 64),
-    torch.bfloat16: (4, 16), torch.int32: (0, 32), torch.int64: (0, 64),
+    torch.bfloat16: (4, 16), torch.int32: (0, 32), torch.int64: (0, 64), torch.uint8: (1, 8),
+    torch.int8: (0, 8), torch.int16: (0, 16),
 }
 
 
@@ -139,6 +140,85 @@ def _lans(op_name, tensor_list, step, learning_rate, beta1, beta2, eps, bias_cor
     check_raf(lib.rafhip_raf_lans_execute(env.handle, n4, descs, dstep, ws_ptr,
                                           env.workspace_bytes, stream))
     return tensor_list
+
+
+_TORCH_DTYPES = {v: k for k, v in _DTYPES.items()}
+
+
+def _alloc_outputs(env: _Env, device) -> List[torch.Tensor]:
+    """Allocate what the op's declare function produced, like the executor's AllocOutputBuffer
+    (src/impl/interpreter.cc:397-426)."""
+    lib = _lib.dialect()
+    outs = []
+    for i in range(lib.rafhip_raf_env_num_outputs(env.handle)):
+        code, bits, ndim = ctypes.c_int32(), ctypes.c_int32(), ctypes.c_int32()
+        shape = (c_int64 * 16)()
+        check_raf(lib.rafhip_raf_env_output(env.handle, i, ctypes.byref(code), ctypes.byref(bits),
+                                            ctypes.byref(ndim), shape, 16))
+        outs.append(torch.empty(tuple(shape[:ndim.value]), dtype=_TORCH_DTYPES[(code.value, bits.value)],
+                                device=device))
+    return outs
+
+
+def l2norm(x: torch.Tensor) -> torch.Tensor:
+    """``raf._op.imp.l2norm(x)``: sqrt(sum(x*x)) as a 0-d tensor of x's dtype on x's device
+    (src/op/declare/reduce.cc:118-124)."""
+    lib = _lib.dialect()
+    keep: list = []
+    dx = _desc(x, keep)
+    key = ("l2norm", _sig(x))
+    env = _env_cache.get(key)
+    if env is None:
+        h = c_void_p(None)
+        check_raf(lib.rafhip_raf_l2norm_make(dx, ctypes.byref(h)))
+        env = _env_cache[key] = _Env(h)
+    (out,) = _alloc_outputs(env, x.device)
+    ws = torch.empty(env.workspace_bytes, dtype=torch.uint8, device=x.device) if env.workspace_bytes else None
+    check_raf(lib.rafhip_raf_l2norm_execute(env.handle, dx, _desc(out, keep), ws.data_ptr() if ws is not None else None,
+                                            env.workspace_bytes, _stream(x)))
+    return out
+
+
+def fuse_tensor(data: Sequence[torch.Tensor]):
+    """``raf._op.imp.fuse_tensor(data)``: one flat 1-d tensor with every tensor's elements back to
+    back (src/op/declare/memory.cc:43-63).  An empty list has no output (None)."""
+    lib = _lib.dialect()
+    data = list(data)
+    keep: list = []
+    descs = (TensorDesc * max(len(data), 1))(*[_desc(t, keep) for t in data])
+    key = ("fuse_tensor", tuple(_sig(t) for t in data))
+    env = _env_cache.get(key)
+    if env is None:
+        h = c_void_p(None)
+        check_raf(lib.rafhip_raf_fuse_tensor_make(len(data), descs, ctypes.byref(h)))
+        env = _env_cache[key] = _Env(h)
+    if not data:
+        return None
+    (out,) = _alloc_outputs(env, data[0].device)
+    check_raf(lib.rafhip_raf_fuse_tensor_execute(env.handle, len(data), descs, _desc(out, keep), _stream(data[0])))
+    return out
+
+
+def defuse_tensor(data: torch.Tensor, sizes, shapes, shape_indices):
+    """``raf._op.imp.defuse_tensor(data, sizes, shapes, shape_indices)``: the inverse of
+    ``fuse_tensor``; ``sizes`` are element counts, ``shapes`` the concatenated dimensions and
+    ``shape_indices`` where each output's dimensions end (src/op/declare/memory.cc:65-93)."""
+    lib = _lib.dialect()
+    keep: list = []
+    dd = _desc(data, keep)
+    sizes, shapes, shape_indices = [int(v) for v in sizes], [int(v) for v in shapes], [int(v) for v in shape_indices]
+    key = ("defuse_tensor", _sig(data), tuple(sizes), tuple(shapes), tuple(shape_indices))
+    env = _env_cache.get(key)
+    if env is None:
+        h = c_void_p(None)
+        arr = lambda v: (c_int64 * max(len(v), 1))(*v)
+        check_raf(lib.rafhip_raf_defuse_tensor_make(dd, len(sizes), arr(sizes), len(shapes), arr(shapes),
+                                                    len(shape_indices), arr(shape_indices), ctypes.byref(h)))
+        env = _env_cache[key] = _Env(h)
+    outs = _alloc_outputs(env, data.device)
+    descs = (TensorDesc * max(len(outs), 1))(*[_desc(t, keep) for t in outs])
+    check_raf(lib.rafhip_raf_defuse_tensor_execute(env.handle, dd, len(outs), descs, _stream(data)))
+    return outs
 
 
 _lans_grad_unscale = 1.0

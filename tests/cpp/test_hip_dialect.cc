@@ -168,6 +168,53 @@ int main() {
     EXPECT(Raises([&] { RunDeclare(MakeCall("raf.op.lans_mixed", l)); }).find("5n tensors") != std::string::npos);
   }
 
+  std::puts("l2norm, fuse_tensor, defuse_tensor: declares and dialect ops");
+  {
+    for (const char* name : {"l2norm", "fuse_tensor", "defuse_tensor"}) {
+      auto l = OpDialect::GetDispatchList(std::string("raf.op.") + name, DevType::kROCM());
+      EXPECT(l.size() == 1 && l.front().dialect_op == std::string("raf.op.hip.") + name && l.front().plevel == 30);
+    }
+    auto n = std::make_shared<schema::L2NormArgs>();
+    n->x = T({2, 3, 4}, DevType::kROCM(), 64);
+    auto nc = MakeCall("raf.op.l2norm", n);
+    RunDeclare(nc);
+    const TensorView& no = value::AsTensor(nc->out)->tensor;
+    EXPECT(no.ndim() == 0 && no.dtype.bits == 64 && nc->device.device_type() == DevType::kROCM());
+
+    auto f = std::make_shared<schema::FuseTensorArgs>();
+    f->data = {T({3, 5}, DevType::kROCM()), T({7}, DevType::kROCM()), T({}, DevType::kROCM())};
+    auto fc = MakeCall("raf.op.fuse_tensor", f);
+    RunDeclare(fc);
+    EXPECT(value::AsTensor(fc->out)->tensor.shape == (std::vector<int64_t>{23}));
+    auto fe = MakeCall("raf.op.fuse_tensor", std::make_shared<schema::FuseTensorArgs>());
+    RunDeclare(fe);
+    EXPECT(fe->callee.empty() && !fe->out);  // empty list: no callee, no output
+
+    auto d = std::make_shared<schema::DefuseTensorArgs>();
+    d->data = T({23}, DevType::kROCM());
+    d->sizes = {15, 7, 1};
+    d->shapes = {3, 5, 7};
+    d->shape_indices = {2, 3, 3};
+    auto dc = MakeCall("raf.op.defuse_tensor", d);
+    RunDeclare(dc);
+    auto outs = value::AsTuple(dc->out)->fields;
+    EXPECT(outs.size() == 3);
+    EXPECT(value::AsTensor(outs[0])->tensor.shape == (std::vector<int64_t>{3, 5}));
+    EXPECT(value::AsTensor(outs[2])->tensor.ndim() == 0);
+    d->sizes = {15, 7, 2};
+    EXPECT(Raises([&] { RunDeclare(MakeCall("raf.op.defuse_tensor", d)); })
+               .find("Input tensor size should be 24, got 23.") != std::string::npos);
+    d->sizes = {15, 7, 1};
+    OpEnvPtr de((*OpEnvMaker::Get("raf.op.hip.defuse_tensor"))(dc));
+    EXPECT((de->arg_indices == std::vector<int>{0}));
+    auto cpu = std::make_shared<schema::L2NormArgs>();
+    cpu->x = T({4}, DevType::kCPU());
+    auto cc = MakeCall("raf.op.l2norm", cpu);
+    RunDeclare(cc);
+    OpEnvPtr ce((*OpEnvMaker::Get("raf.op.hip.l2norm"))(cc));
+    EXPECT(ce->HasError() && ce->error_msgs[0].find("not rocm") != std::string::npos);
+  }
+
   std::puts("extension op lans_mixed: five blocks, 16-bit parameters");
   {
     auto mixed = OpDialect::GetDispatchList("raf.op.lans_mixed", DevType::kROCM());

@@ -29,6 +29,8 @@ def test_dispatch_lists_seen_from_python(native_libs):
     assert op.dispatch_list("raf.op.lans") == [("hip", "raf.op.hip.lans", 30)]
     assert op.dispatch_list("raf.op.sgd") == [("hip", "raf.op.hip.sgd", 30)]
     assert op.dispatch_list("raf.op.lans_mixed") == [("hip", "raf.op.hip.lans_mixed", 30)]
+    for name in ("l2norm", "fuse_tensor", "defuse_tensor"):
+        assert op.dispatch_list(f"raf.op.{name}") == [("hip", f"raf.op.hip.{name}", 30)]
     assert op.dispatch_list("raf.op.lans", op.DEV_CPU) == []
     with op.with_dialect("tvm"):
         assert op.dispatch_list("raf.op.sgd") == []
@@ -57,6 +59,23 @@ def test_declare_errors_reach_python(native_libs):
         op.lans([x] * 3, torch.tensor(1.0), 1e-3, .9, .999, 1e-6, True, 0.01, True, True, True)
     with pytest.raises(_lib.RafError, match="5n tensors"):
         op.lans_mixed([x] * 4, torch.tensor(1.0), 1e-3, .9, .999, 1e-6, True, 0.01, True, True, True)
+
+
+def test_tensor_op_declares_reach_python(native_libs):
+    """Declare-time behaviour of l2norm / fuse_tensor / defuse_tensor without a GPU: size check,
+    the empty list, and no backend for CPU tensors."""
+    from raf_amd import _lib, op
+
+    x = torch.zeros(6)
+    with pytest.raises(_lib.RafError, match="Input tensor size should be 7, got 6"):
+        op.defuse_tensor(x, [3, 4], [3, 4], [1, 2])
+    with pytest.raises(_lib.RafError, match="Cannot find a valid dispatch for op raf.op.defuse_tensor"):
+        op.defuse_tensor(x, [2, 4], [2, 2, 2], [1, 3])
+    with pytest.raises(_lib.RafError, match="Cannot find a valid dispatch for op raf.op.l2norm"):
+        op.l2norm(x)
+    with pytest.raises(_lib.RafError, match="Cannot find a valid dispatch for op raf.op.fuse_tensor"):
+        op.fuse_tensor([x, x])
+    assert op.fuse_tensor([]) is None  # declared as a no-op (src/op/declare/memory.cc:54-55)
 
 
 def test_optimizer_front_end_argument_checks():
