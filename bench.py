@@ -67,6 +67,7 @@ def workloads():
         "lans_gpt2_1p5b_fp32": dict(kind="lans", sizes=shapes.numels(shapes.gpt2_shapes()), g16=False,
                                     zero_state=True, step0=1),
         "sgd_4m_fp32": dict(kind="sgd", n=4_194_304),
+        "sgd_multi_bert_large_fp32": dict(kind="sgd_multi", sizes=shapes.numels(shapes.bert_large_shapes())),
         # neighbours of the optimizer step that reuse its machinery
         "l2norm_bert_large_flat_fp32": dict(kind="l2norm", n=sum(shapes.numels(shapes.bert_large_shapes()))),
         "fuse_bert_large_fp32": dict(kind="fuse", sizes=shapes.numels(shapes.bert_large_shapes()), gather=True),
@@ -323,6 +324,31 @@ def _line(metric, name, dtype, bytes_step, wall_ms, dev_ms, kernel, args, config
     }
 
 
+def bench_sgd_multi(name, wl, args):
+    import torch
+
+    from oracle import c_oracle
+    from raf_amd import kernels
+
+    dev = torch.device("cuda:0")
+    sizes = wl["sizes"]
+    total = sum(sizes)
+    gen = torch.Generator(dev).manual_seed(2024)
+    x = [torch.randn(n, device=dev, generator=gen) * 0.02 for n in sizes]
+    dx = [torch.randn(n, device=dev, generator=gen) * 1e-3 for n in sizes]
+    v = [torch.zeros(n, device=dev) for n in sizes]
+    plan = kernels.SgdPlan(sizes, torch.float32, dev)
+    m = plan.marshal(x, dx, v)
+    wall_ms, dev_ms = _timed(lambda i: plan.step(x, dx, v, 0.01, 0.9, marshalled=m), args)
+    res = _line("multi-tensor SGD momentum step achieved HBM bandwidth (algorithmic bytes / step time)", name, "f32",
+                total * SGD_BYTES_PER_ELT, wall_ms, dev_ms, "sgd_multi_kernel", args,
+                {"tensors": len(sizes), "elements": total, "bytes_per_element": SGD_BYTES_PER_ELT,
+                 "launches_per_step": 1})
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline_sgd(1 << 24)
+    return res
+
+
 def bench_l2norm(name, wl, args):
     import torch
 
@@ -449,7 +475,7 @@ def main():
     _lib.optim()  # fails loudly if the HIP library is not built
     wl = table[args.workload]
     fn = {"lans": bench_lans, "sgd": bench_sgd, "copy": bench_copy, "l2norm": bench_l2norm,
-          "fuse": bench_fuse}[wl["kind"]]
+          "fuse": bench_fuse, "sgd_multi": bench_sgd_multi}[wl["kind"]]
     out = fn(args.workload, wl, args)
     print(json.dumps(out), flush=True)
 

@@ -72,6 +72,29 @@ int rafhip_device_count(void);
 int rafhip_sgd_f32(const float* x, const float* dx, const float* v, float* v_out, float* x_out,
                    int64_t n, double learning_rate, double mu, void* stream);
 
+/*
+ * Multi-tensor momentum SGD, IN PLACE on x and v, one launch for a whole parameter list.  Per
+ * element exactly the four roundings above.  It replaces, per step, the op sequence the reference's
+ * traced optimizer emits for EVERY parameter -- cast(dx, fp32), multiply, add(out=v), multiply,
+ * subtract(out=w), cast(w, dtype), add(out=p) (python/raf/optim/sgd.py:187-215) -- and the
+ * one-call-per-parameter loop of its imperative optimizer (sgd.py:51-58).
+ *   plan       fixes the element counts and the gradient dtype (RAFHIP_F32, _F16, _BF16; half
+ *              gradients are widened exactly, as cast does); owns a small device table.
+ *   x, dx, v   host arrays of n_tensors device pointers: fp32 (master) weights, gradients,
+ *              fp32 velocities.
+ *   p          NULL, or host array of device pointers (entries may be NULL) that receive the new
+ *              weight narrowed to p_dtype (RAFHIP_F16 / RAFHIP_BF16), round to nearest even: the
+ *              half-precision model parameters.
+ * Allocates nothing; one call at a time per plan.
+ */
+typedef struct rafhip_sgd_plan rafhip_sgd_plan;
+int rafhip_sgd_plan_create(int32_t n_tensors, const int64_t* numel, int32_t grad_dtype,
+                           rafhip_sgd_plan** out_plan);
+int rafhip_sgd_plan_destroy(rafhip_sgd_plan* plan);
+int rafhip_sgd_multi_step(rafhip_sgd_plan* plan, float* const* x, const void* const* dx,
+                          float* const* v, void* const* p, int32_t p_dtype, double learning_rate,
+                          double mu, void* stream);
+
 /* ----------------------------------------------------------------------------------------- LANS
  * Hyper-parameters: the non-tensor schema fields of `raf.op.lans`
  * (scripts/src_codegen/def_schema.py:685-693) in schema order, fp32 like the schema's `float`.

@@ -47,3 +47,26 @@ def sgd_step(x0, dx, v0, learning_rate: float, mu: float):
         s = np.multiply(lr32, v1, dtype=np.float32)
         x1 = np.subtract(x0, s, dtype=np.float32)
     return v1, x1
+
+
+def sgd_list_step(x_list, dx_list, v_list, learning_rate: float, mu: float, model_dtype=None):
+    """What the reference's traced optimizer computes per parameter (python/raf/optim/
+    sgd.py:187-215): ``dx`` widened to fp32 (``cast(dxi, "float32")``, exact), then
+
+        v <- fl32(fl32(momentum * v) + dx)           add(multiply(momentum, v), dx, out=v)
+        w <- fl32(w - fl32(learning_rate * v))       subtract(w, multiply(lr, v), out=w)
+
+    -- the same four roundings as ``raf.op.sgd``, ``momentum`` and ``learning_rate`` being fp32
+    arrays (sgd.py:106-107) -- and, for a half-precision model, the parameter as
+    ``cast(new_w, dtype)``.  Gradients may be float32, float16 or bfloat16 bit patterns
+    (uint16).  Returns ``(xs, vs, ps)`` as new arrays; ``ps`` is None without ``model_dtype``."""
+    from oracle.halfs import narrow_weight, widen_grad
+
+    xs, vs = [], []
+    for x0, dx, v0 in zip(x_list, dx_list, v_list):
+        g = widen_grad(dx).reshape(np.asarray(x0).shape)
+        v1, x1 = sgd_step(x0, g, v0, learning_rate, mu)
+        xs.append(x1)
+        vs.append(v1)
+    ps = [narrow_weight(x, model_dtype) for x in xs] if model_dtype else None
+    return xs, vs, ps

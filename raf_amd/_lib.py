@@ -85,6 +85,10 @@ OPTIM_SYMBOLS = {
     "rafhip_lans_step_mixed": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
                                        POINTER(c_void_p), POINTER(c_void_p), c_int32, c_void_p, c_int32,
                                        POINTER(LansHParams), c_void_p, c_int64, c_void_p]),
+    "rafhip_sgd_plan_create": (c_int, [c_int32, POINTER(c_int64), c_int32, POINTER(c_void_p)]),
+    "rafhip_sgd_plan_destroy": (c_int, [c_void_p]),
+    "rafhip_sgd_multi_step": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
+                                      POINTER(c_void_p), c_int32, c_double, c_double, c_void_p]),
     "rafhip_l2norm_workspace_bytes": (c_int64, [c_int64]),
     "rafhip_l2norm": (c_int, [c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_int64, c_void_p]),
     "rafhip_fuse_plan_create": (c_int, [c_int32, POINTER(c_int64), POINTER(c_void_p)]),

@@ -1,0 +1,94 @@
+// A table of per-tensor records (pointers, sizes) that lives in device memory and has to follow
+// the pointers the caller passes with every call.  Shared by the multi-tensor plans (LANS, SGD,
+// fuse/defuse): the records go through a pinned staging buffer and an asynchronous copy on the
+// call's stream, and a call whose records equal the ones sent last time sends nothing -- a
+// training loop updates the same buffers every step.
+//
+// Rec must be trivially copyable with every byte initialised (records are compared with memcmp).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+#include <type_traits>
+#include <vector>
+
+namespace rafhip {
+
+template <typename Rec>
+class RecordUploader {
+  static_assert(std::is_trivially_copyable<Rec>::value, "records are copied and compared bytewise");
+
+ public:
+  RecordUploader() = default;
+  RecordUploader(const RecordUploader&) = delete;
+  RecordUploader& operator=(const RecordUploader&) = delete;
+  ~RecordUploader() { release(); }
+
+  // `device_table` must hold `count` records and outlive this object.
+  hipError_t init(Rec* device_table, size_t count) {
+    release();
+    device_ = device_table;
+    count_ = count;
+    if (count == 0) return hipSuccess;
+    hipError_t e = hipHostMalloc(reinterpret_cast<void**>(&staging_), sizeof(Rec) * count,
+                                 hipHostMallocDefault);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&staging_free_, hipEventDisableTiming);
+    if (e != hipSuccess) release();
+    return e;
+  }
+
+  void release() {
+    if (staging_free_) (void)hipEventDestroy(staging_free_);
+    if (staging_) (void)hipHostFree(staging_);
+    staging_free_ = nullptr;
+    staging_ = nullptr;
+    sent_once_ = false;
+    last_sent_.clear();
+  }
+
+  // Makes the device table equal to `recs` for work enqueued on `s` after this call.  Takes the
+  // vector's contents (swap) when it uploads.
+  hipError_t sync(std::vector<Rec>& recs, hipStream_t s) {
+    if (count_ == 0) return hipSuccess;
+    const size_t bytes = sizeof(Rec) * count_;
+    if (sent_once_ && std::memcmp(last_sent_.data(), recs.data(), bytes) == 0) return hipSuccess;
+    // The previous upload may still be reading the staging buffer.
+    if (sent_once_) {
+      hipError_t e = hipEventSynchronize(staging_free_);
+      if (e != hipSuccess) return e;
+    }
+    std::memcpy(staging_, recs.data(), bytes);
+    hipError_t e = hipMemcpyAsync(device_, staging_, bytes, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) e = hipEventRecord(staging_free_, s);
+    if (e != hipSuccess) return e;
+    last_sent_.swap(recs);
+    sent_once_ = true;
+    return hipSuccess;
+  }
+
+ private:
+  Rec* device_ = nullptr;
+  size_t count_ = 0;
+  Rec* staging_ = nullptr;  // pinned
+  hipEvent_t staging_free_ = nullptr;  // recorded after the last upload was enqueued
+  std::vector<Rec> last_sent_;
+  bool sent_once_ = false;
+};
+
+// CUs x 8 workgroups: enough resident wavefronts to cover HBM latency on every CU; grid-stride
+// loops do the rest.
+inline int streaming_grid_cap() {
+  static int cap = [] {
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) == hipSuccess) {
+      int v = 0;
+      if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
+          v > 0)
+        cus = v;
+    }
+    return cus * 8;
+  }();
+  return cap;
+}
+
+}  // namespace rafhip

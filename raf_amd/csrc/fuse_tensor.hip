@@ -17,10 +17,10 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
-#include <cstring>
 #include <new>
 #include <vector>
 
+#include "device_table.h"
 #include "status.h"
 
 namespace rafhip {
@@ -118,26 +118,21 @@ using namespace rafhip;
 struct rafhip_fuse_plan {
   int32_t n = 0;
   int device = 0;
-  int grid_cap = 2048;
   std::vector<int64_t> nbytes, offset;
   int64_t total_bytes = 0;
   int64_t n_items = 0;
   void* d_tables = nullptr;
   Segment* d_segments = nullptr;
   CopyItem* d_items = nullptr;
-  Segment* h_staging = nullptr;  // pinned
-  hipEvent_t staging_free = nullptr;
-  std::vector<Segment> last_sent;
-  bool sent_once = false;
+  RecordUploader<Segment> segments;
 };
 
 namespace {
 
 void free_plan(rafhip_fuse_plan* p) {
   if (!p) return;
+  p->segments.release();
   if (p->d_tables) (void)hipFree(p->d_tables);
-  if (p->h_staging) (void)hipHostFree(p->h_staging);
-  if (p->staging_free) (void)hipEventDestroy(p->staging_free);
   delete p;
 }
 
@@ -154,19 +149,9 @@ int run(rafhip_fuse_plan* plan, const char* what, void* const* parts, void* flat
     segs[i] = Segment{static_cast<char*>(parts[i]), plan->offset[i], plan->nbytes[i], 0};
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const size_t table_bytes = sizeof(Segment) * (size_t)plan->n;
-  if (!plan->sent_once || std::memcmp(plan->last_sent.data(), segs.data(), table_bytes) != 0) {
-    // The previous upload may still be reading the staging buffer.
-    if (plan->sent_once) RAFHIP_HIP_TRY(hipEventSynchronize(plan->staging_free));
-    std::memcpy(plan->h_staging, segs.data(), table_bytes);
-    RAFHIP_HIP_TRY(hipMemcpyAsync(plan->d_segments, plan->h_staging, table_bytes,
-                                  hipMemcpyHostToDevice, s));
-    RAFHIP_HIP_TRY(hipEventRecord(plan->staging_free, s));
-    plan->last_sent.swap(segs);
-    plan->sent_once = true;
-  }
-  const unsigned grid =
-      (unsigned)(plan->n_items < plan->grid_cap ? plan->n_items : (int64_t)plan->grid_cap);
+  RAFHIP_HIP_TRY(plan->segments.sync(segs, s));
+  const int64_t cap = streaming_grid_cap();
+  const unsigned grid = (unsigned)(plan->n_items < cap ? plan->n_items : cap);
   if (plan->total_bytes > kStreamFromBytes)
     hipLaunchKernelGGL(fuse_copy<true>, dim3(grid), dim3(kCopyBlock), 0, s, plan->d_segments,
                        plan->d_items, plan->n_items, static_cast<char*>(flat), gather ? 1 : 0);
@@ -217,19 +202,14 @@ int rafhip_fuse_plan_create(int32_t n_tensors, const int64_t* nbytes, rafhip_fus
     free_plan(p);
     return fail(RAFHIP_ERR_NO_DEVICE, "rafhip_fuse_plan_create: no HIP device available");
   }
-  int cus = 0;
-  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, p->device) == hipSuccess &&
-      cus > 0)
-    p->grid_cap = cus * 8;
   const size_t seg_bytes = (sizeof(Segment) * (size_t)n_tensors + 255) / 256 * 256;
   hipError_t e = hipMalloc(&p->d_tables, seg_bytes + sizeof(CopyItem) * items.size());
-  if (e == hipSuccess)
-    e = hipHostMalloc(reinterpret_cast<void**>(&p->h_staging), sizeof(Segment) * (size_t)n_tensors,
-                      hipHostMallocDefault);
-  if (e == hipSuccess) e = hipEventCreateWithFlags(&p->staging_free, hipEventDisableTiming);
   if (e == hipSuccess) {
     p->d_segments = static_cast<Segment*>(p->d_tables);
     p->d_items = reinterpret_cast<CopyItem*>(static_cast<char*>(p->d_tables) + seg_bytes);
+    e = p->segments.init(p->d_segments, (size_t)n_tensors);
+  }
+  if (e == hipSuccess) {
     e = hipMemcpy(p->d_items, items.data(), sizeof(CopyItem) * items.size(), hipMemcpyHostToDevice);
   }
   if (e != hipSuccess) {

@@ -4,36 +4,18 @@
 // :95-185 norms; host scalars src/op/dialect/cuda/lans.cc:94-109) evaluated in float64.
 #include "lans_kernels.h"
 
+#include "half_types.h"
 #include "rafhip_optim.h"
 
 namespace rafhip {
 namespace {
 
-// Global-address-space views: tensor pointers come out of a table in memory, so without these the
-// compiler falls back to flat (generic) loads and stores.
-#define RAFHIP_GLOBAL __attribute__((address_space(1)))
-typedef float f32x4 __attribute__((ext_vector_type(4)));  // native vector: HIP's f32x4 is a class
 typedef RAFHIP_GLOBAL const f32x4 gc_float4;
 typedef RAFHIP_GLOBAL f32x4 g_float4;
 typedef RAFHIP_GLOBAL const float gc_float;
 typedef RAFHIP_GLOBAL float g_float;
-typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
-typedef RAFHIP_GLOBAL const half4_t gc_half4;
-typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
-typedef RAFHIP_GLOBAL const half8_t gc_half8;
-typedef RAFHIP_GLOBAL const _Float16 gc_half;
-typedef unsigned short u16x4 __attribute__((ext_vector_type(4)));
-typedef unsigned short u16x8 __attribute__((ext_vector_type(8)));
-typedef RAFHIP_GLOBAL const u16x4 gc_u16x4;
-typedef RAFHIP_GLOBAL const u16x8 gc_u16x8;
 typedef RAFHIP_GLOBAL u16x4 g_u16x4;
-typedef RAFHIP_GLOBAL const unsigned short gc_u16;
 typedef RAFHIP_GLOBAL unsigned short g_u16;
-
-// Gradient element type tag for bfloat16 (two bytes, like the data).
-struct Bf16 {
-  unsigned short bits;
-};
 
 // ------------------------------------------------------------------ cache policy
 // Every pass streams far more data than the 256 MB Infinity Cache holds.  Loads and stores that
@@ -52,107 +34,6 @@ constexpr CachePolicy kPhasedPolicy = {true, false, true, false, true, true};
 constexpr CachePolicy kPipelinedPolicy = {true, true, false, true, true, true};
 // Lists whose whole working set fits in the cache (a few million elements) are better off cached.
 constexpr CachePolicy kResidentPolicy = {false, false, false, false, false, false};
-
-template <bool kNT, typename T>
-__device__ __forceinline__ T ldg(const RAFHIP_GLOBAL T* p) {
-  if constexpr (kNT)
-    return __builtin_nontemporal_load(p);
-  else
-    return *p;
-}
-template <bool kNT, typename T>
-__device__ __forceinline__ void stg(RAFHIP_GLOBAL T* p, T v) {
-  if constexpr (kNT)
-    __builtin_nontemporal_store(v, p);
-  else
-    *p = v;
-}
-
-// ------------------------------------------------------------------ gradient ingest
-// Gradients as fp32, already multiplied by the unscale factor (one fp32 rounding, exact for
-// power-of-two loss scales).
-template <typename G>
-struct GradIO;
-
-template <>
-struct GradIO<float> {
-  // Widest single-lane access used when the gradient is the only array read (pass A): 16 bytes.
-  static constexpr int kWide = 4;
-  template <bool kNT>
-  static __device__ __forceinline__ void load_wide(const void* g, int iw, float us,
-                                                   float (&out)[kWide]) {
-    const f32x4 r = ldg<kNT>((gc_float4*)g + iw);
-    out[0] = r.x * us;
-    out[1] = r.y * us;
-    out[2] = r.z * us;
-    out[3] = r.w * us;
-  }
-  template <bool kNT>
-  static __device__ __forceinline__ f32x4 load4(const void* g, int i4, float us) {
-    const f32x4 r = ldg<kNT>((gc_float4*)g + i4);
-    return f32x4{r.x * us, r.y * us, r.z * us, r.w * us};
-  }
-  static __device__ __forceinline__ float load1(const void* g, int i, float us) {
-    return ((gc_float*)g)[i] * us;
-  }
-};
-
-template <>
-struct GradIO<_Float16> {
-  static constexpr int kWide = 8;
-  template <bool kNT>
-  static __device__ __forceinline__ void load_wide(const void* g, int iw, float us,
-                                                   float (&out)[kWide]) {
-    const half8_t r = ldg<kNT>((gc_half8*)g + iw);
-#pragma unroll
-    for (int j = 0; j < kWide; ++j) out[j] = (float)r[j] * us;
-  }
-  template <bool kNT>
-  static __device__ __forceinline__ f32x4 load4(const void* g, int i4, float us) {
-    const half4_t r = ldg<kNT>((gc_half4*)g + i4);
-    return f32x4{(float)r.x * us, (float)r.y * us, (float)r.z * us, (float)r.w * us};
-  }
-  static __device__ __forceinline__ float load1(const void* g, int i, float us) {
-    return (float)((gc_half*)g)[i] * us;
-  }
-};
-
-template <>
-struct GradIO<Bf16> {
-  static constexpr int kWide = 8;
-  // bfloat16 is the upper half of the fp32 word: widening is a shift.
-  static __device__ __forceinline__ float widen(unsigned short b) {
-    return __uint_as_float((unsigned)b << 16);
-  }
-  template <bool kNT>
-  static __device__ __forceinline__ void load_wide(const void* g, int iw, float us,
-                                                   float (&out)[kWide]) {
-    const u16x8 r = ldg<kNT>((gc_u16x8*)g + iw);
-#pragma unroll
-    for (int j = 0; j < kWide; ++j) out[j] = widen(r[j]) * us;
-  }
-  template <bool kNT>
-  static __device__ __forceinline__ f32x4 load4(const void* g, int i4, float us) {
-    const u16x4 r = ldg<kNT>((gc_u16x4*)g + i4);
-    return f32x4{widen(r.x) * us, widen(r.y) * us, widen(r.z) * us, widen(r.w) * us};
-  }
-  static __device__ __forceinline__ float load1(const void* g, int i, float us) {
-    return widen(((gc_u16*)g)[i]) * us;
-  }
-};
-
-// ------------------------------------------------------------------ 16-bit weight copy
-// The stored fp32 weight narrowed with round to nearest even: binary16 by the hardware conversion,
-// bfloat16 by add-and-shift on the bit pattern (NaN stays a quiet NaN).
-__device__ __forceinline__ unsigned short narrow16(float x, bool bf16) {
-  if (bf16) {
-    const unsigned u = __float_as_uint(x);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x0040u);
-    return (unsigned short)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
-  }
-  const _Float16 h = (_Float16)x;
-  return __builtin_bit_cast(unsigned short, h);
-}
 
 // ------------------------------------------------------------------ reductions
 // Sum over the 64 lanes of a wavefront; the total is valid in lane 0.  Fixed butterfly order.

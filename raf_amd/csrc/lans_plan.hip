@@ -12,6 +12,7 @@
 #include <new>
 #include <vector>
 
+#include "device_table.h"
 #include "lans_kernels.h"
 #include "status.h"
 
@@ -139,12 +140,7 @@ struct rafhip_lans_plan {
   WorkItem* d_pipeline = nullptr;
   uint64_t* d_trace = nullptr;  // diagnostics, only with RAFHIP_LANS_TRACE=1
 
-  // Tensor-table upload: pinned staging + the records last sent, so a step whose pointers did not
-  // move sends nothing.
-  TensorRec* h_staging = nullptr;
-  std::vector<TensorRec> last_sent;
-  bool sent_once = false;
-  hipEvent_t staging_free = nullptr;  // recorded after the last upload was enqueued
+  RecordUploader<TensorRec> tensors;  // a step whose pointers did not move sends nothing
 
   // Optional per-kernel timing: slots x 6 events.
   std::vector<std::array<hipEvent_t, 6>> timing;
@@ -163,8 +159,7 @@ void destroy_timing(rafhip_lans_plan* p) {
 void free_plan(rafhip_lans_plan* p) {
   if (!p) return;
   destroy_timing(p);
-  if (p->staging_free) (void)hipEventDestroy(p->staging_free);
-  if (p->h_staging) (void)hipHostFree(p->h_staging);
+  p->tensors.release();
   if (p->d_tables) (void)hipFree(p->d_tables);
   if (p->d_trace) (void)hipFree(p->d_trace);
   delete p;
@@ -311,9 +306,7 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
     hipError_t e =
         hipMalloc(&p->d_tables, tensors_bytes + phased_bytes + pipe_bytes + a_bytes + kAlign);
     if (e == hipSuccess)
-      e = hipHostMalloc(reinterpret_cast<void**>(&p->h_staging),
-                        sizeof(TensorRec) * (size_t)n_tensors, hipHostMallocDefault);
-    if (e == hipSuccess) e = hipEventCreateWithFlags(&p->staging_free, hipEventDisableTiming);
+      e = p->tensors.init(static_cast<TensorRec*>(p->d_tables), (size_t)n_tensors);
     if (e != hipSuccess) {
       free_plan(p);
       return fail(RAFHIP_ERR_HIP, "rafhip_lans_plan_create: allocation failed: %s",
@@ -435,18 +428,7 @@ int rafhip_lans_step_mixed(rafhip_lans_plan* plan, const void* const* g, float* 
   }
 
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const size_t table_bytes = sizeof(TensorRec) * (size_t)n;
-  if (!plan->sent_once ||
-      std::memcmp(plan->last_sent.data(), recs.data(), table_bytes) != 0) {
-    // The previous upload may still be reading the staging buffer.
-    if (plan->sent_once) RAFHIP_HIP_TRY(hipEventSynchronize(plan->staging_free));
-    std::memcpy(plan->h_staging, recs.data(), table_bytes);
-    RAFHIP_HIP_TRY(hipMemcpyAsync(plan->d_tensors, plan->h_staging, table_bytes,
-                                  hipMemcpyHostToDevice, s));
-    RAFHIP_HIP_TRY(hipEventRecord(plan->staging_free, s));
-    plan->last_sent.swap(recs);
-    plan->sent_once = true;
-  }
+  RAFHIP_HIP_TRY(plan->tensors.sync(recs, s));
 
   char* ws = static_cast<char*>(workspace);
   LansDeviceArgs a;

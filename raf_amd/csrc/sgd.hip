@@ -13,16 +13,24 @@
 // walking the tensor with a grid stride, so consecutive wavefronts touch consecutive 1 KiB lines.
 #include <hip/hip_runtime.h>
 
+//
+// The multi-tensor step further down applies the same four operations, in place, to a whole list
+// of parameters in ONE launch; it stands in for what the reference's traced optimizer emits per
+// parameter -- cast(dx), multiply, add(out=v), multiply, subtract(out=w), cast, add(out=p)
+// (python/raf/optim/sgd.py:187-215) -- and for the one-op-call-per-parameter loop of its imperative
+// optimizer (sgd.py:51-58).
 #include <cstdint>
+#include <new>
+#include <vector>
 
+#include "device_table.h"
+#include "half_types.h"
 #include "status.h"
 
 #pragma clang fp contract(off)
 
 namespace rafhip {
 namespace {
-
-typedef float f32x4 __attribute__((ext_vector_type(4)));  // native vector (HIP's float4 is a class)
 
 constexpr int kSgdBlock = 256;
 constexpr int kSgdUnroll = 2;  // float4 groups in flight per lane per trip
@@ -84,19 +92,96 @@ __global__ __launch_bounds__(kSgdBlock) void sgd_scalar_kernel(
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-int grid_cap() {
-  // Enough resident wavefronts to cover HBM latency on every CU; the grid-stride loop does the rest.
-  static int cap = [] {
-    int dev = 0, cus = 256;
-    if (hipGetDevice(&dev) == hipSuccess) {
-      int v = 0;
-      if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
-          v > 0)
-        cus = v;
+// ------------------------------------------------------------------ multi-tensor, in place
+constexpr int kSgdChunk = 4096;  // elements per work item
+
+struct SgdRec {  // 48 bytes, one per parameter
+  float* x;      // fp32 (master) weight, updated in place
+  const void* dx;  // gradient: fp32, binary16 or bfloat16
+  float* v;      // fp32 velocity, updated in place
+  void* p;       // optional 16-bit copy of the new weight (the model's parameter) or null
+  int64_t numel;
+  int32_t vec_ok;  // every pointer aligned for 4-element lane accesses
+  int32_t reserved;
+};
+
+struct SgdItem {
+  int32_t tensor;
+  int32_t chunk;
+};
+
+template <typename G, bool kNT>
+__global__ __launch_bounds__(kSgdBlock) void sgd_multi_kernel(const SgdRec* recs,
+                                                              const SgdItem* items,
+                                                              int64_t n_items, float lr, float mu,
+                                                              int p_is_bf16) {
+  for (int64_t it = blockIdx.x; it < n_items; it += gridDim.x) {
+    const SgdItem item = items[it];
+    const SgdRec r = recs[item.tensor];
+    const int64_t begin = (int64_t)item.chunk * kSgdChunk;
+    const int64_t rest = r.numel - begin;
+    const int len = rest < kSgdChunk ? (int)rest : kSgdChunk;
+    float* x = r.x + begin;
+    float* v = r.v + begin;
+    const char* dx = static_cast<const char*>(r.dx) + begin * (int64_t)sizeof(G);
+    unsigned short* p = r.p ? static_cast<unsigned short*>(r.p) + begin : nullptr;
+    int done = 0;
+    if (r.vec_ok) {
+      const int n4 = len >> 2;
+      RAFHIP_GLOBAL f32x4* x4 = (RAFHIP_GLOBAL f32x4*)x;
+      RAFHIP_GLOBAL f32x4* v4 = (RAFHIP_GLOBAL f32x4*)v;
+      for (int i0 = threadIdx.x; i0 < n4; i0 += kSgdBlock * kSgdUnroll) {
+        f32x4 rx[kSgdUnroll], rd[kSgdUnroll], rv[kSgdUnroll];
+#pragma unroll
+        for (int u = 0; u < kSgdUnroll; ++u) {
+          const int i = i0 + u * kSgdBlock;
+          if (i < n4) {
+            rx[u] = ldg<kNT>((const RAFHIP_GLOBAL f32x4*)x4 + i);
+            rd[u] = GradIO<G>::template load4<kNT>(dx, i, 1.0f);  // exact widening, no scaling
+            rv[u] = ldg<kNT>((const RAFHIP_GLOBAL f32x4*)v4 + i);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < kSgdUnroll; ++u) {
+          const int i = i0 + u * kSgdBlock;
+          if (i < n4) {
+            float v1[4], x1[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) sgd_elem(rx[u][j], rd[u][j], rv[u][j], lr, mu, v1[j], x1[j]);
+            stg<kNT>(v4 + i, f32x4{v1[0], v1[1], v1[2], v1[3]});
+            stg<kNT>(x4 + i, f32x4{x1[0], x1[1], x1[2], x1[3]});
+            if (p)  // uniform over the workgroup
+              stg<kNT>((RAFHIP_GLOBAL u16x4*)p + i,
+                       u16x4{narrow16(x1[0], p_is_bf16 != 0), narrow16(x1[1], p_is_bf16 != 0),
+                             narrow16(x1[2], p_is_bf16 != 0), narrow16(x1[3], p_is_bf16 != 0)});
+          }
+        }
+      }
+      done = n4 << 2;
     }
-    return cus * 8;
-  }();
-  return cap;
+    for (int i = done + (int)threadIdx.x; i < len; i += kSgdBlock) {
+      float nv, nx;
+      sgd_elem(x[i], GradIO<G>::load1(dx, i, 1.0f), v[i], lr, mu, nv, nx);
+      v[i] = nv;
+      x[i] = nx;
+      if (p) p[i] = narrow16(nx, p_is_bf16 != 0);
+    }
+  }
+}
+
+// A list whose x, dx, v total less than this sits in the 256 MB Infinity Cache between steps and
+// is better off cached; larger ones stream with the non-temporal hint.
+constexpr int64_t kSgdStreamFromBytes = 160LL << 20;
+
+template <typename G>
+void launch_sgd_multi(bool stream_nt, unsigned grid, hipStream_t s, const SgdRec* recs,
+                      const SgdItem* items, int64_t n_items, float lr, float mu, int p_is_bf16) {
+  if (stream_nt)
+    hipLaunchKernelGGL((sgd_multi_kernel<G, true>), dim3(grid), dim3(kSgdBlock), 0, s, recs, items,
+                       n_items, lr, mu, p_is_bf16);
+  else
+    hipLaunchKernelGGL((sgd_multi_kernel<G, false>), dim3(grid), dim3(kSgdBlock), 0, s, recs, items,
+                       n_items, lr, mu, p_is_bf16);
 }
 
 }  // namespace
@@ -115,7 +200,7 @@ extern "C" int rafhip_sgd_f32(const float* x, const float* dx, const float* v, f
   const float lr32 = static_cast<float>(learning_rate);
   const float mu32 = static_cast<float>(mu);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int cap = grid_cap();
+  const int cap = streaming_grid_cap();
 
   const bool vec = aligned16(x) && aligned16(dx) && aligned16(v) && aligned16(v_out) &&
                    aligned16(x_out);
@@ -140,5 +225,138 @@ extern "C" int rafhip_sgd_f32(const float* x, const float* dx, const float* v, f
                        v_out, x_out, done, n, lr32, mu32);
     RAFHIP_HIP_TRY(hipGetLastError());
   }
+  return RAFHIP_OK;
+}
+
+// ------------------------------------------------------------------ multi-tensor plan + entry
+struct rafhip_sgd_plan {
+  int32_t n = 0;
+  int32_t grad_dtype = RAFHIP_F32;
+  std::vector<int64_t> numel;
+  int64_t total_elements = 0;
+  int64_t n_items = 0;
+  void* d_tables = nullptr;
+  rafhip::SgdRec* d_recs = nullptr;
+  rafhip::SgdItem* d_items = nullptr;
+  rafhip::RecordUploader<rafhip::SgdRec> recs;
+};
+
+namespace {
+void free_sgd_plan(rafhip_sgd_plan* p) {
+  if (!p) return;
+  p->recs.release();
+  if (p->d_tables) (void)hipFree(p->d_tables);
+  delete p;
+}
+inline bool aligned_to(const void* p, uintptr_t a) {
+  return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0;
+}
+}  // namespace
+
+extern "C" int rafhip_sgd_plan_create(int32_t n_tensors, const int64_t* numel, int32_t grad_dtype,
+                                      rafhip_sgd_plan** out_plan) {
+  using namespace rafhip;
+  clear_error();
+  if (!out_plan) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_sgd_plan_create: out_plan is NULL");
+  *out_plan = nullptr;
+  if (n_tensors < 0 || (n_tensors > 0 && !numel))
+    return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_sgd_plan_create: bad tensor list");
+  if (grad_dtype != RAFHIP_F32 && grad_dtype != RAFHIP_F16 && grad_dtype != RAFHIP_BF16)
+    return fail(RAFHIP_ERR_UNSUPPORTED,
+                "rafhip_sgd_plan_create: gradient dtype %d (fp32, fp16 or bf16)", grad_dtype);
+  rafhip_sgd_plan* p = new (std::nothrow) rafhip_sgd_plan();
+  if (!p) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_sgd_plan_create: out of host memory");
+  p->n = n_tensors;
+  p->grad_dtype = grad_dtype;
+  std::vector<SgdItem> items;
+  for (int32_t t = 0; t < n_tensors; ++t) {
+    if (numel[t] < 0) {
+      free_sgd_plan(p);
+      return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_sgd_plan_create: numel[%d] = %lld < 0", t,
+                  (long long)numel[t]);
+    }
+    const int64_t chunks = (numel[t] + kSgdChunk - 1) / kSgdChunk;
+    if (chunks > INT32_MAX) {
+      free_sgd_plan(p);
+      return fail(RAFHIP_ERR_UNSUPPORTED, "rafhip_sgd_plan_create: tensor %d is too large", t);
+    }
+    p->numel.push_back(numel[t]);
+    p->total_elements += numel[t];
+    for (int64_t c = 0; c < chunks; ++c) items.push_back(SgdItem{t, (int32_t)c});
+  }
+  p->n_items = (int64_t)items.size();
+  if (p->n_items == 0) {  // nothing to update: valid, nothing to launch
+    *out_plan = p;
+    return RAFHIP_OK;
+  }
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    free_sgd_plan(p);
+    return fail(RAFHIP_ERR_NO_DEVICE, "rafhip_sgd_plan_create: no HIP device available");
+  }
+  const size_t rec_bytes = (sizeof(SgdRec) * (size_t)n_tensors + 255) / 256 * 256;
+  hipError_t e = hipMalloc(&p->d_tables, rec_bytes + sizeof(SgdItem) * items.size());
+  if (e == hipSuccess) {
+    p->d_recs = static_cast<SgdRec*>(p->d_tables);
+    p->d_items = reinterpret_cast<SgdItem*>(static_cast<char*>(p->d_tables) + rec_bytes);
+    e = p->recs.init(p->d_recs, (size_t)n_tensors);
+  }
+  if (e == hipSuccess)
+    e = hipMemcpy(p->d_items, items.data(), sizeof(SgdItem) * items.size(), hipMemcpyHostToDevice);
+  if (e != hipSuccess) {
+    free_sgd_plan(p);
+    return fail(RAFHIP_ERR_HIP, "rafhip_sgd_plan_create: %s", hipGetErrorString(e));
+  }
+  *out_plan = p;
+  return RAFHIP_OK;
+}
+
+extern "C" int rafhip_sgd_plan_destroy(rafhip_sgd_plan* plan) {
+  rafhip::clear_error();
+  free_sgd_plan(plan);
+  return RAFHIP_OK;
+}
+
+extern "C" int rafhip_sgd_multi_step(rafhip_sgd_plan* plan, float* const* x, const void* const* dx,
+                                     float* const* v, void* const* p, int32_t p_dtype,
+                                     double learning_rate, double mu, void* stream) {
+  using namespace rafhip;
+  clear_error();
+  if (!plan) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_sgd_multi_step: plan is NULL");
+  if (p && p_dtype != RAFHIP_F16 && p_dtype != RAFHIP_BF16)
+    return fail(RAFHIP_ERR_UNSUPPORTED,
+                "rafhip_sgd_multi_step: weight-copy dtype %d (binary16 or bfloat16)", p_dtype);
+  if (plan->n_items == 0) return RAFHIP_OK;
+  if (!x || !dx || !v) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_sgd_multi_step: null pointer list");
+  const uintptr_t g_elem = plan->grad_dtype == RAFHIP_F32 ? 4 : 2;
+  std::vector<SgdRec> recs((size_t)plan->n);
+  for (int32_t t = 0; t < plan->n; ++t) {
+    SgdRec& r = recs[t];
+    r = SgdRec{x[t], dx[t], v[t], p ? p[t] : nullptr, plan->numel[t], 0, 0};
+    if (r.numel == 0) continue;
+    if (!r.x || !r.dx || !r.v)
+      return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_sgd_multi_step: tensor %d has a null data pointer", t);
+    if (!aligned_to(r.x, 4) || !aligned_to(r.v, 4) || !aligned_to(r.dx, g_elem) || !aligned_to(r.p, 2))
+      return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_sgd_multi_step: tensor %d is not element-aligned", t);
+    r.vec_ok = aligned_to(r.x, 16) && aligned_to(r.v, 16) && aligned_to(r.dx, 4 * g_elem) &&
+               aligned_to(r.p, 8);
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  RAFHIP_HIP_TRY(plan->recs.sync(recs, s));
+  // One rounding double -> fp32, as for the single-tensor op.
+  const float lr32 = static_cast<float>(learning_rate);
+  const float mu32 = static_cast<float>(mu);
+  const int64_t cap = streaming_grid_cap();
+  const unsigned grid = (unsigned)(plan->n_items < cap ? plan->n_items : cap);
+  const bool nt = plan->total_elements * (int64_t)(8 + g_elem) > kSgdStreamFromBytes;
+  const int bf = p_dtype == RAFHIP_BF16 ? 1 : 0;
+  if (plan->grad_dtype == RAFHIP_F16)
+    launch_sgd_multi<_Float16>(nt, grid, s, plan->d_recs, plan->d_items, plan->n_items, lr32, mu32, bf);
+  else if (plan->grad_dtype == RAFHIP_BF16)
+    launch_sgd_multi<Bf16>(nt, grid, s, plan->d_recs, plan->d_items, plan->n_items, lr32, mu32, bf);
+  else
+    launch_sgd_multi<float>(nt, grid, s, plan->d_recs, plan->d_items, plan->n_items, lr32, mu32, bf);
+  RAFHIP_HIP_TRY(hipGetLastError());
   return RAFHIP_OK;
 }

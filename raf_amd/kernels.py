@@ -43,6 +43,66 @@ def sgd_f32(x: torch.Tensor, dx: torch.Tensor, v: torch.Tensor, learning_rate: f
     return v1, x1
 
 
+_DTYPE_CODE = {torch.float32: RAFHIP_F32, torch.float16: RAFHIP_F16, torch.bfloat16: RAFHIP_BF16}
+
+
+class SgdPlan:
+    """Owns a ``rafhip_sgd_plan``: momentum SGD over a whole parameter list, in place, one launch."""
+
+    def __init__(self, numels: Sequence[int], grad_dtype=torch.float32, device="cuda:0"):
+        self._h = c_void_p(None)
+        self.lib = _lib.optim()
+        self.device = torch.device(device)
+        self.numels = [int(n) for n in numels]
+        self.n = len(self.numels)
+        if grad_dtype not in _DTYPE_CODE:
+            raise TypeError(f"SGD gradients must be float32, float16 or bfloat16, got {grad_dtype}")
+        self.grad_dtype = grad_dtype
+        arr = (c_int64 * max(self.n, 1))(*self.numels)
+        with torch.cuda.device(self.device):
+            check(self.lib.rafhip_sgd_plan_create(self.n, arr, _DTYPE_CODE[grad_dtype], ctypes.byref(self._h)))
+
+    def close(self):
+        if self._h:
+            self.lib.rafhip_sgd_plan_destroy(self._h)
+            self._h = c_void_p(None)
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:  # interpreter shutdown
+            pass
+
+    def _ptrs(self, tensors, dtype, what, optional=False):
+        if len(tensors) != self.n:
+            raise ValueError(f"{what}: expected {self.n} tensors, got {len(tensors)}")
+        arr = (c_void_p * max(self.n, 1))()
+        for i, t in enumerate(tensors):
+            if t is None and optional:
+                continue
+            if not t.is_cuda or t.dtype != dtype or not t.is_contiguous() or t.numel() != self.numels[i]:
+                raise TypeError(f"{what}[{i}]: need a contiguous {dtype} GPU tensor of {self.numels[i]} elements")
+            arr[i] = t.data_ptr()
+        return arr
+
+    def marshal(self, x, dx, v, p=None):
+        """Pointer lists for ``step``; reusable while the tensors stay where they are."""
+        pp, p_code = None, RAFHIP_F16
+        if p is not None:
+            dt = next((t.dtype for t in p if t is not None), torch.float16)
+            if dt not in (torch.float16, torch.bfloat16):
+                raise TypeError(f"16-bit weight copies must be float16 or bfloat16, got {dt}")
+            pp, p_code = self._ptrs(p, dt, "p", optional=True), _DTYPE_CODE[dt]
+        return (self._ptrs(x, torch.float32, "x"), self._ptrs(dx, self.grad_dtype, "dx"),
+                self._ptrs(v, torch.float32, "v"), pp, p_code, (list(x), list(dx), list(v), p))
+
+    def step(self, x, dx, v, learning_rate: float, mu: float, p=None, marshalled=None):
+        """x, v updated in place; ``p``: optional float16 / bfloat16 tensors receiving the new x."""
+        xp, dp, vp, pp, p_code, _ = marshalled if marshalled is not None else self.marshal(x, dx, v, p)
+        check(self.lib.rafhip_sgd_multi_step(self._h, xp, dp, vp, pp, p_code, float(learning_rate),
+                                             float(mu), _current_stream(self.device)))
+
+
 _NORM_DTYPES = {torch.float32: RAFHIP_F32, torch.float64: RAFHIP_F64, torch.float16: RAFHIP_F16,
                 torch.bfloat16: RAFHIP_BF16}
 
@@ -152,9 +212,6 @@ def pipeline_order(numels: Sequence[int], group_elements: int = 0):
     buf = (ctypes.c_int32 * max(3 * count.value, 1))()
     check(lib.rafhip_lans_pipeline_order(n, arr, group_elements, buf, count.value, ctypes.byref(count)))
     return [(buf[3 * i], buf[3 * i + 1], buf[3 * i + 2]) for i in range(count.value)]
-
-
-_DTYPE_CODE = {torch.float32: RAFHIP_F32, torch.float16: RAFHIP_F16, torch.bfloat16: RAFHIP_BF16}
 
 
 class LansPlan:

@@ -11,9 +11,16 @@ from . import op as _op
 
 
 class SGD:
-    """Stochastic gradient descent with momentum: one ``raf.op.sgd`` call per parameter."""
+    """Stochastic gradient descent with momentum.
 
-    def __init__(self, params, learning_rate, momentum=0):
+    ``multi_tensor=False`` follows the reference's imperative optimizer literally: one
+    ``raf.op.sgd`` call per parameter and a rebinding of the results (python/raf/optim/sgd.py:51-58).
+    The default updates the whole parameter list in place with one multi-tensor launch -- the same
+    four roundings per element, so the same bits -- and, for float16 / bfloat16 parameters, keeps
+    fp32 master weights and velocities the way the traced optimizer does (sgd.py:152-166,
+    :187-215)."""
+
+    def __init__(self, params, learning_rate, momentum=0, multi_tensor=True):
         if learning_rate < 0.0:
             raise ValueError("Invalid learning rate: {}".format(learning_rate))
         if momentum < 0.0:
@@ -21,20 +28,41 @@ class SGD:
         self.params = []
         self._lr = learning_rate
         self._momentum = momentum
+        params = list(params)
+        halves = {x.dtype for x in params if isinstance(x, torch.Tensor)} & {torch.float16, torch.bfloat16}
+        self.mixed = bool(halves)
+        if self.mixed and (len(halves) > 1 or any(x.dtype not in halves for x in params)):
+            raise TypeError("a half-precision model must use one 16-bit dtype for all parameters")
+        self.multi_tensor = bool(multi_tensor) or self.mixed
+        self._plans = {}
         for x in params:
             assert isinstance(x, torch.Tensor), "Only tensors can be optimized!"
-            self.params.append((x, torch.zeros_like(x)))  # velocity starts at zero (sgd.py:47-49)
+            w = x.data.float() if self.mixed else x.data  # fp32 master weight (sgd.py:152-160)
+            self.params.append((x, w, torch.zeros_like(w)))  # velocity starts at zero (sgd.py:47-49)
 
     def step(self):
         """Update the parameters with gradients."""
-        for x0, v0 in self.params:
-            if x0.grad is None:
-                continue
-            v1, x1 = _op.sgd(x0.data, x0.grad, v0, self._lr, self._momentum)
-            # the reference rebinds the arrays (x0.update(x1)); the same effect on a torch
-            # parameter is a device-to-device copy into its storage
-            x0.data.copy_(x1)
-            v0.copy_(v1)
+        live = [(x, w, v) for x, w, v in self.params if x.grad is not None]
+        if not live:
+            return
+        if not self.multi_tensor:
+            for x0, _, v0 in live:
+                v1, x1 = _op.sgd(x0.data, x0.grad, v0, self._lr, self._momentum)
+                # the reference rebinds the arrays (x0.update(x1)); the same effect on a torch
+                # parameter is a device-to-device copy into its storage
+                x0.data.copy_(x1)
+                v0.copy_(v1)
+            return
+        from . import kernels
+
+        grads = [x.grad for x, _, _ in live]
+        key = (tuple(id(x) for x, _, _ in live), grads[0].dtype)
+        plan = self._plans.get(key)
+        if plan is None:
+            plan = self._plans[key] = kernels.SgdPlan([w.numel() for _, w, _ in live], grads[0].dtype,
+                                                      live[0][1].device)
+        plan.step([w for _, w, _ in live], [g.contiguous() for g in grads], [v for _, _, v in live],
+                  self._lr, self._momentum, p=[x.data for x, _, _ in live] if self.mixed else None)
 
 
 class LANS:

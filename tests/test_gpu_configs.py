@@ -156,19 +156,39 @@ def test_optim_classes_follow_reference_semantics(native_libs):
     shapes_ = [(6, 3, 5, 5), (6,), (10, 1536), (10,)]  # the small CNN of the reference's tests
     ws = [r.normal(0, .1, s).astype(np.float32) for s in shapes_]
     # SGD: lr .1, momentum .01, 10 iterations (tests/python/optim/test_sgd.py:80-125)
+    # both the per-parameter op loop of the reference and the one-launch multi-tensor path
     params = [torch.from_numpy(a.copy()).to(DEV) for a in ws]
-    sgd = optim.SGD(params, 0.1, 0.01)
+    params_mt = [torch.from_numpy(a.copy()).to(DEV) for a in ws]
+    sgd = optim.SGD(params, 0.1, 0.01, multi_tensor=False)
+    sgd_mt = optim.SGD(params_mt, 0.1, 0.01)
     hx = [a.copy() for a in ws]
     hv = [np.zeros_like(a) for a in ws]
     for _ in range(10):
         grads = [r.normal(0, 1, s).astype(np.float32) for s in shapes_]
-        for p, gr in zip(params, grads):
+        for p, q, gr in zip(params, params_mt, grads):
             p.grad = torch.from_numpy(gr).to(DEV)
+            q.grad = torch.from_numpy(gr).to(DEV)
         sgd.step()
+        sgd_mt.step()
         for i, gr in enumerate(grads):
             hv[i], hx[i] = sgd_f32.sgd_step(hx[i], gr, hv[i], 0.1, 0.01)
-    for p, a in zip(params, hx):
-        assert np.array_equal(p.cpu().numpy(), a)
+    for p, q, a in zip(params, params_mt, hx):
+        assert np.array_equal(p.cpu().numpy(), a) and np.array_equal(q.cpu().numpy(), a)
+    # a half-precision model: fp32 master weights and velocities, parameters are their narrowing
+    from oracle import halfs
+    half = [torch.from_numpy(a.copy()).to(DEV).to(torch.bfloat16) for a in ws]
+    sgd_h = optim.SGD(half, 0.1, 0.01)
+    mx = [p.float().cpu().numpy() for p in half]
+    mv = [np.zeros_like(a) for a in mx]
+    for _ in range(3):
+        gb = [halfs.f32_to_bf16_bits(r.normal(0, 1, s).astype(np.float32)) for s in shapes_]
+        for p, g in zip(half, gb):
+            p.grad = torch.from_numpy(g.view(np.int16)).to(DEV).view(torch.bfloat16)
+        sgd_h.step()
+        mx, mv, mp = sgd_f32.sgd_list_step(mx, gb, mv, 0.1, 0.01, "bfloat16")
+    for (p, w, v), a, b, c in zip(sgd_h.params, mx, mv, mp):
+        assert np.array_equal(w.cpu().numpy(), a) and np.array_equal(v.cpu().numpy(), b)
+        assert np.array_equal(p.view(torch.int16).cpu().numpy().view(np.uint16), c.reshape(p.shape))
     # LANS: defaults, step counter starts at 1 and advances per call (lans.py:66, :103)
     params = [torch.from_numpy(a.copy()).to(DEV) for a in ws]
     lans = optim.LANS(params)

@@ -127,3 +127,26 @@ def test_c_restatement_bit_equal(c_oracle, n):
         b = c_oracle.sgd_step(x0, dx, v0, 0.01, 0.9, threads=threads)
         assert np.array_equal(a[0].view(np.uint32), b[0].view(np.uint32))
         assert np.array_equal(a[1].view(np.uint32), b[1].view(np.uint32))
+
+
+def test_list_step_is_the_op_per_parameter_with_exact_widening_and_rne_copies():
+    """The traced optimizer's per-parameter sequence (python/raf/optim/sgd.py:187-215): the same
+    four roundings as the op on the widened gradient, then cast(new_w, dtype)."""
+    import torch
+    from oracle import halfs
+
+    rng = np.random.default_rng(9)
+    xs = [rng.normal(0, 0.02, n).astype(np.float32) for n in (7, 1000)]
+    vs = [rng.normal(0, 1e-3, n).astype(np.float32) for n in (7, 1000)]
+    d32 = [rng.normal(0, 1e-3, n).astype(np.float32) for n in (7, 1000)]
+    for name, tdt, grads in (("float16", torch.float16, [d.astype(np.float16) for d in d32]),
+                             ("bfloat16", torch.bfloat16, [halfs.f32_to_bf16_bits(d) for d in d32])):
+        nx, nv, ps = sgd_f32.sgd_list_step(xs, grads, vs, 0.01, 0.9, name)
+        for x0, g, v0, x1, v1, p in zip(xs, grads, vs, nx, nv, ps):
+            wide = torch.from_numpy(g.view(np.int16)).view(tdt).float().numpy()  # torch's own widening
+            ev, ex = sgd_f32.sgd_step(x0, wide, v0, 0.01, 0.9)
+            assert np.array_equal(ev, v1) and np.array_equal(ex, x1)
+            t = torch.from_numpy(x1).to(tdt).view(torch.int16).numpy().view(np.uint16)
+            assert np.array_equal(p.view(np.uint16), t)
+    nx, nv, ps = sgd_f32.sgd_list_step(xs, d32, vs, 0.01, 0.9)
+    assert ps is None and np.array_equal(nx[1], sgd_f32.sgd_step(xs[1], d32[1], vs[1], 0.01, 0.9)[1])
