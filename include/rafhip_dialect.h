@@ -77,6 +77,16 @@ int rafhip_raf_lans_execute(rafhip_raf_env* env, int32_t list_len,
                             const rafhip_tensor_desc* tensor_list, const rafhip_tensor_desc* step,
                             void* workspace, int64_t workspace_bytes, void* stream);
 
+/* Extension ops raf.op.sgd_multi(tensor_list, learning_rate, mu) with tensor_list = x..., dx...,
+ * v... (3n descriptors) and raf.op.sgd_multi_mixed with a fourth block p... (the model's float16 /
+ * bfloat16 parameters): momentum SGD over the whole list, in place on x and v, per element the
+ * four roundings of raf.op.sgd.  No counterpart in the reference's op set; they replace the
+ * per-parameter op sequence of its traced optimizer (python/raf/optim/sgd.py:187-215). */
+int rafhip_raf_sgd_multi_make(int32_t mixed, int32_t list_len, const rafhip_tensor_desc* tensor_list,
+                              double learning_rate, double mu, rafhip_raf_env** env_out);
+int rafhip_raf_sgd_multi_execute(rafhip_raf_env* env, int32_t list_len,
+                                 const rafhip_tensor_desc* tensor_list, void* stream);
+
 /* raf.op.l2norm(x) -> 0-d tensor of x's dtype; scripts/src_codegen/def_schema.py:425-427,
  * src/op/declare/reduce.cc:118-126. */
 int rafhip_raf_l2norm_make(const rafhip_tensor_desc* x, rafhip_raf_env** env_out);

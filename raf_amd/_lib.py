@@ -132,6 +132,9 @@ DIALECT_SYMBOLS = {
                                      c_int32, POINTER(c_void_p)]),
     "rafhip_raf_lans_execute": (c_int, [c_void_p, c_int32, POINTER(TensorDesc),
                                         POINTER(TensorDesc), c_void_p, c_int64, c_void_p]),
+    "rafhip_raf_sgd_multi_make": (c_int, [c_int32, c_int32, POINTER(TensorDesc), c_double, c_double,
+                                          POINTER(c_void_p)]),
+    "rafhip_raf_sgd_multi_execute": (c_int, [c_void_p, c_int32, POINTER(TensorDesc), c_void_p]),
     "rafhip_raf_l2norm_make": (c_int, [POINTER(TensorDesc), POINTER(c_void_p)]),
     "rafhip_raf_l2norm_execute": (c_int, [c_void_p, POINTER(TensorDesc), POINTER(TensorDesc), c_void_p,
                                           c_int64, c_void_p]),

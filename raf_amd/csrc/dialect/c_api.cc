@@ -238,6 +238,39 @@ int rafhip_raf_lans_execute(rafhip_raf_env* env, int32_t list_len,
   });
 }
 
+int rafhip_raf_sgd_multi_make(int32_t mixed, int32_t list_len, const rafhip_tensor_desc* tensor_list,
+                              double learning_rate, double mu, rafhip_raf_env** env_out) {
+  return Guard([&] {
+    if (!env_out) throw Error("rafhip_raf_sgd_multi_make: env_out is NULL");
+    *env_out = nullptr;
+    if (list_len < 0 || (list_len > 0 && !tensor_list))
+      throw Error("rafhip_raf_sgd_multi_make: bad tensor list");
+    auto args = std::make_shared<schema::SgdMultiArgs>();
+    for (int32_t i = 0; i < list_len; ++i)
+      args->tensor_list.push_back(FromDesc(&tensor_list[i], "tensor_list"));
+    args->learning_rate = learning_rate;
+    args->mu = mu;
+    *env_out = Finish(MakeCall(mixed ? "raf.op.sgd_multi_mixed" : "raf.op.sgd_multi", args));
+  });
+}
+
+int rafhip_raf_sgd_multi_execute(rafhip_raf_env* env, int32_t list_len,
+                                 const rafhip_tensor_desc* tensor_list, void* stream) {
+  return Guard([&] {
+    if (!env || !env->env) throw Error("rafhip_raf_sgd_multi_execute: env is NULL");
+    if (list_len < 0 || (list_len > 0 && !tensor_list))
+      throw Error("rafhip_raf_sgd_multi_execute: bad tensor list");
+    std::vector<value::Value> fields;
+    for (int32_t i = 0; i < list_len; ++i)
+      fields.push_back(FromDesc(&tensor_list[i], "tensor_list"));
+    value::Value tuple = value::MakeTuple(fields);
+    std::vector<value::Value> inputs = {tuple};
+    OpEnv::SetStreamForAllBackends(env->call->device, stream);
+    WorkspaceBinding bind(env->env.get(), nullptr, 0);
+    env->env->Execute(inputs, tuple);  // output aliases the inputs
+  });
+}
+
 int rafhip_raf_l2norm_make(const rafhip_tensor_desc* x, rafhip_raf_env** env_out) {
   return Guard([&] {
     if (!env_out) throw Error("rafhip_raf_l2norm_make: env_out is NULL");

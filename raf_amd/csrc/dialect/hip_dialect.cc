@@ -109,6 +109,107 @@ class SgdHipEnv : public OpEnv {
   std::string name_ = TruncateName(GetUniqueName("raf.op.hip.sgd"));
 };
 
+// ---------------------------------------------------------------------- multi-tensor SGD
+// Extension ops raf.op.sgd_multi / raf.op.sgd_multi_mixed: what the reference's traced optimizer
+// emits per parameter as cast, multiply, add(out=), multiply, subtract(out=), cast, add(out=)
+// (python/raf/optim/sgd.py:187-215), as one in-place launch over the whole list.
+class SgdMultiHipEnv : public OpEnv {
+ public:
+  SgdMultiHipEnv(const CallValues& cv, bool mixed)
+      : blocks_(mixed ? 4 : 3),
+        op_(mixed ? "raf.op.hip.sgd_multi_mixed" : "raf.op.hip.sgd_multi"),
+        name_(TruncateName(GetUniqueName(op_))) {
+    const auto* args = cv->args_as<schema::SgdMultiArgs>();
+    if (!args) {
+      error_msgs.push_back(op_ + ": call does not carry SgdMultiArgs");
+      return;
+    }
+    arg_indices = {args->FieldIndex("tensor_list")};
+    learning_rate_ = args->learning_rate;
+    mu_ = args->mu;
+    const size_t total = args->tensor_list.size();
+    if (total % (size_t)blocks_ != 0) {
+      error_msgs.push_back(op_ + ": tensor_list must hold " + std::to_string(blocks_) + "n tensors");
+      return;
+    }
+    n_ = (int32_t)(total / (size_t)blocks_);
+    if (cv->device.device_type() != DevType::kROCM()) error_msgs.push_back(op_ + ": device is not rocm");
+    int32_t grad_dtype = RAFHIP_F32;
+    std::vector<int64_t> numels;
+    for (int32_t i = 0; i < n_ && error_msgs.empty(); ++i) {
+      const TensorView& x = args->tensor_list[i]->tensor;
+      const TensorView& dx = args->tensor_list[n_ + i]->tensor;
+      const TensorView& v = args->tensor_list[2 * n_ + i]->tensor;
+      if (!IsF32(x.dtype) || !IsF32(v.dtype))
+        error_msgs.push_back(op_ + ": weights and velocities must be float32");
+      const int32_t gd = KernelDType(dx.dtype);
+      if (gd < 0 || (i > 0 && gd != grad_dtype))
+        error_msgs.push_back(op_ + ": gradients must all be float32, all float16 or all bfloat16");
+      grad_dtype = gd;
+      if (blocks_ == 4) {
+        const int32_t pd = KernelDType(args->tensor_list[3 * n_ + i]->tensor.dtype);
+        if (pd != RAFHIP_F16 && pd != RAFHIP_BF16)
+          error_msgs.push_back(op_ + ": model parameters must be float16 or bfloat16");
+        else if (i > 0 && pd != copy_dtype_)
+          error_msgs.push_back(op_ + ": model parameters must share one dtype");
+        copy_dtype_ = pd;
+      }
+      numels.push_back(x.numel());
+    }
+    if (!error_msgs.empty()) return;
+    if (rafhip_device_count() <= 0) {
+      error_msgs.push_back(op_ + ": no HIP device is visible");
+      return;
+    }
+    int st = rafhip_sgd_plan_create(n_, numels.data(), grad_dtype, &plan_);
+    if (st != RAFHIP_OK) error_msgs.push_back(KernelError("rafhip_sgd_plan_create", st));
+  }
+
+  ~SgdMultiHipEnv() override {
+    if (plan_) rafhip_sgd_plan_destroy(plan_);
+  }
+
+  std::string name() const override { return name_; }
+
+  void Execute(const CallValues& cv) override {
+    const auto* args = cv->args_as<schema::SgdMultiArgs>();
+    RAF_CHECK(args != nullptr, op_ + " expects SgdMultiArgs");
+    std::vector<Value> fields(args->tensor_list.begin(), args->tensor_list.end());
+    Execute(std::vector<Value>{value::MakeTuple(std::move(fields))}, cv->out);
+  }
+
+  void Execute(const std::vector<Value>& inputs, Value output) override {
+    (void)output;  // aliases the inputs: the update is in place
+    RAF_CHECK(inputs.size() == 1, op_ + " takes (tensor_list)");
+    auto tuple = AsTuple(inputs[0]);
+    RAF_CHECK((int64_t)tuple->fields.size() == (int64_t)blocks_ * (int64_t)n_,
+              op_ + ": tensor_list length changed since the OpEnv was made");
+    std::vector<void*> ptrs(tuple->fields.size());
+    for (size_t i = 0; i < ptrs.size(); ++i) ptrs[i] = AsTensor(tuple->fields[i])->tensor.data;
+    void** p = ptrs.data();
+    void* stream = DeviceAPI::Get(DevType::kROCM())->GetStream();
+    int st = rafhip_sgd_multi_step(plan_, reinterpret_cast<float* const*>(p),
+                                   reinterpret_cast<const void* const*>(p + n_),
+                                   reinterpret_cast<float* const*>(p + 2 * n_),
+                                   blocks_ == 4 ? p + 3 * n_ : nullptr, copy_dtype_, learning_rate_,
+                                   mu_, stream);
+    if (st != RAFHIP_OK) throw Error(KernelError("rafhip_sgd_multi_step", st));
+  }
+
+  static OpEnv* make(const CallValues& cv) { return new SgdMultiHipEnv(cv, false); }
+  static OpEnv* make_mixed(const CallValues& cv) { return new SgdMultiHipEnv(cv, true); }
+
+ private:
+  int blocks_;
+  std::string op_;
+  std::string name_;
+  double learning_rate_ = 0.0;
+  double mu_ = 0.0;
+  int32_t n_ = 0;
+  int32_t copy_dtype_ = RAFHIP_F16;
+  rafhip_sgd_plan* plan_ = nullptr;
+};
+
 // ---------------------------------------------------------------------------------------- LANS
 // One class serves raf.op.lans (tensor_list = g, w, m, v blocks) and the extension op
 // raf.op.lans_mixed (a fifth block p: the model's float16 / bfloat16 parameters, which receive the
@@ -399,6 +500,10 @@ RAF_REGISTER_DIALECT_OP(hip, lans_mixed, 30);
 RAF_OP_ENV_MAKER("raf.op.hip.lans_mixed", LansHipEnv::make_mixed);
 RAF_REGISTER_DIALECT_OP(hip, sgd, 30);
 RAF_OP_ENV_MAKER("raf.op.hip.sgd", SgdHipEnv::make);
+RAF_REGISTER_DIALECT_OP(hip, sgd_multi, 30);
+RAF_OP_ENV_MAKER("raf.op.hip.sgd_multi", SgdMultiHipEnv::make);
+RAF_REGISTER_DIALECT_OP(hip, sgd_multi_mixed, 30);
+RAF_OP_ENV_MAKER("raf.op.hip.sgd_multi_mixed", SgdMultiHipEnv::make_mixed);
 // cublas l2norm is plevel 15, tvm 10; cuda fuse_tensor / defuse_tensor are plevel 10.
 RAF_REGISTER_DIALECT_OP(hip, l2norm, 30);
 RAF_OP_ENV_MAKER("raf.op.hip.l2norm", L2NormHipEnv::make);

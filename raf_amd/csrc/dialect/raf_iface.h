@@ -164,6 +164,15 @@ struct LansArgs : ArgsBase {  // def_schema.py:678-694
   int FieldIndex(const std::string& name) const override;
 };
 
+// Extension ops raf.op.sgd_multi / raf.op.sgd_multi_mixed: momentum SGD over a parameter list in
+// place.  tensor_list = [x..., dx..., v...] (+ [p...], the model's 16-bit parameters, for _mixed).
+struct SgdMultiArgs : ArgsBase {
+  std::vector<value::TensorValue> tensor_list;
+  double learning_rate = 0.0;
+  double mu = 0.0;
+  int FieldIndex(const std::string& name) const override;
+};
+
 struct L2NormArgs : ArgsBase {  // def_schema.py:425-427
   value::TensorValue x;
   int FieldIndex(const std::string& name) const override;

@@ -84,6 +84,11 @@ int LansArgs::FieldIndex(const std::string& name) const {
   return IndexIn(kNames, 11, name);
 }
 
+int SgdMultiArgs::FieldIndex(const std::string& name) const {
+  static const char* const kNames[] = {"tensor_list", "learning_rate", "mu"};
+  return IndexIn(kNames, 3, name);
+}
+
 int L2NormArgs::FieldIndex(const std::string& name) const {
   static const char* const kNames[] = {"x"};
   return IndexIn(kNames, 1, name);
@@ -165,6 +170,27 @@ void LansMixedDecl(const CallValues& call) {
   call->out = value::MakeTuple(std::move(out));
 }
 
+// Extension ops raf.op.sgd_multi (3n tensors: x, dx, v) and raf.op.sgd_multi_mixed (4n: and the
+// 16-bit model parameters): in place like raf.op.lans, so the output tuple is the input values.
+void SgdMultiDecl(const CallValues& call, size_t blocks) {
+  const auto* args = call->args_as<schema::SgdMultiArgs>();
+  RAF_CHECK(args != nullptr, "raf.op.sgd_multi expects SgdMultiArgs");
+  RAF_CHECK(args->tensor_list.size() % blocks == 0,
+            "tensor_list must hold " + std::to_string(blocks) + "n tensors");
+  const size_t n = args->tensor_list.size() / blocks;
+  std::vector<value::Value> out;
+  for (const auto& t : args->tensor_list) {
+    RAF_CHECK(t != nullptr, "tensor_list holds a null tensor");
+    out.push_back(t);
+  }
+  for (size_t i = 0; i < n; ++i)  // x, dx, v (and p) of one parameter agree in shape
+    for (size_t b = 1; b < blocks; ++b)
+      RAF_CHECK(args->tensor_list[b * n + i]->tensor.shape == args->tensor_list[i]->tensor.shape,
+                "tensors of one parameter differ in shape");
+  if (!args->tensor_list.empty()) call->device = args->tensor_list[0]->tensor.device;
+  call->out = value::MakeTuple(std::move(out));
+}
+
 // src/op/declare/reduce.cc:118-124: a 0-d output of x's dtype on x's device.
 void L2NormDecl(const CallValues& call) {
   const auto* args = call->args_as<schema::L2NormArgs>();
@@ -236,6 +262,8 @@ void RunDeclare(const CallValues& call) {
   if (op == "raf.op.sgd") return SgdDecl(call);
   if (op == "raf.op.lans") return LansDecl(call);
   if (op == "raf.op.lans_mixed") return LansMixedDecl(call);
+  if (op == "raf.op.sgd_multi") return SgdMultiDecl(call, 3);
+  if (op == "raf.op.sgd_multi_mixed") return SgdMultiDecl(call, 4);
   if (op == "raf.op.l2norm") return L2NormDecl(call);
   if (op == "raf.op.fuse_tensor") return FuseTensorDecl(call);
   if (op == "raf.op.defuse_tensor") return DefuseTensorDecl(call);

@@ -94,6 +94,36 @@ def sgd(x, dx, v, learning_rate, mu):
     return v1, x1
 
 
+def sgd_multi(tensor_list: Sequence[torch.Tensor], learning_rate, mu):
+    """Extension op: momentum SGD over a parameter list ``[x..., dx..., v...]`` in place (x and v
+    are updated, the list is returned), one launch; per element the four roundings of ``sgd``."""
+    return _sgd_multi(False, tensor_list, learning_rate, mu)
+
+
+def sgd_multi_mixed(tensor_list: Sequence[torch.Tensor], learning_rate, mu):
+    """Extension op for half-precision models: ``[x..., dx..., v..., p...]`` with fp32 master weights
+    ``x``, gradients of the model's dtype and the model's float16 / bfloat16 parameters ``p``, which
+    receive the new weights narrowed to 16 bits (python/raf/optim/sgd.py:187-215 in one op)."""
+    return _sgd_multi(True, tensor_list, learning_rate, mu)
+
+
+def _sgd_multi(mixed, tensor_list, learning_rate, mu):
+    lib = _lib.dialect()
+    tensor_list = list(tensor_list)
+    keep: list = []
+    n = len(tensor_list)
+    descs = (TensorDesc * max(n, 1))(*[_desc(t, keep) for t in tensor_list])
+    key = ("sgd_multi", mixed, tuple(_sig(t) for t in tensor_list), float(learning_rate), float(mu))
+    env = _env_cache.get(key)
+    if env is None:
+        h = c_void_p(None)
+        check_raf(lib.rafhip_raf_sgd_multi_make(int(mixed), n, descs, float(learning_rate), float(mu),
+                                                ctypes.byref(h)))
+        env = _env_cache[key] = _Env(h)
+    check_raf(lib.rafhip_raf_sgd_multi_execute(env.handle, n, descs, _stream(tensor_list[0]) if n else None))
+    return tensor_list
+
+
 def lans(tensor_list: Sequence[torch.Tensor], step: torch.Tensor, learning_rate, beta1, beta2, eps,
          bias_correction, weight_decay, grad_averaging, mode, normalize_grad):
     """``raf._op.imp.lans(...)``: updates the w, m, v quarters of ``tensor_list`` in place and

@@ -34,7 +34,6 @@ class SGD:
         if self.mixed and (len(halves) > 1 or any(x.dtype not in halves for x in params)):
             raise TypeError("a half-precision model must use one 16-bit dtype for all parameters")
         self.multi_tensor = bool(multi_tensor) or self.mixed
-        self._plans = {}
         for x in params:
             assert isinstance(x, torch.Tensor), "Only tensors can be optimized!"
             w = x.data.float() if self.mixed else x.data  # fp32 master weight (sgd.py:152-160)
@@ -53,16 +52,11 @@ class SGD:
                 x0.data.copy_(x1)
                 v0.copy_(v1)
             return
-        from . import kernels
-
-        grads = [x.grad for x, _, _ in live]
-        key = (tuple(id(x) for x, _, _ in live), grads[0].dtype)
-        plan = self._plans.get(key)
-        if plan is None:
-            plan = self._plans[key] = kernels.SgdPlan([w.numel() for _, w, _ in live], grads[0].dtype,
-                                                      live[0][1].device)
-        plan.step([w for _, w, _ in live], [g.contiguous() for g in grads], [v for _, _, v in live],
-                  self._lr, self._momentum, p=[x.data for x, _, _ in live] if self.mixed else None)
+        tensor_list = [w for _, w, _ in live] + [x.grad for x, _, _ in live] + [v for _, _, v in live]
+        if self.mixed:
+            _op.sgd_multi_mixed(tensor_list + [x.data for x, _, _ in live], self._lr, self._momentum)
+        else:
+            _op.sgd_multi(tensor_list, self._lr, self._momentum)
 
 
 class LANS:

@@ -113,3 +113,28 @@ def test_multi_tensor_sgd_errors_and_empty(native_libs):
         kernels.SgdPlan([8], torch.float64, DEV)
     with pytest.raises(ValueError):
         plan.step(f + f, [f[0].half()], f, 0.1, 0.9)
+
+
+def test_sgd_multi_ops_through_dialect_dispatch(native_libs):
+    """raf_amd.op.sgd_multi / sgd_multi_mixed: declare -> dispatch to the hip dialect -> OpEnv."""
+    from raf_amd import op
+
+    sizes = [(3, 5), (7,), (4100,)]
+    xs = [rng_for(210, t, 1).normal(0, 0.02, s).astype(np.float32) for t, s in enumerate(sizes)]
+    ds = [rng_for(210, t, 0).normal(0, 1e-3, s).astype(np.float32) for t, s in enumerate(sizes)]
+    vs = [rng_for(210, t, 2).normal(0, 1e-3, s).astype(np.float32) for t, s in enumerate(sizes)]
+    tl = [_dev(a) for a in xs + ds + vs]
+    out = op.sgd_multi(tl, 0.01, 0.9)
+    assert out[0] is tl[0] and len(out) == 9
+    ox, ov, _ = sgd_f32.sgd_list_step(xs, ds, vs, 0.01, 0.9)
+    for t in range(3):
+        assert np.array_equal(tl[t].cpu().numpy(), ox[t]) and np.array_equal(tl[6 + t].cpu().numpy(), ov[t])
+    d16 = [d.astype(np.float16) for d in ds]
+    tl = [_dev(a) for a in xs + d16 + vs] + [torch.zeros(s, dtype=torch.float16, device=DEV) for s in sizes]
+    op.sgd_multi_mixed(tl, 0.01, 0.9)
+    ox, ov, opp = sgd_f32.sgd_list_step(xs, d16, vs, 0.01, 0.9, "float16")
+    for t in range(3):
+        assert np.array_equal(tl[t].cpu().numpy(), ox[t]) and np.array_equal(tl[6 + t].cpu().numpy(), ov[t])
+        assert np.array_equal(tl[9 + t].cpu().numpy(), opp[t])
+    with pytest.raises(native_libs.RafError, match="float16 or bfloat16"):
+        op.sgd_multi_mixed(tl[:9] + [t.float() for t in tl[9:]], 0.01, 0.9)

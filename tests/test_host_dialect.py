@@ -29,7 +29,7 @@ def test_dispatch_lists_seen_from_python(native_libs):
     assert op.dispatch_list("raf.op.lans") == [("hip", "raf.op.hip.lans", 30)]
     assert op.dispatch_list("raf.op.sgd") == [("hip", "raf.op.hip.sgd", 30)]
     assert op.dispatch_list("raf.op.lans_mixed") == [("hip", "raf.op.hip.lans_mixed", 30)]
-    for name in ("l2norm", "fuse_tensor", "defuse_tensor"):
+    for name in ("l2norm", "fuse_tensor", "defuse_tensor", "sgd_multi", "sgd_multi_mixed"):
         assert op.dispatch_list(f"raf.op.{name}") == [("hip", f"raf.op.hip.{name}", 30)]
     assert op.dispatch_list("raf.op.lans", op.DEV_CPU) == []
     with op.with_dialect("tvm"):
@@ -57,6 +57,12 @@ def test_declare_errors_reach_python(native_libs):
         op.sgd(x, torch.zeros(4, 5), x, 0.1, 0.9)
     with pytest.raises(_lib.RafError, match="4n tensors"):
         op.lans([x] * 3, torch.tensor(1.0), 1e-3, .9, .999, 1e-6, True, 0.01, True, True, True)
+    with pytest.raises(_lib.RafError, match="3n tensors"):
+        op.sgd_multi([x] * 4, 0.1, 0.9)
+    with pytest.raises(_lib.RafError, match="differ in shape"):
+        op.sgd_multi([x, torch.zeros(4, 5), x], 0.1, 0.9)
+    with pytest.raises(_lib.RafError, match="Cannot find a valid dispatch for op raf.op.sgd_multi"):
+        op.sgd_multi([x] * 3, 0.1, 0.9)
     with pytest.raises(_lib.RafError, match="5n tensors"):
         op.lans_mixed([x] * 4, torch.tensor(1.0), 1e-3, .9, .999, 1e-6, True, 0.01, True, True, True)
 
