@@ -46,6 +46,11 @@ MEASURED_TRAFFIC = {
     ("lans_bert_large_fp16grad", "lans_pipelined"): 14_088_400_000,
     ("lans_bert_large_fp16grad", "lans_apply"): 8_716_600_000,
     ("sgd_4m_fp32", "sgd_vec4_kernel"): 83_925_600,
+    ("lans_bert_large_mixed_fp16", "lans_pipelined"): 14_759_300_000,
+    ("sgd_multi_bert_large_fp32", "sgd_multi_kernel"): 6_708_200_000,
+    ("l2norm_bert_large_flat_fp32", "l2norm_partials"): 1_340_800_000,
+    ("fuse_bert_large_fp32", "fuse_copy"): 2_683_900_000,
+    ("defuse_bert_large_fp32", "fuse_copy"): 2_683_900_000,
 }
 
 
