@@ -119,6 +119,44 @@ int rafhip_raf_env_output(const rafhip_raf_env* env, int32_t index, int32_t* dty
                           int32_t* dtype_bits, int32_t* ndim, int64_t* shape_out,
                           int32_t shape_capacity);
 
+/* ------------------------------------------------------------- device API and memory pools
+ * The `rocm` DeviceAPI (the ROCm counterpart of src/device_api/cuda/cuda.cc:25-248; interface
+ * include/raf/device_api.h:19-177) and the memory-pool front end (include/raf/memory_pool.h:28-56,
+ * src/impl/memory_pool.cc:89-180) seen from C.  device_type: 1 cpu, 10 rocm.  The default pool of
+ * a rocm device is "no_pool" (stream-ordered allocation from the HIP memory pool), of the cpu
+ * "page_unit_pool".
+ */
+int rafhip_raf_device_count(int32_t device_type, int32_t* count_out);
+/* DeviceAPI::CopyDataFromTo on two contiguous tensors of equal byte size; stream may be NULL. */
+int rafhip_raf_device_copy(const rafhip_tensor_desc* from, const rafhip_tensor_desc* to, void* stream);
+int rafhip_raf_stream_create(int32_t device_type, int32_t device_id, void** stream_out);
+int rafhip_raf_stream_free(int32_t device_type, int32_t device_id, void* stream);
+int rafhip_raf_event_create(int32_t device_type, int32_t device_id, uint32_t flags, void** event_out);
+int rafhip_raf_event_free(int32_t device_type, int32_t device_id, void* event);
+int rafhip_raf_event_record(int32_t device_type, void* event, void* stream);
+int rafhip_raf_event_elapsed_ms(int32_t device_type, void* start_event, void* end_event, float* ms_out);
+int rafhip_raf_stream_wait_event(int32_t device_type, void* stream, void* event);
+/* WaitDevice (what = 0, handle ignored), WaitStream (1) or WaitEvent (2). */
+int rafhip_raf_wait(int32_t device_type, int32_t device_id, int32_t what, void* handle);
+
+/* Memory::Alloc (stream_ordered = 0) or Memory::AllocAsync on the device's pool; alignment <= 0
+ * selects the default (64).  The handle keeps the chunk alive; freeing it hands the chunk back to
+ * its pool (or, stream-ordered, to the stream it came from). */
+typedef struct rafhip_raf_memory rafhip_raf_memory;
+int rafhip_raf_memory_alloc(int32_t device_type, int32_t device_id, int64_t nbytes, int64_t alignment,
+                            int32_t stream_ordered, void* stream, rafhip_raf_memory** mem_out);
+void* rafhip_raf_memory_data(const rafhip_raf_memory* mem);
+int rafhip_raf_memory_free(rafhip_raf_memory* mem);
+/* raf.memory_pool.InitPool / RemovePool / ResetPool (src/impl/memory_pool.cc:144-180). */
+int rafhip_raf_pool_init(int32_t device_type, int32_t device_id, const char* pool_name);
+int rafhip_raf_pool_remove(int32_t device_type, int32_t device_id);
+int rafhip_raf_pool_reset(int32_t device_type, int32_t device_id);
+/* Name of the device's pool and <used, pool> sizes in MB; any output may be NULL. */
+int rafhip_raf_pool_info(int32_t device_type, int32_t device_id, char* name_buf, int32_t buflen,
+                         float* used_mb_out, float* pool_mb_out);
+/* Memory::GetAllocBytes: what a request of nbytes really takes from the pool; -1 on error. */
+int64_t rafhip_raf_pool_alloc_bytes(int32_t device_type, int32_t device_id, int64_t nbytes);
+
 /* Total bytes of the OpEnv's workspace requests (each rounded up to 256). */
 int64_t rafhip_raf_env_workspace_bytes(const rafhip_raf_env* env);
 /* OpEnv::name() and the dialect op the dispatcher picked; pointers stay valid until destroy. */

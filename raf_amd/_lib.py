@@ -148,10 +148,50 @@ DIALECT_SYMBOLS = {
     "rafhip_raf_env_num_outputs": (c_int32, [c_void_p]),
     "rafhip_raf_env_output": (c_int, [c_void_p, c_int32, POINTER(c_int32), POINTER(c_int32), POINTER(c_int32),
                                       POINTER(c_int64), c_int32]),
+    "rafhip_raf_device_count": (c_int, [c_int32, POINTER(c_int32)]),
+    "rafhip_raf_device_copy": (c_int, [POINTER(TensorDesc), POINTER(TensorDesc), c_void_p]),
+    "rafhip_raf_stream_create": (c_int, [c_int32, c_int32, POINTER(c_void_p)]),
+    "rafhip_raf_stream_free": (c_int, [c_int32, c_int32, c_void_p]),
+    "rafhip_raf_event_create": (c_int, [c_int32, c_int32, ctypes.c_uint32, POINTER(c_void_p)]),
+    "rafhip_raf_event_free": (c_int, [c_int32, c_int32, c_void_p]),
+    "rafhip_raf_event_record": (c_int, [c_int32, c_void_p, c_void_p]),
+    "rafhip_raf_event_elapsed_ms": (c_int, [c_int32, c_void_p, c_void_p, POINTER(c_float)]),
+    "rafhip_raf_stream_wait_event": (c_int, [c_int32, c_void_p, c_void_p]),
+    "rafhip_raf_wait": (c_int, [c_int32, c_int32, c_int32, c_void_p]),
+    "rafhip_raf_memory_alloc": (c_int, [c_int32, c_int32, c_int64, c_int64, c_int32, c_void_p, POINTER(c_void_p)]),
+    "rafhip_raf_memory_data": (c_void_p, [c_void_p]),
+    "rafhip_raf_memory_free": (c_int, [c_void_p]),
+    "rafhip_raf_pool_init": (c_int, [c_int32, c_int32, c_char_p]),
+    "rafhip_raf_pool_remove": (c_int, [c_int32, c_int32]),
+    "rafhip_raf_pool_reset": (c_int, [c_int32, c_int32]),
+    "rafhip_raf_pool_info": (c_int, [c_int32, c_int32, c_char_p, c_int32, POINTER(c_float), POINTER(c_float)]),
+    "rafhip_raf_pool_alloc_bytes": (c_int64, [c_int32, c_int32, c_int64]),
     "rafhip_raf_env_workspace_bytes": (c_int64, [c_void_p]),
     "rafhip_raf_env_name": (c_char_p, [c_void_p]),
     "rafhip_raf_env_op": (c_char_p, [c_void_p]),
     "rafhip_raf_env_destroy": (c_int, [c_void_p]),
+}
+
+# include/rafhip_device.h: the HIP runtime calls behind the rocm DeviceAPI (same library)
+DEVICE_SYMBOLS = {
+    "rafhip_dev_set": (c_int, [c_int32]),
+    "rafhip_dev_alloc": (c_int, [c_int64, POINTER(c_void_p)]),
+    "rafhip_dev_free": (c_int, [c_void_p]),
+    "rafhip_dev_alloc_async": (c_int, [c_int32, c_int64, c_void_p, POINTER(c_void_p)]),
+    "rafhip_dev_free_async": (c_int, [c_void_p, c_void_p]),
+    "rafhip_dev_pool_size": (c_int, [c_int32, POINTER(c_int64), POINTER(c_int64)]),
+    "rafhip_dev_memcpy": (c_int, [c_void_p, c_void_p, c_int64, c_int32, c_void_p]),
+    "rafhip_dev_memcpy_peer": (c_int, [c_void_p, c_int32, c_void_p, c_int32, c_int64, c_void_p]),
+    "rafhip_dev_stream_create": (c_int, [c_int32, POINTER(c_void_p)]),
+    "rafhip_dev_stream_destroy": (c_int, [c_int32, c_void_p]),
+    "rafhip_dev_event_create": (c_int, [c_int32, ctypes.c_uint32, POINTER(c_void_p)]),
+    "rafhip_dev_event_destroy": (c_int, [c_int32, c_void_p]),
+    "rafhip_dev_event_elapsed_ms": (c_int, [c_void_p, c_void_p, POINTER(c_float)]),
+    "rafhip_dev_event_record": (c_int, [c_void_p, c_void_p]),
+    "rafhip_dev_stream_wait_event": (c_int, [c_void_p, c_void_p]),
+    "rafhip_dev_sync_device": (c_int, [c_int32]),
+    "rafhip_dev_sync_stream": (c_int, [c_void_p]),
+    "rafhip_dev_sync_event": (c_int, [c_void_p]),
 }
 
 _optim = None
@@ -175,6 +215,7 @@ def optim():
                 "(hipcc --offload-arch=gfx950); there is no fallback path")
         lib = ctypes.CDLL(str(OPTIM_LIB), mode=ctypes.RTLD_GLOBAL)
         _bind(lib, OPTIM_SYMBOLS)
+        _bind(lib, DEVICE_SYMBOLS)
         _optim = lib
     return _optim
 

@@ -5,11 +5,16 @@
 #include <string>
 
 #include "hip_dialect.h"
+#include "memory_pool.h"
 #include "raf_iface.h"
 #include "rafhip_dialect.h"
 
 using namespace raf;
 using namespace raf::op;
+
+struct rafhip_raf_memory {
+  std::shared_ptr<memory_pool::Memory> mem;
+};
 
 struct rafhip_raf_env {
   OpEnvPtr env;
@@ -374,6 +379,144 @@ int rafhip_raf_env_output(const rafhip_raf_env* env, int32_t index, int32_t* dty
       for (int i = 0; i < t.ndim(); ++i) shape_out[i] = t.shape[(size_t)i];
     }
   });
+}
+
+// ------------------------------------------------------------------ device API and memory pools
+int rafhip_raf_device_count(int32_t device_type, int32_t* count_out) {
+  return Guard([&] {
+    if (!count_out) throw Error("rafhip_raf_device_count: count_out is NULL");
+    *count_out = device_api::DeviceAPI::Get(DevType(device_type))->GetDeviceCount();
+  });
+}
+
+int rafhip_raf_device_copy(const rafhip_tensor_desc* from, const rafhip_tensor_desc* to, void* stream) {
+  return Guard([&] {
+    auto f = FromDesc(from, "from"), t = FromDesc(to, "to");
+    const bool gpu = f->tensor.device.device_type() == DevType::kROCM() ||
+                     t->tensor.device.device_type() == DevType::kROCM();
+    device_api::DeviceAPI::Get(gpu ? DevType::kROCM() : DevType::kCPU())
+        ->CopyDataFromTo(f->tensor, t->tensor, stream);
+  });
+}
+
+int rafhip_raf_stream_create(int32_t device_type, int32_t device_id, void** stream_out) {
+  return Guard([&] {
+    if (!stream_out) throw Error("rafhip_raf_stream_create: stream_out is NULL");
+    *stream_out = device_api::DeviceAPI::Get(DevType(device_type))
+                      ->CreateStream(Device(DevType(device_type), device_id));
+  });
+}
+
+int rafhip_raf_stream_free(int32_t device_type, int32_t device_id, void* stream) {
+  return Guard([&] {
+    device_api::DeviceAPI::Get(DevType(device_type))->FreeStream(Device(DevType(device_type), device_id), stream);
+  });
+}
+
+int rafhip_raf_event_create(int32_t device_type, int32_t device_id, uint32_t flags, void** event_out) {
+  return Guard([&] {
+    if (!event_out) throw Error("rafhip_raf_event_create: event_out is NULL");
+    *event_out = device_api::DeviceAPI::Get(DevType(device_type))
+                     ->CreateEvent(Device(DevType(device_type), device_id), flags);
+  });
+}
+
+int rafhip_raf_event_free(int32_t device_type, int32_t device_id, void* event) {
+  return Guard([&] {
+    device_api::DeviceAPI::Get(DevType(device_type))->FreeEvent(Device(DevType(device_type), device_id), event);
+  });
+}
+
+int rafhip_raf_event_record(int32_t device_type, void* event, void* stream) {
+  return Guard([&] { device_api::DeviceAPI::Get(DevType(device_type))->EventRecordOnStream(event, stream); });
+}
+
+int rafhip_raf_event_elapsed_ms(int32_t device_type, void* start_event, void* end_event, float* ms_out) {
+  return Guard([&] {
+    if (!ms_out) throw Error("rafhip_raf_event_elapsed_ms: ms_out is NULL");
+    *ms_out = device_api::DeviceAPI::Get(DevType(device_type))
+                  ->EventElapsedTimeInMilliSeconds(start_event, end_event);
+  });
+}
+
+int rafhip_raf_stream_wait_event(int32_t device_type, void* stream, void* event) {
+  return Guard([&] { device_api::DeviceAPI::Get(DevType(device_type))->StreamWaitEvent(stream, event); });
+}
+
+int rafhip_raf_wait(int32_t device_type, int32_t device_id, int32_t what, void* handle) {
+  return Guard([&] {
+    auto api = device_api::DeviceAPI::Get(DevType(device_type));
+    switch (what) {
+      case 0:
+        api->WaitDevice(Device(DevType(device_type), device_id));
+        break;
+      case 1:
+        api->WaitStream(handle);
+        break;
+      case 2:
+        api->WaitEvent(handle);
+        break;
+      default:
+        throw Error("rafhip_raf_wait: what must be 0 (device), 1 (stream) or 2 (event)");
+    }
+  });
+}
+
+int rafhip_raf_memory_alloc(int32_t device_type, int32_t device_id, int64_t nbytes, int64_t alignment,
+                            int32_t stream_ordered, void* stream, rafhip_raf_memory** mem_out) {
+  return Guard([&] {
+    if (!mem_out) throw Error("rafhip_raf_memory_alloc: mem_out is NULL");
+    *mem_out = nullptr;
+    const Device dev(DevType(device_type), device_id);
+    if (alignment <= 0) alignment = kDefaultMemoryAlignment;
+    auto m = stream_ordered ? memory_pool::Memory::AllocAsync(dev, nbytes, stream, alignment)
+                            : memory_pool::Memory::Alloc(dev, nbytes, alignment);
+    *mem_out = new rafhip_raf_memory{std::move(m)};
+  });
+}
+
+void* rafhip_raf_memory_data(const rafhip_raf_memory* mem) { return mem ? mem->mem->data : nullptr; }
+
+int rafhip_raf_memory_free(rafhip_raf_memory* mem) {
+  return Guard([&] { delete mem; });
+}
+
+int rafhip_raf_pool_init(int32_t device_type, int32_t device_id, const char* pool_name) {
+  return Guard([&] {
+    if (!pool_name) throw Error("rafhip_raf_pool_init: pool_name is NULL");
+    memory_pool::InitPool(Device(DevType(device_type), device_id), pool_name);
+  });
+}
+
+int rafhip_raf_pool_remove(int32_t device_type, int32_t device_id) {
+  return Guard([&] { memory_pool::RemovePool(Device(DevType(device_type), device_id)); });
+}
+
+int rafhip_raf_pool_reset(int32_t device_type, int32_t device_id) {
+  return Guard([&] { memory_pool::ResetPool(Device(DevType(device_type), device_id)); });
+}
+
+int rafhip_raf_pool_info(int32_t device_type, int32_t device_id, char* name_buf, int32_t buflen,
+                         float* used_mb_out, float* pool_mb_out) {
+  return Guard([&] {
+    const Device dev(DevType(device_type), device_id);
+    memory_pool::MemoryPool* pool = memory_pool::Memory::GetPool(dev);
+    if (name_buf && buflen > 0) {
+      std::strncpy(name_buf, pool->GetName().c_str(), (size_t)buflen - 1);
+      name_buf[buflen - 1] = '\0';
+    }
+    if (used_mb_out || pool_mb_out) {
+      auto sz = pool->GetPoolSize();
+      if (used_mb_out) *used_mb_out = sz.first;
+      if (pool_mb_out) *pool_mb_out = sz.second;
+    }
+  });
+}
+
+int64_t rafhip_raf_pool_alloc_bytes(int32_t device_type, int32_t device_id, int64_t nbytes) {
+  int64_t r = -1;
+  Guard([&] { r = memory_pool::Memory::GetAllocBytes(Device(DevType(device_type), device_id), nbytes); });
+  return r;
 }
 
 int64_t rafhip_raf_env_workspace_bytes(const rafhip_raf_env* env) {

@@ -16,6 +16,7 @@
 //   schemas ................. scripts/src_codegen/def_schema.py:671-694
 //   declare ................. src/op/declare/optimizer.cc:22-62
 //   registration macros ..... include/raf/dialect.h:231-243, include/raf/op.h:331-334
+//   DeviceAPI ............... include/raf/device_api.h:19-177, src/impl/device_api.cc:18-50
 // Failures that the reference raises through CHECK / LOG(FATAL) (a dmlc::Error) are raf::Error here.
 #pragma once
 
@@ -27,6 +28,7 @@
 #include <mutex>
 #include <stdexcept>
 #include <string>
+#include <utility>
 #include <vector>
 
 namespace raf {
@@ -115,21 +117,46 @@ TupleValue AsTuple(const Value& v);
 }  // namespace value
 
 // -------------------------------------------------------------------------------------- device api
+// include/raf/device.h:24 takes this from TVM's runtime (kAllocAlignment); 64 in the TVM
+// generation the reference was written against.
+constexpr int64_t kDefaultMemoryAlignment = 64;
+
 namespace device_api {
 
-// Only the part an OpEnv uses: the compute stream the executor made current
-// (include/raf/device_api.h, src/device_api/cuda/cuda.cc:168-177).
+// The reference's unified low-level device interface, include/raf/device_api.h:19-177, method for
+// method.  Implementations register a maker under the device type's name (the reference's
+// "raf.device_api._make.<devtype>" global, src/impl/device_api.cc:26-31) and Get creates one
+// instance per device type on first use (:37-47).
 class DeviceAPI {
  public:
-  static DeviceAPI* Get(DevType device_type);
-  void* GetStream() const { return stream_; }
-  void SetStream(const Device& dev, void* stream) {
-    (void)dev;
-    stream_ = stream;
-  }
+  virtual ~DeviceAPI() = default;
+  virtual int GetDeviceCount() = 0;
+  virtual void* AllocMemory(int64_t nbytes, int64_t alignment) = 0;
+  virtual void* AllocMemoryAsync(int64_t nbytes, void* stream, int64_t alignment) = 0;
+  virtual void FreeMemory(void* ptr) = 0;
+  virtual void FreeMemoryAsync(void* ptr, void* stream) = 0;
+  // Contiguous tensors of equal byte size; `stream` may be null (synchronous copy).
+  virtual void CopyDataFromTo(const TensorView& from, const TensorView& to, void* stream = nullptr) = 0;
+  // <bytes handed to users, bytes taken from the system> of the device's own pool, if it has one.
+  virtual std::pair<int64_t, int64_t> GetPoolSize() { return std::make_pair(0, 0); }
+  virtual void SetDevice(const int device_id) = 0;
+  virtual void* CreateStream(const Device& dev) = 0;
+  virtual void FreeStream(const Device& dev, void* stream) = 0;
+  virtual void SetStream(const Device& dev, void* stream) = 0;
+  virtual void* GetStream() = 0;
+  virtual void* CreateEvent(const Device& dev, uint32_t flags = 0) = 0;
+  virtual void FreeEvent(const Device& dev, void* event) = 0;
+  virtual float EventElapsedTimeInMilliSeconds(void* start_event, void* end_event) = 0;
+  virtual void EventRecordOnStream(void* event, void* stream) = 0;
+  virtual void StreamWaitEvent(void* stream, void* event) = 0;
+  virtual void WaitDevice(const Device& dev) = 0;
+  virtual void WaitStream(void* stream) = 0;
+  virtual void WaitEvent(void* event) = 0;
 
- private:
-  void* stream_ = nullptr;
+  // Raises raf::Error if no maker is registered for the device type.
+  static std::shared_ptr<DeviceAPI> Get(DevType device_type);
+  using Maker = DeviceAPI* (*)();
+  static bool RegisterMaker(const std::string& devtype_name, Maker maker);
 };
 
 }  // namespace device_api

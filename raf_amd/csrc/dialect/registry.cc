@@ -48,19 +48,6 @@ TupleValue AsTuple(const Value& v) {
 
 }  // namespace value
 
-namespace device_api {
-
-DeviceAPI* DeviceAPI::Get(DevType device_type) {
-  static std::mutex mu;
-  static std::map<int, std::unique_ptr<DeviceAPI>> apis;
-  std::lock_guard<std::mutex> lock(mu);
-  auto& slot = apis[(int)device_type];
-  if (!slot) slot.reset(new DeviceAPI());
-  return slot.get();
-}
-
-}  // namespace device_api
-
 namespace op {
 
 // ------------------------------------------------------------------------------------- schemas
@@ -276,7 +263,7 @@ void OpEnv::RequestWorkspace(void** dest, const Device& device, int64_t nbytes) 
 }
 
 void OpEnv::SetStreamForAllBackends(Device device, void* stream) {
-  device_api::DeviceAPI::Get(device.device_type())->SetStream(device, stream);
+  device_api::DeviceAPI::Get(device.device_type())->SetStream(device, stream);  // src/impl/op.cc:92-96
 }
 
 // ------------------------------------------------------------------------------------ registries

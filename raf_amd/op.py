@@ -17,7 +17,7 @@ from typing import Dict, List, Sequence, Tuple
 
 import torch
 
-from . import _lib
+from . import _lib, runtime
 from ._lib import TensorDesc, check_raf
 
 DEV_CPU, DEV_CUDA, DEV_ROCM = 1, 2, 10  # include/raf/device.h:37-50
@@ -61,6 +61,13 @@ class _Env:
             _lib.dialect().rafhip_raf_env_destroy(self.handle)
         except Exception:
             pass
+
+
+def _workspace(env: "_Env", like: torch.Tensor, stream) -> runtime.Memory:
+    """The OpEnv's workspace requests as one chunk from the device's memory pool, allocated on the
+    call's stream like the VM does around Execute (src/impl/vm/vm.cc:1099-1105, :846-853)."""
+    dev_id = like.device.index if like.device.index is not None else 0
+    return runtime.Memory(DEV_ROCM, dev_id, env.workspace_bytes, 256, stream, stream_ordered=True)
 
 
 _env_cache: Dict[Tuple, _Env] = {}
@@ -161,14 +168,12 @@ def _lans(op_name, tensor_list, step, learning_rate, beta1, beta2, eps, bias_cor
         make = lib.rafhip_raf_lans_make if op_name == "lans" else lib.rafhip_raf_lans_mixed_make
         check_raf(make(n4, descs, dstep, *hp, ctypes.byref(h)))
         env = _env_cache[key] = _Env(h)
-    ws = None
-    ws_ptr = None
-    if env.workspace_bytes > 0:
-        ws = torch.empty(env.workspace_bytes, dtype=torch.uint8, device=tensor_list[0].device)
-        ws_ptr = ws.data_ptr()
     stream = _stream(tensor_list[0]) if n4 else None
-    check_raf(lib.rafhip_raf_lans_execute(env.handle, n4, descs, dstep, ws_ptr,
+    ws = _workspace(env, tensor_list[0], stream) if env.workspace_bytes > 0 else None
+    check_raf(lib.rafhip_raf_lans_execute(env.handle, n4, descs, dstep, ws.data if ws else None,
                                           env.workspace_bytes, stream))
+    if ws:
+        ws.close()  # stream-ordered: the memory goes back to the pool after the step's kernels
     return tensor_list
 
 
@@ -203,9 +208,11 @@ def l2norm(x: torch.Tensor) -> torch.Tensor:
         check_raf(lib.rafhip_raf_l2norm_make(dx, ctypes.byref(h)))
         env = _env_cache[key] = _Env(h)
     (out,) = _alloc_outputs(env, x.device)
-    ws = torch.empty(env.workspace_bytes, dtype=torch.uint8, device=x.device) if env.workspace_bytes else None
-    check_raf(lib.rafhip_raf_l2norm_execute(env.handle, dx, _desc(out, keep), ws.data_ptr() if ws is not None else None,
+    ws = _workspace(env, x, _stream(x)) if env.workspace_bytes else None
+    check_raf(lib.rafhip_raf_l2norm_execute(env.handle, dx, _desc(out, keep), ws.data if ws else None,
                                             env.workspace_bytes, _stream(x)))
+    if ws:
+        ws.close()
     return out
 
 

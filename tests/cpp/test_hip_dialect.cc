@@ -5,8 +5,10 @@
 // name of each check so a failure names itself.  Runs without a GPU.
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <string>
 
+#include "memory_pool.h"
 #include "raf_iface.h"
 
 using namespace raf;
@@ -69,6 +71,11 @@ static CallValues SgdCall(DevType dev, std::vector<int64_t> xs = {4, 4},
   a->learning_rate = 0.1;
   a->mu = 0.9;
   return MakeCall("raf.op.sgd", a);
+}
+
+// The rocm pool's constructor makes its device current, which needs a GPU.
+static bool DeviceAPI_count_is_zero() {
+  return device_api::DeviceAPI::Get(DevType::kROCM())->GetDeviceCount() == 0;
 }
 
 int main() {
@@ -248,6 +255,82 @@ int main() {
   EXPECT(device_api::DeviceAPI::Get(DevType::kROCM())->GetStream() == &dummy);
   EXPECT(device_api::DeviceAPI::Get(DevType::kCPU())->GetStream() == nullptr);
   OpEnv::SetStreamForAllBackends(Device(DevType::kROCM(), 0), nullptr);
+
+  std::puts("device APIs: registration, the cpu API, rocm without a device");
+  {
+    using device_api::DeviceAPI;
+    EXPECT(DeviceAPI::Get(DevType::kCPU()) == DeviceAPI::Get(DevType::kCPU()));  // one instance per type
+    EXPECT(Raises([] { DeviceAPI::Get(DevType::kCUDA()); }).find("raf.device_api._make.cuda") != std::string::npos);
+    auto cpu = DeviceAPI::Get(DevType::kCPU());
+    EXPECT(cpu->GetDeviceCount() >= 1);
+    void* a = cpu->AllocMemory(1000, 256);
+    EXPECT(a != nullptr && reinterpret_cast<uintptr_t>(a) % 256 == 0);
+    TensorView from, to;
+    std::vector<float> src(250, 1.5f);
+    from.data = src.data();
+    from.shape = {250};
+    from.device = Device(DevType::kCPU(), 0);
+    to = from;
+    to.data = a;
+    cpu->CopyDataFromTo(from, to, nullptr);
+    EXPECT(static_cast<float*>(a)[249] == 1.5f);
+    to.shape = {249};
+    EXPECT(!Raises([&] { cpu->CopyDataFromTo(from, to, nullptr); }).empty());
+    cpu->FreeMemory(a);
+    EXPECT(Raises([&] { cpu->CreateStream(Device(DevType::kCPU(), 0)); }).find("no CreateStream") != std::string::npos);
+    EXPECT(cpu->GetPoolSize() == (std::pair<int64_t, int64_t>{0, 0}));
+    auto rocm = DeviceAPI::Get(DevType::kROCM());
+    if (rocm->GetDeviceCount() == 0) {  // no GPU in this process: runtime calls fail as raf::Error
+      EXPECT(Raises([&] { rocm->AllocMemory(64, 64); }).find("failed with status") != std::string::npos);
+      EXPECT(!Raises([&] { rocm->WaitEvent(nullptr); }).empty());
+    }
+    EXPECT(!Raises([&] { rocm->CreateStream(Device(DevType::kCPU(), 0)); }).empty());
+  }
+
+  std::puts("memory pools on the cpu device API");
+  {
+    using memory_pool::Memory;
+    const Device cpu(DevType::kCPU(), 0);
+    EXPECT(Memory::GetPool(cpu)->GetName() == "page_unit_pool");  // the default for cpu
+    EXPECT(Memory::GetAllocBytes(cpu, 1) == 4096 && Memory::GetAllocBytes(cpu, 4096) == 4096 &&
+           Memory::GetAllocBytes(cpu, 4097) == 8192 && Memory::GetAllocBytes(cpu, 0) == 0);
+    auto m1 = Memory::Alloc(cpu, 5000);
+    void* p1 = m1->data;
+    EXPECT(p1 != nullptr && reinterpret_cast<uintptr_t>(p1) % 64 == 0);
+    auto sz = Memory::GetPoolSize(cpu);
+    EXPECT(sz.first == 8192.f / 1048576.f && sz.second == sz.first);
+    auto m2 = Memory::Alloc(cpu, 6000);  // same page count, the first chunk is busy: a second chunk
+    EXPECT(m2->data != p1);
+    m1.reset();                          // idle now: the next request of that size gets it back
+    auto m3 = Memory::Alloc(cpu, 8000);
+    EXPECT(m3->data == p1);
+    sz = Memory::GetPoolSize(cpu);
+    EXPECT(sz.first == sz.second && sz.second == 16384.f / 1048576.f);
+    m2.reset();
+    sz = Memory::GetPoolSize(cpu);
+    EXPECT(sz.first == 8192.f / 1048576.f && sz.second == 16384.f / 1048576.f);
+    EXPECT(Memory::Alloc(cpu, 0)->data == nullptr);
+    EXPECT(Raises([&] { Memory::Alloc(cpu, 64, 48); }).find("is not aligned to 64") != std::string::npos);
+    EXPECT(Raises([&] { Memory::AllocAsync(cpu, 64, nullptr); }).find("Please use NoPool") != std::string::npos);
+    auto batch = Memory::AllocBatch(cpu, {100, 200, 0});
+    EXPECT(batch.size() == 3 && batch[0]->data != batch[1]->data && batch[2]->data == nullptr);
+    // a removed pool stops serving, its chunks live on with their users; reset keeps the kind
+    memory_pool::RemovePool(cpu);
+    std::memset(m3->data, 7, 8000);
+    memory_pool::InitPool(cpu, "no_pool");
+    EXPECT(Memory::GetPool(cpu)->GetName() == "no_pool" && Memory::GetAllocBytes(cpu, 5) == 5);
+    auto n1 = Memory::Alloc(cpu, 5000);
+    EXPECT(n1->data != nullptr && n1->device.device_type() == DevType::kCPU());
+    EXPECT(Raises([&] { Memory::AllocAsync(cpu, 64, nullptr); }).find("no AllocMemoryAsync") != std::string::npos);
+    memory_pool::ResetPool(cpu);
+    EXPECT(Memory::GetPool(cpu)->GetName() == "no_pool");
+    EXPECT(Raises([&] { memory_pool::InitPool(cpu, "nope"); }).find("raf.memory_pool._make.nope") != std::string::npos);
+    memory_pool::InitPool(cpu, "page_unit_pool");
+    if (DeviceAPI_count_is_zero())  // the rocm pool makes its device current: a raf::Error without a GPU
+      EXPECT(Raises([] { Memory::GetPool(Device(DevType::kROCM(), 0)); }).find("hipSetDevice") != std::string::npos);
+    else
+      EXPECT(Memory::GetPool(Device(DevType::kROCM(), 0))->GetName() == "no_pool");
+  }
 
   std::puts("ALL OK");
   return 0;

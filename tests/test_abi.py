@@ -26,6 +26,15 @@ def test_optim_header_symbols_all_exported_and_bound(native_libs):
     assert sorted(native_libs.OPTIM_SYMBOLS) == names, "ctypes table and header disagree"
 
 
+def test_device_header_symbols_all_exported_and_bound(native_libs):
+    lib = native_libs.optim()
+    names = _declared("rafhip_device.h")
+    assert len(names) == 18
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in rafhip_device.h but not exported"
+    assert sorted(native_libs.DEVICE_SYMBOLS) == names
+
+
 def test_dialect_header_symbols_all_exported_and_bound(native_libs):
     lib = native_libs.dialect()
     names = _declared("rafhip_dialect.h")

@@ -15,7 +15,8 @@ def test_cpp_registry_dispatch_declare(native_libs, tmp_path):
     d = ROOT / "raf_amd" / "csrc" / "dialect"
     subprocess.run(["g++", "-O1", "-std=c++17", "-Wall", f"-I{d}", f"-I{ROOT / 'include'}",
                     str(ROOT / "tests" / "cpp" / "test_hip_dialect.cc"),
-                    str(d / "registry.cc"), str(d / "hip_dialect.cc"),
+                    str(d / "registry.cc"), str(d / "hip_dialect.cc"), str(d / "device_api.cc"),
+                    str(d / "memory_pool.cc"),
                     f"-L{native_libs.LIB_DIR}", "-lraf_hip_optim", f"-Wl,-rpath,{native_libs.LIB_DIR}",
                     "-o", str(exe)], check=True)
     r = subprocess.run([str(exe)], capture_output=True, text=True)
