@@ -28,10 +28,11 @@ struct CachePolicy {  // true = non-temporal
   bool a_g, b_g, b_wmv, c_g, c_wmv, c_stores;
 };
 constexpr CachePolicy kPhasedPolicy = {true, false, true, false, true, true};
-// Pipelined: pass B loads w, m, v temporally so that they are cached when pass C of the same group
-// reads them a round later; pass C reads non-temporally (a hit is consumed, not kept) and writes
-// non-temporally; the gradient is not worth cache space there.  Measured best of seven combinations.
-constexpr CachePolicy kPipelinedPolicy = {true, true, false, true, true, true};
+// Pipelined: pass A leaves the gradient cached for pass B of the same group a round later, which
+// consumes it (non-temporal); pass B loads w, m, v temporally so that they are cached when pass C
+// of the group reads them another round later; pass C reads non-temporally (a hit is consumed, not
+// kept) and writes non-temporally.  Measured best of nine combinations.
+constexpr CachePolicy kPipelinedPolicy = {false, true, false, true, true, true};
 // Lists whose whole working set fits in the cache (a few million elements) are better off cached.
 constexpr CachePolicy kResidentPolicy = {false, false, false, false, false, false};
 
