@@ -268,3 +268,40 @@ def test_op_lans_mixed_and_half_precision_optimizer(native_libs, dtype):
     with pytest.raises(native_libs.RafError, match="float16 or bfloat16"):
         op.lans_mixed(tl[:12] + [t.float() for t in tl[12:]], torch.tensor(4.0, device=DEV), 1e-3, 0.9, 0.999,
                       1e-6, True, 0.01, True, True, True)
+
+
+@pytest.mark.parametrize("schedule", ["pipelined", "phased"])
+def test_tensor_beyond_two_to_the_31_elements(native_libs, schedule):
+    """Element counts are 64-bit end to end (the reference's are int: lans.cc:57).  One tensor of
+    2049 * 2^20 = 2,148,532,224 elements built as 2049 copies of a 2^20-element block, followed by
+    a small tensor.  Without gradient normalisation the trust ratios ||w|| / ||u|| of the tiled
+    tensor equal the block's, so every copy must carry the block's result: copies bitwise equal to
+    one another (every chunk indexed correctly), the first one within tolerance of the oracle on
+    the block, and the norms sqrt(2049) times the block's."""
+    from oracle import lans_f64
+    from raf_amd import kernels
+    from tests.helpers import lans_inputs
+
+    P, K = 1 << 20, 2049
+    hp = lans_f64.LansHParams(normalize_grad=False, grad_unscale=1 / 1024)
+    g, w, m, v = lans_inputs([P, 1000], cfg=400, g16=True)
+    dev = lambda a: torch.from_numpy(a).to(DEV)
+    big = lambda a: dev(a).repeat(K)
+    tg, tw, tm, tv = ([big(x[0]), dev(x[1])] for x in (g, w, m, v))
+    assert tw[0].numel() == P * K > 2 ** 31
+    plan = kernels.LansPlan([P * K, 1000], torch.float16, DEV)
+    plan.set_schedule(schedule)
+    plan.step(tg, tw, tm, tv, torch.tensor(3.0, device=DEV), kernels.make_hparams(normalize_grad=False,
+                                                                                  grad_unscale=1 / 1024))
+    torch.cuda.synchronize()
+    norms = plan.read_norms()
+    ow, om, ov, on = lans_f64.lans_step(g, w, m, v, 3, hp)
+    for got, want in ((tw, ow), (tm, om), (tv, ov)):
+        tiles = got[0].view(K, P)
+        assert torch.equal(tiles, tiles[0].expand(K, P)), "copies of the block differ"
+        assert max_rel_err(tiles[0].cpu().numpy(), want[0]) <= 1e-5
+        assert max_rel_err(got[1].cpu().numpy(), want[1]) <= 1e-5
+    assert np.allclose(norms[0], on[0] * np.sqrt(K), rtol=1e-12, atol=0)
+    assert np.allclose(norms[1], on[1], rtol=1e-12, atol=0)
+    assert torch.equal(tg[0][-P:], dev(g[0])), "gradients must stay untouched"
+    plan.close()

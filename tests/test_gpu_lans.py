@@ -295,3 +295,48 @@ def test_pipelined_schedule_is_bitwise_equal_to_phased(native_libs, monkeypatch,
             ow, om, ov, on = lans_f64.lans_step(g, ow, om, ov, step, hp)
         _assert_close(results["pipelined"][0], ow + om + ov, TOL_1, name)
         _assert_norms(results["pipelined"][1], on)
+
+
+# ------------------------------------------------------------------ graph capture
+@pytest.mark.parametrize("schedule", ["phased", "pipelined"])
+def test_step_can_be_captured_in_a_hip_graph(native_libs, schedule):
+    """A step enqueues kernels only (no allocation, no host synchronisation once the pointer table
+    has been sent), so it can be captured; every replay, with eager work and synchronisations in
+    between, must give the bits of the eager step from the same state."""
+    from raf_amd import kernels
+
+    sizes = [70001, 5, 8192, 300000, 1]
+    g, w, m, v = lans_inputs(sizes, cfg=85)
+    tg, tw, tm, tv = _to_dev(g), _to_dev(w), _to_dev(m), _to_dev(v)
+    plan = kernels.LansPlan(sizes, torch.float32, DEV)
+    plan.set_schedule(schedule)
+    plan.bind(tg, tw, tm, tv, _khp(LansHParams()))
+    step = torch.full((), 1.0, device=DEV)
+
+    def one_step():
+        plan.step_bound(step)
+        step.add_(1.0)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up on the side stream: the pointer table goes out here
+        one_step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        one_step()
+    torch.cuda.synchronize()
+    for _ in range(4):
+        state = [t.clone() for t in tw + tm + tv] + [step.clone()]
+        one_step()  # eager
+        torch.cuda.synchronize()
+        want = [t.clone() for t in tw + tm + tv]
+        for dst, src in zip(tw + tm + tv + [step], state):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert all(torch.equal(a, b) for a, b in zip(tw + tm + tv, want))
+        assert plan.read_norms().shape == (len(sizes), 4)
+    plan.close()

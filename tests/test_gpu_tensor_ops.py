@@ -59,6 +59,23 @@ def test_l2norm_special_values_and_views(native_libs):
     assert float(kernels.l2norm(x)) == pytest.approx(float(torch.sqrt(torch.sum(x * x))), rel=1e-6)
 
 
+def test_l2norm_beyond_two_to_the_31_elements(native_libs):
+    """64-bit element counts: 2^31 + 12345 halves and quarters, whose sum of squares is exact."""
+    import math
+    from raf_amd import kernels
+
+    n = 2 ** 31 + 12345
+    x = torch.full((n,), 0.5, device=DEV, dtype=torch.float16)
+    x[-7:] = 0.25
+    want = math.sqrt((n - 7) * 0.25 + 7 * 0.0625)
+    got = kernels.l2norm(x)
+    assert float(got) == float(np.float16(want))
+    del x, got
+    y = torch.full((n,), 0.5, device=DEV)
+    y[-7:] = 0.25
+    assert float(kernels.l2norm(y)) == float(np.float32(want))
+
+
 def test_l2norm_argument_errors(native_libs):
     from raf_amd import kernels
 
