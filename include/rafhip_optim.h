@@ -118,8 +118,8 @@ void rafhip_lans_default_hparams(rafhip_lans_hparams* hp);
 /*
  * A plan fixes what LansImpl's constructor fixes: the number of tensors and their element counts
  * (lans.cc:51-72), plus the gradient dtype.  Creation builds the device-side chunk table (one
- * hipMalloc + upload); the step calls then launch a fixed five-kernel sequence without touching
- * the allocator.  A plan belongs to the device that was current at creation and is not
+ * hipMalloc + upload); the step calls then launch a fixed kernel sequence (see the schedules
+ * below) without touching the allocator.  A plan belongs to the device that was current at creation and is not
  * thread-safe: one step at a time per plan.
  */
 typedef struct rafhip_lans_plan rafhip_lans_plan;
@@ -220,9 +220,9 @@ int rafhip_lans_read_norms(const rafhip_lans_plan* plan, const void* workspace, 
 
 /*
  * Optional per-kernel timing.  slots > 0 makes each following step record HIP events around its
- * five kernels on the step's stream into slot (step_index % slots); slots == 0 turns it off.
- * rafhip_lans_timing_read waits for that slot's last event and returns the five durations in
- * milliseconds.  Phased schedule: [0] norms of g,w  [1] finish  [2] norms of u_m,u_g  [3] finish
+ * kernels on the step's stream into slot (step_index % slots); slots == 0 turns it off.
+ * rafhip_lans_timing_read waits for that slot's last event and returns five durations in
+ * milliseconds.  Phased schedule: [0] norm of g  [1] finish  [2] norms of u_m, u_g, w  [3] finish
  * [4] apply.  Pipelined schedule: [0] set-up  [1] the persistent kernel  [2..4] zero.
  */
 int rafhip_lans_timing_enable(rafhip_lans_plan* plan, int32_t slots);

@@ -12,11 +12,13 @@
 // reference stores them: 16 B/element of extra traffic plus a 4 B/element buffer).
 //
 // Two schedules run the same per-chunk code and give bit-identical results:
-//   phased     five launches (A, finish, B, finish, C), each over all chunks of all tensors.
+//   phased     a set-up launch plus five launches (A, finish, B, finish, C), each over all chunks
+//              of all tensors.
 //   pipelined  one small set-up launch plus ONE persistent launch.  Tensors are packed into groups
 //              whose working set is a fraction of the 256 MB Infinity Cache, and the work list
-//              interleaves pass A of group s with pass B of group s-1 and pass C of group s-2, so a
-//              group's second and third reads are served by the cache instead of HBM.  Workgroups
+//              interleaves pass A of group s with pass B of group s-1 and pass C of group s-2, so
+//              that pass B finds the group's gradient, and pass C its w, m, v, in the cache
+//              instead of HBM.  Workgroups
 //              draw items from an atomic ticket.  Chunk items of pass A and B just store their
 //              partial sums; a "finish" item per tensor and pass, placed after them in the list,
 //              waits for those partials, adds them and publishes the tensor's statistics; items of
@@ -30,7 +32,8 @@
 // Determinism.  A chunk's partial sum depends only on the chunk (fixed lane order, fixed wave
 // tree); a tensor's total adds its chunk partials in a fixed order whichever workgroup does it.
 // Results are bit-identical from run to run, across grid sizes and across the two schedules.
-// Atomics are used for tickets, counters and flags only, never to accumulate values.
+// The only atomic read-modify-write is the work-list ticket; values are never accumulated
+// atomically.
 //
 // Mixed precision.  Gradients may arrive as binary16 or bfloat16 (widened exactly on load, which
 // replaces the reference's group_cast, python/raf/optim/lans.py:261-265), and pass C can write,

@@ -262,7 +262,7 @@ def test_default_schedule_follows_list_length(native_libs, monkeypatch):
 @pytest.mark.parametrize("g16", [False, True])
 def test_pipelined_schedule_is_bitwise_equal_to_phased(native_libs, monkeypatch, g16, group_elems):
     """The persistent, cache-aware schedule runs the same per-chunk code and adds the same partials
-    in the same order as the five-launch schedule: every output bit must agree, and both must
+    in the same order as the one-launch-per-pass schedule: every output bit must agree, and both must
     match the oracle."""
     from raf_amd import kernels, shapes
 

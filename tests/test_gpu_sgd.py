@@ -76,7 +76,7 @@ def test_outputs_may_alias_inputs(native_libs):
 
 
 def test_config1_full_size_bitwise(native_libs, c_oracle):
-    """BASELINE config 1: one fp32 tensor of 4,194,304 elements, w~N(0,.02), grad~N(0,1e-3),
+    """Benchmark configuration 1: one fp32 tensor of 4,194,304 elements, w~N(0,.02), grad~N(0,1e-3),
     velocity 0, lr .01, momentum .9 -- every element compared."""
     from raf_amd import kernels
 
