@@ -18,7 +18,7 @@ import numpy as np
 HERE = Path(__file__).resolve().parent
 sys.path.insert(0, str(HERE.parent.parent))
 
-from oracle import lans_f64, sgd_f32  # noqa: E402
+from oracle import halfs, lans_f64, sgd_f32, tensor_ops  # noqa: E402
 from tests.helpers import lans_inputs  # noqa: E402
 
 LANS_SIZES = [1, 3, 4, 5, 63, 65, 512, 513]
@@ -69,8 +69,58 @@ def lans_fixture():
     np.savez_compressed(HERE / "lans_kat.npz", **out)
 
 
+MIXED_SIZES = [1, 4, 5, 257, 1027]
+MIXED_CASES = {
+    # name: (gradient dtype, model dtype)
+    "f16_f16": ("float16", "float16"),
+    "bf16_bf16": ("bfloat16", "bfloat16"),
+    "bf16_f16": ("bfloat16", "float16"),
+}
+NORM_SIZES = [1, 5, 1000, 70001]
+NORM_DTYPES = ("float32", "float64", "float16", "bfloat16")
+
+
+def norm_input(n, dtype, k):
+    x = np.random.default_rng([2024, 7, k]).normal(0, 0.02, n)
+    if dtype == "bfloat16":
+        return halfs.f32_to_bf16_bits(x.astype(np.float32))
+    return x.astype(dtype)
+
+
+def mixed_fixture():
+    """The mixed-precision LANS step (half gradients in, 16-bit weight copies out), the
+    multi-tensor SGD step with half gradients and copies, and l2norm in its four dtypes."""
+    out = {}
+    hp = lans_f64.LansHParams(grad_unscale=1.0 / 1024)
+    for name, (gdt, mdt) in MIXED_CASES.items():
+        g, w, m, v = lans_inputs(MIXED_SIZES, cfg=120 + len(name), g16=gdt)
+        for t in range(len(MIXED_SIZES)):
+            out[f"lans/{name}/g{t}"], out[f"lans/{name}/w{t}"] = g[t], w[t]
+            out[f"lans/{name}/m{t}"], out[f"lans/{name}/v{t}"] = m[t], v[t]
+        for s in range(2):
+            w, m, v, p, _ = lans_f64.lans_mixed_step(g, w, m, v, 2 + s, hp, mdt)
+        for t in range(len(MIXED_SIZES)):
+            out[f"lans/{name}/w{t}_after2"] = w[t]
+            out[f"lans/{name}/p{t}_after2"] = p[t].view(np.uint16)
+        # SGD on the same tensors: x = w, dx = g (not unscaled), v = m
+        g, x, vel, _ = lans_inputs(MIXED_SIZES, cfg=120 + len(name), g16=gdt)
+        for s in range(2):
+            x, vel, p = sgd_f32.sgd_list_step(x, g, vel, 0.01, 0.9, mdt)
+        for t in range(len(MIXED_SIZES)):
+            out[f"sgd/{name}/x{t}_after2"] = x[t].view(np.uint32)
+            out[f"sgd/{name}/v{t}_after2"] = vel[t].view(np.uint32)
+            out[f"sgd/{name}/p{t}_after2"] = p[t].view(np.uint16)
+    for dt in NORM_DTYPES:
+        for k, n in enumerate(NORM_SIZES):
+            r = tensor_ops.l2norm(norm_input(n, dt, k))
+            out[f"l2norm/{dt}/{n}"] = np.frombuffer(r.tobytes(), dtype=np.uint8)
+    np.savez_compressed(HERE / "mixed_kat.npz", **out)
+
+
+FIXTURES = {"sgd_kat.npz": sgd_fixture, "lans_kat.npz": lans_fixture, "mixed_kat.npz": mixed_fixture}
+
 if __name__ == "__main__":
-    sgd_fixture()
-    lans_fixture()
-    for f in ("sgd_kat.npz", "lans_kat.npz"):
+    # no arguments: every fixture; otherwise the named files only
+    for f in sys.argv[1:] or FIXTURES:
+        FIXTURES[f]()
         print(f, (HERE / f).stat().st_size, "bytes")

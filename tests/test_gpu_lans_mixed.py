@@ -212,3 +212,35 @@ def test_mixed_argument_errors(native_libs):
                                     plan.workspace.data_ptr(), plan.workspace.numel(), None)
     assert st == native_libs.RAFHIP_ERR_UNSUPPORTED and b"weight-copy dtype" in lib.rafhip_last_error()
     plan.close()
+
+
+# ------------------------------------------------------------------ committed fixtures
+@pytest.mark.parametrize("name", ["f16_f16", "bf16_bf16", "bf16_f16"])
+def test_mixed_golden_fixture(native_libs, name):
+    """Mixed-precision LANS, multi-tensor SGD with half gradients and copies, against the stored
+    vectors: LANS weights within 1e-5, their 16-bit copies equal to the narrowing of what was
+    stored; SGD bit-exact on x, v and the copies."""
+    from raf_amd import kernels
+    from tests.golden import make_fixtures as mf
+
+    z = np.load(mf.HERE / "mixed_kat.npz")
+    gdt, mdt = mf.MIXED_CASES[name]
+    nt = len(mf.MIXED_SIZES)
+    g, w, m, v = ([z[f"lans/{name}/{q}{t}"] for t in range(nt)] for q in "gwmv")
+    out = _run(g, w, m, v, LansHParams(grad_unscale=1 / 1024), 2, model_dtype=mdt, first_step=2)
+    for t in range(nt):
+        assert max_rel_err(out[0][t], z[f"lans/{name}/w{t}_after2"]) <= TOL_1
+        assert np.array_equal(out[3][t], halfs.narrow_weight(out[0][t], mdt).view(np.uint16))
+        d = np.abs(out[3][t].astype(np.int32) - z[f"lans/{name}/p{t}_after2"].astype(np.int32))
+        assert d.max(initial=0) <= 1
+    tx, td, tv = _to_dev(w), _to_dev(g), _to_dev(m)
+    tp = [torch.zeros(a.size, dtype=TORCH_DT[mdt], device=DEV) for a in w]
+    plan = kernels.SgdPlan([a.size for a in w], td[0].dtype, DEV)
+    for _ in range(2):
+        plan.step(tx, td, tv, 0.01, 0.9, p=tp)
+    torch.cuda.synchronize()
+    for t in range(nt):
+        assert np.array_equal(tx[t].cpu().numpy().view(np.uint32), z[f"sgd/{name}/x{t}_after2"])
+        assert np.array_equal(tv[t].cpu().numpy().view(np.uint32), z[f"sgd/{name}/v{t}_after2"])
+        assert np.array_equal(_bits(tp[t]), z[f"sgd/{name}/p{t}_after2"])
+    plan.close()

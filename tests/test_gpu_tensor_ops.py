@@ -220,3 +220,22 @@ def test_ops_through_dialect_dispatch(native_libs):
     with op.with_dialect("cuda"):  # no such dialect here: nothing to dispatch to
         with pytest.raises(native_libs.RafError, match="Cannot find a valid dispatch"):
             op.l2norm(torch.randn(9, device=DEV))
+
+
+def test_l2norm_golden_fixture(native_libs):
+    """Stored l2norm results (four dtypes): equal, or one unit in the last place apart where the
+    float64 sums differ in their last bits."""
+    from raf_amd import kernels
+    from tests.golden import make_fixtures as mf
+
+    z = np.load(mf.HERE / "mixed_kat.npz")
+    tdt = {"float32": torch.float32, "float64": torch.float64, "float16": torch.float16, "bfloat16": torch.bfloat16}
+    idt = {"float32": np.int32, "float64": np.int64, "float16": np.int16, "bfloat16": np.int16}
+    for dt in mf.NORM_DTYPES:
+        for k, n in enumerate(mf.NORM_SIZES):
+            a = mf.norm_input(n, dt, k)
+            t = (torch.from_numpy(a.view(np.int16).copy()).to(DEV).view(torch.bfloat16) if dt == "bfloat16"
+                 else torch.from_numpy(a).to(DEV))
+            got = kernels.l2norm(t).cpu().view(-1).view({2: torch.int16, 4: torch.int32, 8: torch.int64}[t.element_size()])
+            want = np.frombuffer(z[f"l2norm/{dt}/{n}"].tobytes(), dtype=idt[dt])
+            assert abs(int(got[0]) - int(want[0])) <= 1, (dt, n)
