@@ -130,10 +130,12 @@ typedef struct rafhip_lans_plan rafhip_lans_plan;
 int rafhip_lans_query_layout(int32_t n_tensors, const int64_t* numel, int64_t* n_chunks_out,
                              int64_t* workspace_bytes_out);
 
-/* Elements per chunk, the unit of work and of the partial sums of the second and third pass, and
- * elements per unit of the first pass (a multiple of the chunk: that pass reads the gradient only). */
-int32_t rafhip_lans_chunk_elements(void);
-int32_t rafhip_lans_pass_a_unit_elements(void);
+/* Elements per chunk -- the unit of work and of the partial sums of the second and third pass --
+ * for a tensor of numel elements (it depends on the tensor's own size only: small tensors are cut
+ * finer), and elements per unit of the first pass (a multiple of the chunk: that pass reads the
+ * gradient only). */
+int32_t rafhip_lans_chunk_elements(int64_t numel);
+int32_t rafhip_lans_pass_a_unit_elements(int64_t numel);
 
 /*
  * Schedules of a step; both run the same per-chunk code and give bit-identical results.

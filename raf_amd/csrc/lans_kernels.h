@@ -1,6 +1,7 @@
 // Device-side data layout and launchers of the multi-tensor LANS step for gfx950.
 //
-// Work decomposition.  Every tensor is cut into chunks of kChunk elements; the plan keeps, in HBM,
+// Work decomposition.  Every tensor is cut into chunks of kChunk elements (kSmallChunk for small
+// tensors); the plan keeps, in HBM,
 // a tensor table (pointers, element count, first chunk) and a work list of (phase, tensor, chunk)
 // items.  One workgroup handles one item at a time.
 //
@@ -55,11 +56,23 @@ namespace rafhip {
 
 constexpr int kLansBlock = 256;  // 4 wavefronts
 constexpr int kLansWaves = kLansBlock / 64;
-constexpr int kChunk = 8192;     // elements per chunk (multiple of 4 * kLansBlock)
-constexpr int kChunksPerA = 8;   // pass A reads 2-4 bytes per element, so its unit of work (and of
+constexpr int kChunk = 8192;     // elements per chunk (multiple of 4 * kLansBlock) ...
+constexpr int kSmallChunk = 4096;              // ... and of tensors below kSmallTensorBelow elements:
+constexpr int64_t kSmallTensorBelow = 1 << 19;  // finer work for lists of small tensors, which are
+                                                // short of parallelism, not of bandwidth
+constexpr int kChunksPerAShift = 3;
+constexpr int kChunksPerA = 1 << kChunksPerAShift;   // pass A reads 2-4 bytes per element, so its unit of work (and of
                                  // partial sums) is 8 chunks; its partial lives in the first one's slot
 constexpr int kUnroll = 2;       // 4-element groups in flight per lane per trip
 constexpr int kPartialSlots = 4; // doubles per chunk: [0] sum g^2 | [1] sum u_m^2 [2] sum u_g^2 [3] sum w^2
+
+// A tensor's chunk size depends on its own element count alone, so its result does not depend on
+// which list it is part of.
+__host__ __device__ inline int chunk_shift_for(int64_t numel) {  // chunks are powers of two
+  return numel < kSmallTensorBelow ? 12 : 13;
+}
+__host__ __device__ inline int chunk_elems_for(int64_t numel) { return 1 << chunk_shift_for(numel); }
+static_assert(kSmallChunk == 1 << 12 && kChunk == 1 << 13, "chunk_shift_for must match the chunk sizes");
 
 struct TensorRec {  // 64 bytes, one per tensor
   const void* g;
@@ -70,7 +83,8 @@ struct TensorRec {  // 64 bytes, one per tensor
   int64_t numel;
   int32_t first_chunk;
   int32_t vec_ok;  // 1: every base pointer is aligned for 4-element lane accesses
-  int64_t reserved;
+  int32_t chunk_shift;  // chunk_shift_for(numel): the tensor's chunks hold 1 << chunk_shift elements
+  int32_t reserved;
 };
 
 // One unit of work: kind in the top three bits of `chunk_phase`, chunk number within the tensor

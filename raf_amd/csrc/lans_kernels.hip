@@ -205,9 +205,10 @@ struct ChunkView {
   int vec_ok;
 };
 
-// `unit` is kChunk for passes B and C and kChunksPerA * kChunk for pass A.
+// `unit_chunks` is 1 for passes B and C and kChunksPerA for pass A.
 __device__ __forceinline__ ChunkView chunk_view(const TensorRec& tr, uint32_t chunk,
-                                                int g_elem_bytes, int unit = kChunk) {
+                                                int g_elem_bytes, int unit_chunks = 1) {
+  const int unit = unit_chunks << tr.chunk_shift;
   const int64_t base = (int64_t)chunk * unit;
   const int64_t rest = tr.numel - base;
   ChunkView cv;
@@ -441,11 +442,11 @@ __device__ __forceinline__ void stats_after_b(TensorStats* st, const double (&to
 }
 
 __device__ __forceinline__ int64_t chunks_of(const TensorRec& tr) {
-  return (tr.numel + kChunk - 1) / kChunk;
+  return (tr.numel + ((int64_t)1 << tr.chunk_shift) - 1) >> tr.chunk_shift;
 }
-constexpr int kUnitA = kChunksPerA * kChunk;
 __device__ __forceinline__ int64_t units_a_of(const TensorRec& tr) {
-  return (tr.numel + kUnitA - 1) / kUnitA;
+  const int shift = tr.chunk_shift + kChunksPerAShift;
+  return (tr.numel + ((int64_t)1 << shift) - 1) >> shift;
 }
 
 // ------------------------------------------------------------------ set-up launch
@@ -497,7 +498,7 @@ __global__ __launch_bounds__(kLansBlock) void lans_norm_g(LansDeviceArgs a) {
     const WorkItem it = a.items_a[i];
     const TensorRec tr = a.tensors[it.tensor];
     const uint32_t unit = it.chunk_phase & kChunkMask;
-    const ChunkView cv = chunk_view(tr, unit, (int)sizeof(G), kUnitA);
+    const ChunkView cv = chunk_view(tr, unit, (int)sizeof(G), kChunksPerA);
     double s[1] = {chunk_sum_g<G, kP.a_g>(cv, a.unscale)};
     block_sum<1>(s, red);
     if (threadIdx.x == 0)
@@ -605,7 +606,7 @@ __global__ __launch_bounds__(kLansBlock) void lans_pipelined(LansDeviceArgs a) {
     const uint32_t phase = it.chunk_phase >> kPhaseShift;
     const uint32_t chunk = it.chunk_phase & kChunkMask;
     const bool unit_a = phase == kPhaseA;  // pass-A items count in units of kChunksPerA chunks
-    const ChunkView cv = chunk_view(tr, chunk, (int)sizeof(G), unit_a ? kUnitA : kChunk);
+    const ChunkView cv = chunk_view(tr, chunk, (int)sizeof(G), unit_a ? kChunksPerA : 1);
     const int64_t n_chunks = chunks_of(tr);
     double* part = a.partials + kPartialSlots * ((int64_t)tr.first_chunk +
                                                   (int64_t)chunk * (unit_a ? kChunksPerA : 1));

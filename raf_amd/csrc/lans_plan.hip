@@ -37,9 +37,13 @@ WorkspaceLayout make_layout(int32_t n_tensors, int64_t n_chunks) {
   return l;
 }
 
-inline int64_t chunks_of(int64_t numel) { return (numel + kChunk - 1) / kChunk; }
+inline int64_t chunks_of(int64_t numel) {
+  const int64_t c = chunk_elems_for(numel);
+  return (numel + c - 1) / c;
+}
 inline int64_t units_a_of(int64_t numel) {
-  return (numel + (int64_t)kChunksPerA * kChunk - 1) / ((int64_t)kChunksPerA * kChunk);
+  const int64_t u = (int64_t)kChunksPerA * chunk_elems_for(numel);
+  return (numel + u - 1) / u;
 }
 
 // Default size of a cache group in elements (measured optimum on MI355X for BERT-large and
@@ -202,8 +206,8 @@ void rafhip_lans_default_hparams(rafhip_lans_hparams* hp) {
   hp->grad_unscale = 1.0f;
 }
 
-int32_t rafhip_lans_chunk_elements(void) { return kChunk; }
-int32_t rafhip_lans_pass_a_unit_elements(void) { return kChunksPerA * kChunk; }
+int32_t rafhip_lans_chunk_elements(int64_t numel) { return chunk_elems_for(numel); }
+int32_t rafhip_lans_pass_a_unit_elements(int64_t numel) { return kChunksPerA * chunk_elems_for(numel); }
 
 int rafhip_lans_query_layout(int32_t n_tensors, const int64_t* numel, int64_t* n_chunks_out,
                              int64_t* workspace_bytes_out) {
@@ -416,6 +420,7 @@ int rafhip_lans_step_mixed(rafhip_lans_plan* plan, const void* const* g, float* 
     r.numel = plan->numel[t];
     r.first_chunk = plan->first_chunk[t];
     r.vec_ok = 0;
+    r.chunk_shift = chunk_shift_for(r.numel);
     r.reserved = 0;
     if (r.numel == 0) continue;
     if (!r.g || !r.w || !r.m || !r.v)

@@ -68,15 +68,16 @@ def test_sgd_argument_validation(native_libs):
 def test_lans_layout_query_is_host_arithmetic(native_libs):
     from raf_amd import kernels, shapes
 
-    chunk = native_libs.optim().rafhip_lans_chunk_elements()
-    assert chunk % 1024 == 0
+    per_tensor = native_libs.optim().rafhip_lans_chunk_elements
+    chunk = per_tensor(1)
+    assert chunk % 1024 == 0 and per_tensor(1 << 22) % chunk == 0
     sizes = [0, 1, chunk - 1, chunk, chunk + 1, 10 * chunk + 3]
     chunks, ws = kernels.query_layout(sizes)
     assert chunks == sum(-(-n // chunk) for n in sizes) == 0 + 1 + 1 + 1 + 2 + 11
     assert ws % 256 == 0 and ws >= 32 * chunks + 64 * len(sizes)
     big = shapes.numels(shapes.bert_large_shapes())
     chunks, ws = kernels.query_layout(big)
-    assert chunks == sum(-(-n // chunk) for n in big)
+    assert chunks == sum(-(-n // per_tensor(n)) for n in big)
     assert ws < 2 << 20  # no per-element scratch: under two megabytes for 335M elements
     assert kernels.query_layout([])[0] == 0
     lib = native_libs.optim()

@@ -5,9 +5,10 @@ import pytest
 KIND_A, KIND_B, KIND_C, KIND_WHOLE, KIND_FIN_A, KIND_FIN_B = range(6)
 
 
-def _check(order, sizes, chunk, unit_a):
-    n_chunks = [-(-n // chunk) for n in sizes]
-    n_units = [-(-n // unit_a) for n in sizes]
+def _check(order, sizes, lib):
+    # a tensor's chunk size (and first-pass unit) depends on its own element count
+    n_chunks = [-(-n // lib.rafhip_lans_chunk_elements(n)) for n in sizes]
+    n_units = [-(-n // lib.rafhip_lans_pass_a_unit_elements(n)) for n in sizes]
     seen = {}
     for pos, (kind, t, c) in enumerate(order):
         assert 0 <= t < len(sizes) and sizes[t] > 0, "empty tensors contribute no work"
@@ -35,18 +36,21 @@ def _check(order, sizes, chunk, unit_a):
 def test_order_invariants(native_libs, group):
     from raf_amd import kernels, shapes
 
-    chunk = native_libs.optim().rafhip_lans_chunk_elements()
-    unit_a = native_libs.optim().rafhip_lans_pass_a_unit_elements()
-    assert unit_a % chunk == 0
+    lib = native_libs.optim()
+    chunk, unit_a = lib.rafhip_lans_chunk_elements(1), lib.rafhip_lans_pass_a_unit_elements(1)
+    big = 1 << 19  # from here on tensors are cut into larger chunks
+    assert unit_a % chunk == 0 and lib.rafhip_lans_chunk_elements(big) > lib.rafhip_lans_chunk_elements(big - 1) == chunk
+    assert lib.rafhip_lans_pass_a_unit_elements(big) % lib.rafhip_lans_chunk_elements(big) == 0
     lists = [
-        [1, 3, 0, chunk - 1, chunk, chunk + 1, 5 * chunk + 7, 0, 2 * chunk, 17, unit_a, unit_a + 1, 3 * unit_a - 1],
+        [1, 3, 0, chunk - 1, chunk, chunk + 1, 5 * chunk + 7, 0, 2 * chunk, 17, unit_a, unit_a + 1, 3 * unit_a - 1,
+         big - 1, big, big + 1, 3 * big + 5],
         shapes.log_uniform_numels(300, seed=7),
         shapes.numels(shapes.bert_base_shapes()),
         [],
         [0, 0],
     ]
     for sizes in lists:
-        _check(kernels.pipeline_order(sizes, group), sizes, chunk, unit_a)
+        _check(kernels.pipeline_order(sizes, group), sizes, lib)
 
 
 def test_groups_bound_the_reuse_distance(native_libs):
@@ -54,7 +58,7 @@ def test_groups_bound_the_reuse_distance(native_libs):
     other tensors' work, which is what keeps the tensor in the Infinity Cache."""
     from raf_amd import kernels
 
-    chunk = native_libs.optim().rafhip_lans_chunk_elements()
+    chunk = native_libs.optim().rafhip_lans_chunk_elements(1)
     sizes = [8 * chunk] * 40  # 40 equal tensors, group = 2 tensors
     order = kernels.pipeline_order(sizes, 16 * chunk)
     first_a = {t: min(i for i, (k, tt, _) in enumerate(order) if k == KIND_A and tt == t) for t in range(40)}
@@ -74,6 +78,7 @@ def test_bert_large_group_structure(native_libs):
 
     sizes = shapes.numels(shapes.bert_large_shapes())
     order = kernels.pipeline_order(sizes)
-    chunk = native_libs.optim().rafhip_lans_chunk_elements()
-    _check(order, sizes, chunk, native_libs.optim().rafhip_lans_pass_a_unit_elements())
-    assert sum(1 for k, _, _ in order if k == KIND_WHOLE) == sum(1 for n in sizes if 0 < n <= chunk)
+    lib = native_libs.optim()
+    _check(order, sizes, lib)
+    assert sum(1 for k, _, _ in order if k == KIND_WHOLE) == sum(
+        1 for n in sizes if 0 < n <= lib.rafhip_lans_chunk_elements(n))
