@@ -51,7 +51,24 @@ class RecordUploader {
   hipError_t sync(std::vector<Rec>& recs, hipStream_t s) {
     if (count_ == 0) return hipSuccess;
     const size_t bytes = sizeof(Rec) * count_;
-    if (sent_once_ && std::memcmp(last_sent_.data(), recs.data(), bytes) == 0) return hipSuccess;
+    if (sent_once_ && std::memcmp(last_sent_.data(), recs.data(), bytes) == 0) {
+      // Same records, but a different stream than the one that carried them: order this stream
+      // behind the upload unless it has landed already.  A stream under graph capture is left
+      // alone (event queries are not allowed there): capture after a warm-up call has completed.
+      if (s != last_stream_) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &capturing) != hipSuccess) (void)hipGetLastError();
+        if (capturing == hipStreamCaptureStatusNone) {
+          if (hipEventQuery(staging_free_) == hipErrorNotReady) {
+            (void)hipGetLastError();  // "not ready" is an answer, not a failure
+            hipError_t e = hipStreamWaitEvent(s, staging_free_, 0);
+            if (e != hipSuccess) return e;
+          }
+          last_stream_ = s;
+        }
+      }
+      return hipSuccess;
+    }
     // The previous upload may still be reading the staging buffer.
     if (sent_once_) {
       hipError_t e = hipEventSynchronize(staging_free_);
@@ -63,6 +80,7 @@ class RecordUploader {
     if (e != hipSuccess) return e;
     last_sent_.swap(recs);
     sent_once_ = true;
+    last_stream_ = s;
     return hipSuccess;
   }
 
@@ -71,6 +89,7 @@ class RecordUploader {
   size_t count_ = 0;
   Rec* staging_ = nullptr;  // pinned
   hipEvent_t staging_free_ = nullptr;  // recorded after the last upload was enqueued
+  hipStream_t last_stream_ = nullptr;  // the stream that upload went to
   std::vector<Rec> last_sent_;
   bool sent_once_ = false;
 };

@@ -1,7 +1,6 @@
 """GPU parity of raf.op.lans: the HIP kernels, called through the C ABI, against the float64
 oracle.  Tolerances are the stated ones -- max relative error per element 1e-5 after one step and
 1e-4 after 100 steps -- on w, m and v; norms must agree to 1e-10."""
-import ctypes
 
 import numpy as np
 import pytest
@@ -339,4 +338,29 @@ def test_step_can_be_captured_in_a_hip_graph(native_libs, schedule):
         torch.cuda.synchronize()
         assert all(torch.equal(a, b) for a, b in zip(tw + tm + tv, want))
         assert plan.read_norms().shape == (len(sizes), 4)
+    plan.close()
+
+
+def test_same_tensors_on_another_stream(native_libs):
+    """The pointer table is uploaded on the first call's stream; a second call with the same tensors
+    on another stream must still see it (the library orders the new stream behind the upload)."""
+    from raf_amd import kernels
+
+    sizes = [300000, 17, 70001]
+    g, w, m, v = lans_inputs(sizes, cfg=86)
+    hp = LansHParams()
+    ow, om, ov = w, m, v
+    for step in (1, 2):
+        ow, om, ov, _ = lans_f64.lans_step(g, ow, om, ov, step, hp)
+    tg, tw, tm, tv = _to_dev(g), _to_dev(w), _to_dev(m), _to_dev(v)
+    plan = kernels.LansPlan(sizes, torch.float32, DEV)
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s1):
+        plan.step(tg, tw, tm, tv, 1, _khp(hp))
+    s2.wait_stream(s1)  # the caller orders the two steps; the table upload is the library's business
+    with torch.cuda.stream(s2):
+        plan.step(tg, tw, tm, tv, 2, _khp(hp))
+    torch.cuda.synchronize()
+    _assert_close([t.cpu().numpy() for t in tw], ow, TOL_1, "w")
     plan.close()
