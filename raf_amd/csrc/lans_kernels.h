@@ -157,8 +157,11 @@ struct LansDeviceArgs {
 void launch_prepare(hipStream_t s, const LansDeviceArgs& a, const float* step_dev,
                     int32_t step_host, HParamsPod hp);
 // `streaming`: the list is much larger than the Infinity Cache (non-temporal accesses) or fits in it.
-void launch_phased(int grad_dtype, bool streaming, hipStream_t s, const LansDeviceArgs& a,
-                   hipEvent_t* marks);
+// `inline_finish` (non-streaming lists only): every tensor has at most kInlineFinishChunks chunks,
+// so the passes add the partials themselves and the two finish launches are skipped.
+constexpr int kInlineFinishChunks = 32;
+void launch_phased(int grad_dtype, bool streaming, bool inline_finish, hipStream_t s,
+                   const LansDeviceArgs& a, hipEvent_t* marks);
 void launch_pipelined(int grad_dtype, unsigned grid, hipStream_t s, const LansDeviceArgs& a);
 // Resident workgroups per CU of the pipelined kernel (occupancy query), 0 on failure.
 int pipelined_blocks_per_cu(int grad_dtype);

@@ -415,10 +415,13 @@ __device__ __forceinline__ void chunk_apply(const ChunkView& cv, float unscale, 
 // ------------------------------------------------------------------ per-tensor finishes
 // From the total of pass A: the gradient norm and divisor (multi_tensor_lans.cu:284-286: divide
 // only when normalising and the norm is non-zero).  Executed by one thread.
+__device__ __forceinline__ double grad_divisor(double gn, const StepScalars& k) {
+  return (k.normalize_grad && gn != 0.0) ? 1.0 / (gn + k.eps) : 1.0;
+}
 __device__ __forceinline__ double stats_after_a(TensorStats* st, double sum_g,
                                                 const StepScalars& k) {
   const double gn = sqrt(sum_g);
-  const double inv_gdiv = (k.normalize_grad && gn != 0.0) ? 1.0 / (gn + k.eps) : 1.0;
+  const double inv_gdiv = grad_divisor(gn, k);
   publish(&st->grad_norm, gn);
   publish(&st->inv_grad_div, inv_gdiv);
   return inv_gdiv;
@@ -426,14 +429,23 @@ __device__ __forceinline__ double stats_after_a(TensorStats* st, double sum_g,
 
 // From the totals of pass B: ||w|| and the two trust ratios (multi_tensor_lans.cu:349-352) with
 // beta1 / beta3 folded in.  Executed by one thread.
-__device__ __forceinline__ void stats_after_b(TensorStats* st, const double (&tot)[3],
-                                              const StepScalars& k, double& ratio_m,
-                                              double& ratio_g) {
+struct NormsAfterB {
+  double unm, ung, pn;
+};
+__device__ __forceinline__ NormsAfterB trust_ratios(const double (&tot)[3], const StepScalars& k,
+                                                    double& ratio_m, double& ratio_g) {
   const double unm = sqrt(tot[0]), ung = sqrt(tot[1]), pn = sqrt(tot[2]);
   const double rm = (unm != 0.0 && pn != 0.0) ? k.lr * (pn / unm) : k.lr;
   const double rg = (ung != 0.0 && pn != 0.0) ? k.lr * (pn / ung) : k.lr;
   ratio_m = rm * k.beta1;
   ratio_g = rg * k.beta3;
+  return NormsAfterB{unm, ung, pn};
+}
+__device__ __forceinline__ void stats_after_b(TensorStats* st, const double (&tot)[3],
+                                              const StepScalars& k, double& ratio_m,
+                                              double& ratio_g) {
+  const NormsAfterB n = trust_ratios(tot, k, ratio_m, ratio_g);
+  const double unm = n.unm, ung = n.ung, pn = n.pn;
   publish(&st->param_norm, pn);
   publish(&st->um_norm, unm);
   publish(&st->ug_norm, ung);
@@ -490,9 +502,16 @@ __global__ __launch_bounds__(kLansBlock) void lans_prepare(LansDeviceArgs a, con
 }
 
 // ------------------------------------------------------------------ phased schedule
-template <typename G, bool kStream>
+// Three variants: streaming (lists far larger than the Infinity Cache), resident (lists that fit),
+// and resident with inline finishes for lists of short tensors only: there every workgroup of pass
+// B (C) adds the few chunk partials of its tensor itself -- the same sums in the same order as the
+// finish launch would -- and the two one-workgroup-per-tensor launches disappear, which is a fifth
+// of the step for a list of thousands of small tensors.
+enum PhasedMode { kModeStreaming = 0, kModeResident = 1, kModeResidentInline = 2 };
+
+template <typename G, int kMode>
 __global__ __launch_bounds__(kLansBlock) void lans_norm_g(LansDeviceArgs a) {
-  constexpr CachePolicy kP = kStream ? kPhasedPolicy : kResidentPolicy;
+  constexpr CachePolicy kP = kMode == kModeStreaming ? kPhasedPolicy : kResidentPolicy;
   __shared__ double red[3][kLansWaves];
   for (int64_t i = blockIdx.x; i < a.n_items_a; i += gridDim.x) {
     const WorkItem it = a.items_a[i];
@@ -524,9 +543,9 @@ __global__ __launch_bounds__(kLansBlock) void lans_finish(LansDeviceArgs a, int 
   }
 }
 
-template <typename G, bool kStream>
+template <typename G, int kMode>
 __global__ __launch_bounds__(kLansBlock) void lans_norm_u(LansDeviceArgs a) {
-  constexpr CachePolicy kP = kStream ? kPhasedPolicy : kResidentPolicy;
+  constexpr CachePolicy kP = kMode == kModeStreaming ? kPhasedPolicy : kResidentPolicy;
   __shared__ double red[3][kLansWaves];
   const StepScalars k = *a.scalars;
   // Back to front: pass A has just streamed the gradients front to back, so the end of the list is
@@ -535,8 +554,20 @@ __global__ __launch_bounds__(kLansBlock) void lans_norm_u(LansDeviceArgs a) {
     const int64_t c = a.n_chunks - 1 - b;
     const WorkItem it = a.items[c];
     const TensorRec tr = a.tensors[it.tensor];
-    const ChunkView cv = chunk_view(tr, it.chunk_phase & kChunkMask, (int)sizeof(G));
-    const double inv_gdiv = a.stats[it.tensor].inv_grad_div;
+    const uint32_t chunk = it.chunk_phase & kChunkMask;
+    const ChunkView cv = chunk_view(tr, chunk, (int)sizeof(G));
+    double inv_gdiv;
+    if constexpr (kMode == kModeResidentInline) {
+      double tot[1];
+      tensor_totals<1, false>(a.partials + kPartialSlots * (int64_t)tr.first_chunk, 0, units_a_of(tr),
+                              kChunksPerA, tot, red, nullptr);
+      if (chunk == 0 && threadIdx.x == 0)  // one workgroup per tensor leaves the statistics
+        inv_gdiv = stats_after_a(&a.stats[it.tensor], tot[0], k);
+      else
+        inv_gdiv = grad_divisor(sqrt(tot[0]), k);
+    } else {
+      inv_gdiv = a.stats[it.tensor].inv_grad_div;
+    }
     double s[3];
     chunk_sums_u<G, kP.b_g, kP.b_wmv>(cv, a.unscale, k, [&] { return inv_gdiv; }, s);
     block_sum<3>(s, red);
@@ -548,16 +579,30 @@ __global__ __launch_bounds__(kLansBlock) void lans_norm_u(LansDeviceArgs a) {
   }
 }
 
-template <typename G, bool kStream>
+template <typename G, int kMode>
 __global__ __launch_bounds__(kLansBlock) void lans_apply(LansDeviceArgs a) {
-  constexpr CachePolicy kP = kStream ? kPhasedPolicy : kResidentPolicy;
+  constexpr CachePolicy kP = kMode == kModeStreaming ? kPhasedPolicy : kResidentPolicy;
+  __shared__ double red[3][kLansWaves];
   const StepScalars k = *a.scalars;
   for (int64_t c = blockIdx.x; c < a.n_chunks; c += gridDim.x) {
     const WorkItem it = a.items[c];
     const TensorRec tr = a.tensors[it.tensor];
-    const ChunkView cv = chunk_view(tr, it.chunk_phase & kChunkMask, (int)sizeof(G));
-    const TensorStats st = a.stats[it.tensor];
-    const ApplyParams p{st.inv_grad_div, st.ratio_m, st.ratio_g};
+    const uint32_t chunk = it.chunk_phase & kChunkMask;
+    const ChunkView cv = chunk_view(tr, chunk, (int)sizeof(G));
+    ApplyParams p;
+    if constexpr (kMode == kModeResidentInline) {
+      double tot[3];
+      tensor_totals<3, false>(a.partials + kPartialSlots * (int64_t)tr.first_chunk, 1, chunks_of(tr), 1,
+                              tot, red, nullptr);
+      p.inv_gdiv = a.stats[it.tensor].inv_grad_div;  // left by pass B
+      if (chunk == 0 && threadIdx.x == 0)
+        stats_after_b(&a.stats[it.tensor], tot, k, p.rm, p.rg);
+      else
+        (void)trust_ratios(tot, k, p.rm, p.rg);
+    } else {
+      const TensorStats st = a.stats[it.tensor];
+      p = ApplyParams{st.inv_grad_div, st.ratio_m, st.ratio_g};
+    }
     chunk_apply<G, kP.c_g, kP.c_wmv, kP.c_stores>(cv, a.unscale, a.p_is_bf16 != 0, k, [&] { return p; });
   }
 }
@@ -687,7 +732,7 @@ void launch_prepare(hipStream_t s, const LansDeviceArgs& a, const float* step_de
 }
 
 namespace {
-template <typename G, bool kStream>
+template <typename G, int kMode>
 void launch_phased_t(hipStream_t s, const LansDeviceArgs& a, hipEvent_t* marks) {
   const unsigned grid = (unsigned)(a.n_chunks < (1 << 20) ? a.n_chunks : (1 << 20));
   const unsigned grid_a = (unsigned)(a.n_items_a < (1 << 20) ? a.n_items_a : (1 << 20));
@@ -695,27 +740,32 @@ void launch_phased_t(hipStream_t s, const LansDeviceArgs& a, hipEvent_t* marks) 
     if (marks) (void)hipEventRecord(marks[i], s);
   };
   mark(0);
-  hipLaunchKernelGGL((lans_norm_g<G, kStream>), dim3(grid_a), dim3(kLansBlock), 0, s, a);
+  constexpr bool kFinishLaunches = kMode != kModeResidentInline;
+  hipLaunchKernelGGL((lans_norm_g<G, kMode>), dim3(grid_a), dim3(kLansBlock), 0, s, a);
   mark(1);
-  hipLaunchKernelGGL(lans_finish, dim3((unsigned)a.n_tensors), dim3(kLansBlock), 0, s, a, 0);
+  if (kFinishLaunches)
+    hipLaunchKernelGGL(lans_finish, dim3((unsigned)a.n_tensors), dim3(kLansBlock), 0, s, a, 0);
   mark(2);
-  hipLaunchKernelGGL((lans_norm_u<G, kStream>), dim3(grid), dim3(kLansBlock), 0, s, a);
+  hipLaunchKernelGGL((lans_norm_u<G, kMode>), dim3(grid), dim3(kLansBlock), 0, s, a);
   mark(3);
-  hipLaunchKernelGGL(lans_finish, dim3((unsigned)a.n_tensors), dim3(kLansBlock), 0, s, a, 1);
+  if (kFinishLaunches)
+    hipLaunchKernelGGL(lans_finish, dim3((unsigned)a.n_tensors), dim3(kLansBlock), 0, s, a, 1);
   mark(4);
-  hipLaunchKernelGGL((lans_apply<G, kStream>), dim3(grid), dim3(kLansBlock), 0, s, a);
+  hipLaunchKernelGGL((lans_apply<G, kMode>), dim3(grid), dim3(kLansBlock), 0, s, a);
   mark(5);
 }
 }  // namespace
 
-void launch_phased(int grad_dtype, bool streaming, hipStream_t s, const LansDeviceArgs& a,
-                   hipEvent_t* marks) {
+void launch_phased(int grad_dtype, bool streaming, bool inline_finish, hipStream_t s,
+                   const LansDeviceArgs& a, hipEvent_t* marks) {
   auto go = [&](auto tag) {
     using G = decltype(tag);
     if (streaming)
-      launch_phased_t<G, true>(s, a, marks);
+      launch_phased_t<G, kModeStreaming>(s, a, marks);
+    else if (inline_finish)
+      launch_phased_t<G, kModeResidentInline>(s, a, marks);
     else
-      launch_phased_t<G, false>(s, a, marks);
+      launch_phased_t<G, kModeResident>(s, a, marks);
   };
   if (grad_dtype == RAFHIP_F16)
     go(_Float16{});

@@ -129,6 +129,7 @@ struct rafhip_lans_plan {
   int32_t schedule = RAFHIP_LANS_PHASED;
   int64_t n_chunks = 0;
   int64_t total_elements = 0;
+  bool short_tensors_only = false;  // no tensor has more than kInlineFinishChunks chunks
   uint32_t n_pipeline_items = 0;
   unsigned pipeline_grid = 0;
   std::vector<int64_t> numel;
@@ -259,12 +260,14 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
   p->grad_dtype = grad_dtype;
   p->numel.assign(numel, numel + n_tensors);
   p->first_chunk.resize(n_tensors);
-  int64_t chunks = 0, total = 0;
+  int64_t chunks = 0, total = 0, longest = 0;
   for (int32_t t = 0; t < n_tensors; ++t) {
     p->first_chunk[t] = (int32_t)chunks;
     chunks += chunks_of(numel[t]);
+    longest = std::max(longest, chunks_of(numel[t]));
     total += numel[t];
   }
+  p->short_tensors_only = longest <= kInlineFinishChunks;
   p->n_chunks = chunks;
   p->total_elements = total;
   p->schedule = schedule_setting(total);
@@ -478,8 +481,8 @@ int rafhip_lans_step_mixed(rafhip_lans_plan* plan, const void* const* g, float* 
   } else {
     launch_prepare(s, a, step_dev, step_host, pod);
     const int64_t bytes_per_elt = plan->grad_dtype == RAFHIP_F32 ? 16 : 14;
-    launch_phased(plan->grad_dtype, plan->total_elements * bytes_per_elt > kResidentBytes, s, a,
-                  marks);
+    launch_phased(plan->grad_dtype, plan->total_elements * bytes_per_elt > kResidentBytes,
+                  plan->short_tensors_only, s, a, marks);
   }
   RAFHIP_HIP_TRY(hipGetLastError());
   plan->steps_done++;
