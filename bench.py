@@ -207,7 +207,7 @@ def bench_lans(name, wl, args):
                    "bytes_per_element": a + b + c, "bytes_per_step": bytes_step,
                    "kernel_bytes_per_element": ka + kb + kc,
                    "pct_of_hbm_peak": round(100 * bytes_step / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
-                   "schedule": schedule, "launches_per_step": 6 if schedule == "phased" else 2},
+                   "schedule": schedule, "launches_per_step": 5 if schedule == "phased" else 2},
     }
     if not args.no_kernel_events:
         ts = np.array([plan.timing_read(i) for i in range(args.steps)], dtype=np.float64)

@@ -139,7 +139,8 @@ int32_t rafhip_lans_pass_a_unit_elements(int64_t numel);
 
 /*
  * Schedules of a step; both run the same per-chunk code and give bit-identical results.
- *   PHASED     one launch per pass over all chunks of all tensors (set-up + 5 launches).
+ *   PHASED     one launch per pass over all chunks of all tensors plus two small per-tensor
+ *              launches between them (5 launches; 3 for a list of short tensors only).
  *   PIPELINED  set-up + ONE persistent launch whose work list interleaves the three passes of
  *              neighbouring cache-sized tensor groups, so that a group's second and third reads
  *              come from the 256 MB Infinity Cache instead of HBM.

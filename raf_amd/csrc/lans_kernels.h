@@ -13,8 +13,8 @@
 // reference stores them: 16 B/element of extra traffic plus a 4 B/element buffer).
 //
 // Two schedules run the same per-chunk code and give bit-identical results:
-//   phased     a set-up launch plus five launches (A, finish, B, finish, C), each over all chunks
-//              of all tensors.
+//   phased     five launches (A, finish, B, finish, C), each over all chunks of all tensors; the
+//              first also writes the step scalars.  Lists of short tensors need no finish launches.
 //   pipelined  one small set-up launch plus ONE persistent launch.  Tensors are packed into groups
 //              whose working set is a fraction of the 256 MB Infinity Cache, and the work list
 //              interleaves pass A of group s with pass B of group s-1 and pass C of group s-2, so
@@ -160,8 +160,10 @@ void launch_prepare(hipStream_t s, const LansDeviceArgs& a, const float* step_de
 // `inline_finish` (non-streaming lists only): every tensor has at most kInlineFinishChunks chunks,
 // so the passes add the partials themselves and the two finish launches are skipped.
 constexpr int kInlineFinishChunks = 32;
+// The first pass also writes the step scalars: no set-up launch in this schedule.
 void launch_phased(int grad_dtype, bool streaming, bool inline_finish, hipStream_t s,
-                   const LansDeviceArgs& a, hipEvent_t* marks);
+                   const LansDeviceArgs& a, const float* step_dev, int32_t step_host,
+                   HParamsPod hp, hipEvent_t* marks);
 void launch_pipelined(int grad_dtype, unsigned grid, hipStream_t s, const LansDeviceArgs& a);
 // Resident workgroups per CU of the pipelined kernel (occupancy query), 0 on failure.
 int pipelined_blocks_per_cu(int grad_dtype);

@@ -461,10 +461,39 @@ __device__ __forceinline__ int64_t units_a_of(const TensorRec& tr) {
   return (tr.numel + ((int64_t)1 << shift) - 1) >> shift;
 }
 
-// ------------------------------------------------------------------ set-up launch
 // Host scalars of the reference (lans.cc:94-109), evaluated on the device so that the step tensor
-// never has to be copied to the host; also marks every word the pipelined schedule waits on
-// (chunk partials, per-tensor statistics) as not ready and rewinds the ticket.
+// never has to be copied to the host; also rewinds the ticket and clears the error word.  One thread.
+__device__ __forceinline__ void write_step_scalars(const LansDeviceArgs& a, const float* step_dev,
+                                                   int32_t step_host, const HParamsPod& hp) {
+  a.sync->ticket = 0u;
+  a.sync->error = 0u;
+  const int step = step_dev ? (int)(*step_dev) : step_host;
+  float bc1 = 1.0f, bc2 = 1.0f;
+  if (hp.bias_correction == 1) {  // double pow, then one rounding to fp32 (lans.cc:103-104)
+    bc1 = (float)(1.0 - pow((double)hp.beta1, (double)step));
+    bc2 = (float)(1.0 - pow((double)hp.beta2, (double)step));
+  }
+  StepScalars k;
+  k.beta1 = hp.beta1;
+  k.beta2 = hp.beta2;
+  k.one_minus_beta2 = 1.0f - hp.beta2;                             // fp32 subtraction (:291)
+  k.beta3 = (hp.grad_averaging == 1) ? (1.0f - hp.beta1) : 1.0f;  // fp32 (lans.cc:107-109)
+  k.eps = hp.eps;
+  k.wd = hp.weight_decay;
+  k.inv_bc1 = 1.0 / (double)bc1;
+  k.inv_bc2 = 1.0 / (double)bc2;
+  k.lr = hp.learning_rate;
+  k.decay_into_grad = hp.mode == 0 ? 1.0 : 0.0;
+  k.decay_into_dir = hp.mode == 0 ? 0.0 : 1.0;
+  k.normalize_grad = hp.normalize_grad;
+  k.pad = 0;
+  *a.scalars = k;
+}
+
+// ------------------------------------------------------------------ set-up launch
+// Set-up of a pipelined step: the step scalars, and every word the schedule waits on (chunk
+// partials, per-tensor statistics) marked as not ready.  The phased schedule waits on nothing and
+// writes its scalars from the first pass instead.
 __global__ __launch_bounds__(kLansBlock) void lans_prepare(LansDeviceArgs a, const float* step_dev,
                                                            int32_t step_host, HParamsPod hp) {
   const uint64_t tid = (uint64_t)blockIdx.x * kLansBlock + threadIdx.x;
@@ -474,31 +503,7 @@ __global__ __launch_bounds__(kLansBlock) void lans_prepare(LansDeviceArgs a, con
   uint64_t* part_words = reinterpret_cast<uint64_t*>(a.partials);
   for (uint64_t i = tid; i < (uint64_t)kPartialSlots * (uint64_t)a.n_chunks; i += nthr)
     part_words[i] = kNotReady;
-  if (tid == 0) {
-    a.sync->ticket = 0u;
-    a.sync->error = 0u;
-    const int step = step_dev ? (int)(*step_dev) : step_host;
-    float bc1 = 1.0f, bc2 = 1.0f;
-    if (hp.bias_correction == 1) {  // double pow, then one rounding to fp32 (lans.cc:103-104)
-      bc1 = (float)(1.0 - pow((double)hp.beta1, (double)step));
-      bc2 = (float)(1.0 - pow((double)hp.beta2, (double)step));
-    }
-    StepScalars k;
-    k.beta1 = hp.beta1;
-    k.beta2 = hp.beta2;
-    k.one_minus_beta2 = 1.0f - hp.beta2;                             // fp32 subtraction (:291)
-    k.beta3 = (hp.grad_averaging == 1) ? (1.0f - hp.beta1) : 1.0f;  // fp32 (lans.cc:107-109)
-    k.eps = hp.eps;
-    k.wd = hp.weight_decay;
-    k.inv_bc1 = 1.0 / (double)bc1;
-    k.inv_bc2 = 1.0 / (double)bc2;
-    k.lr = hp.learning_rate;
-    k.decay_into_grad = hp.mode == 0 ? 1.0 : 0.0;
-    k.decay_into_dir = hp.mode == 0 ? 0.0 : 1.0;
-    k.normalize_grad = hp.normalize_grad;
-    k.pad = 0;
-    *a.scalars = k;
-  }
+  if (tid == 0) write_step_scalars(a, step_dev, step_host, hp);
 }
 
 // ------------------------------------------------------------------ phased schedule
@@ -510,9 +515,12 @@ __global__ __launch_bounds__(kLansBlock) void lans_prepare(LansDeviceArgs a, con
 enum PhasedMode { kModeStreaming = 0, kModeResident = 1, kModeResidentInline = 2 };
 
 template <typename G, int kMode>
-__global__ __launch_bounds__(kLansBlock) void lans_norm_g(LansDeviceArgs a) {
+__global__ __launch_bounds__(kLansBlock) void lans_norm_g(LansDeviceArgs a, const float* step_dev,
+                                                          int32_t step_host, HParamsPod hp) {
   constexpr CachePolicy kP = kMode == kModeStreaming ? kPhasedPolicy : kResidentPolicy;
   __shared__ double red[3][kLansWaves];
+  // This pass needs no scalars; the later launches find them written by the first workgroup.
+  if (blockIdx.x == 0 && threadIdx.x == 0) write_step_scalars(a, step_dev, step_host, hp);
   for (int64_t i = blockIdx.x; i < a.n_items_a; i += gridDim.x) {
     const WorkItem it = a.items_a[i];
     const TensorRec tr = a.tensors[it.tensor];
@@ -733,7 +741,8 @@ void launch_prepare(hipStream_t s, const LansDeviceArgs& a, const float* step_de
 
 namespace {
 template <typename G, int kMode>
-void launch_phased_t(hipStream_t s, const LansDeviceArgs& a, hipEvent_t* marks) {
+void launch_phased_t(hipStream_t s, const LansDeviceArgs& a, const float* step_dev,
+                     int32_t step_host, const HParamsPod& hp, hipEvent_t* marks) {
   const unsigned grid = (unsigned)(a.n_chunks < (1 << 20) ? a.n_chunks : (1 << 20));
   const unsigned grid_a = (unsigned)(a.n_items_a < (1 << 20) ? a.n_items_a : (1 << 20));
   auto mark = [&](int i) {
@@ -741,7 +750,8 @@ void launch_phased_t(hipStream_t s, const LansDeviceArgs& a, hipEvent_t* marks) 
   };
   mark(0);
   constexpr bool kFinishLaunches = kMode != kModeResidentInline;
-  hipLaunchKernelGGL((lans_norm_g<G, kMode>), dim3(grid_a), dim3(kLansBlock), 0, s, a);
+  hipLaunchKernelGGL((lans_norm_g<G, kMode>), dim3(grid_a), dim3(kLansBlock), 0, s, a, step_dev,
+                     step_host, hp);
   mark(1);
   if (kFinishLaunches)
     hipLaunchKernelGGL(lans_finish, dim3((unsigned)a.n_tensors), dim3(kLansBlock), 0, s, a, 0);
@@ -757,15 +767,16 @@ void launch_phased_t(hipStream_t s, const LansDeviceArgs& a, hipEvent_t* marks) 
 }  // namespace
 
 void launch_phased(int grad_dtype, bool streaming, bool inline_finish, hipStream_t s,
-                   const LansDeviceArgs& a, hipEvent_t* marks) {
+                   const LansDeviceArgs& a, const float* step_dev, int32_t step_host,
+                   HParamsPod hp, hipEvent_t* marks) {
   auto go = [&](auto tag) {
     using G = decltype(tag);
     if (streaming)
-      launch_phased_t<G, kModeStreaming>(s, a, marks);
+      launch_phased_t<G, kModeStreaming>(s, a, step_dev, step_host, hp, marks);
     else if (inline_finish)
-      launch_phased_t<G, kModeResidentInline>(s, a, marks);
+      launch_phased_t<G, kModeResidentInline>(s, a, step_dev, step_host, hp, marks);
     else
-      launch_phased_t<G, kModeResident>(s, a, marks);
+      launch_phased_t<G, kModeResident>(s, a, step_dev, step_host, hp, marks);
   };
   if (grad_dtype == RAFHIP_F16)
     go(_Float16{});

@@ -479,10 +479,9 @@ int rafhip_lans_step_mixed(rafhip_lans_plan* plan, const void* const* g, float* 
     if (marks)
       for (int i = 2; i < 6; ++i) RAFHIP_HIP_TRY(hipEventRecord(marks[i], s));
   } else {
-    launch_prepare(s, a, step_dev, step_host, pod);
     const int64_t bytes_per_elt = plan->grad_dtype == RAFHIP_F32 ? 16 : 14;
     launch_phased(plan->grad_dtype, plan->total_elements * bytes_per_elt > kResidentBytes,
-                  plan->short_tensors_only, s, a, marks);
+                  plan->short_tensors_only, s, a, step_dev, step_host, pod, marks);
   }
   RAFHIP_HIP_TRY(hipGetLastError());
   plan->steps_done++;
