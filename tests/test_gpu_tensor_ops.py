@@ -239,3 +239,22 @@ def test_l2norm_golden_fixture(native_libs):
             got = kernels.l2norm(t).cpu().view(-1).view({2: torch.int16, 4: torch.int32, 8: torch.int64}[t.element_size()])
             want = np.frombuffer(z[f"l2norm/{dt}/{n}"].tobytes(), dtype=idt[dt])
             assert abs(int(got[0]) - int(want[0])) <= 1, (dt, n)
+
+
+@pytest.mark.parametrize("shape", [(64, 128), (128, 256)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_tensor_fusion_and_defusion(native_libs, shape, dtype):
+    """The reference's own test of the two ops (tests/python/op/cuda/test_cuda_memory.py:13-43):
+    the same tensor fused with itself and defused again, here with random data and exact equality."""
+    from raf_amd import op
+
+    size = shape[0] * shape[1]
+    sizes = [size, size]
+    tuple_shape = shape + shape
+    shape_indices = [len(shape), 2 * len(shape)]
+    x = torch.randn(shape, device=DEV).to(dtype)
+    with op.with_dialect(["tvm", "hip"]):
+        x_2 = op.fuse_tensor([x, x])
+        x_3 = op.defuse_tensor(x_2, sizes, tuple_shape, shape_indices)
+    assert x_2.shape == (2 * size,) and x_2.dtype == dtype
+    assert len(x_3) == 2 and all(y.shape == x.shape and torch.equal(y, x) for y in x_3)
