@@ -12,6 +12,7 @@ standing in for RAF's memory pool) and the current stream, nothing else.
 from __future__ import annotations
 
 import ctypes
+import weakref
 from ctypes import c_int64, c_void_p
 from typing import Dict, List, Sequence, Tuple
 
@@ -29,13 +30,17 @@ _DTYPES = {
 }
 
 
+_SHAPE_ARRAYS = [c_int64 * max(d, 1) for d in range(9)]  # ctypes array types are costly to make
+
+
 def _desc(t: torch.Tensor, keep: list) -> TensorDesc:
     if not isinstance(t, torch.Tensor):
         raise TypeError(f"expected a tensor, got {type(t).__name__}")
     if not t.is_contiguous():
         raise ValueError("tensors must be contiguous")
     code, bits = _DTYPES[t.dtype]
-    shape = (c_int64 * max(t.dim(), 1))(*t.shape)
+    nd = t.dim()
+    shape = (_SHAPE_ARRAYS[nd] if nd < 9 else c_int64 * nd)(*t.shape)
     keep.append(shape)
     # torch on ROCm reports its devices as "cuda"; they are ROCm devices for RAF's purposes.
     dev_type = DEV_ROCM if t.is_cuda else DEV_CPU
@@ -55,6 +60,7 @@ class _Env:
         self.name = lib.rafhip_raf_env_name(handle).decode()
         self.op = lib.rafhip_raf_env_op(handle).decode()
         self.workspace_bytes = lib.rafhip_raf_env_workspace_bytes(handle)
+        self.workspaces = {}  # stream handle -> runtime.Memory
 
     def __del__(self):
         try:
@@ -65,9 +71,16 @@ class _Env:
 
 def _workspace(env: "_Env", like: torch.Tensor, stream) -> runtime.Memory:
     """The OpEnv's workspace requests as one chunk from the device's memory pool, allocated on the
-    call's stream like the VM does around Execute (src/impl/vm/vm.cc:1099-1105, :846-853)."""
-    dev_id = like.device.index if like.device.index is not None else 0
-    return runtime.Memory(DEV_ROCM, dev_id, env.workspace_bytes, 256, stream, stream_ordered=True)
+    call's stream like the VM does around Execute (src/impl/vm/vm.cc:1099-1105, :846-853).  The
+    chunk is kept with the OpEnv and reused by later calls on the same stream (which run after this
+    one): on ROCm 7.2 a stream-ordered allocation waits for the stream's pending work, which would
+    serialise host and device once per step."""
+    ws = env.workspaces.get(stream)
+    if ws is None:
+        dev_id = like.device.index if like.device.index is not None else 0
+        ws = env.workspaces[stream] = runtime.Memory(DEV_ROCM, dev_id, env.workspace_bytes, 256, stream,
+                                                     stream_ordered=True)
+    return ws
 
 
 _env_cache: Dict[Tuple, _Env] = {}
@@ -75,6 +88,38 @@ _env_cache: Dict[Tuple, _Env] = {}
 
 def clear_op_env_cache() -> None:
     _env_cache.clear()
+    _marshalled.clear()
+
+
+class _Marshalled:
+    """Descriptors, signature and identity of a tensor list that has been handed to an op before."""
+
+    def __init__(self, tensors):
+        self.keep: list = []
+        self.descs = (TensorDesc * max(len(tensors), 1))(*[_desc(t, self.keep) for t in tensors])
+        self.sig = tuple(_sig(t) for t in tensors)
+        self.refs = [weakref.ref(t) for t in tensors]
+        self.ptrs = [t.data_ptr() for t in tensors]
+
+    def still_describes(self, tensors) -> bool:
+        # the same live objects (a weak reference cannot be fooled by a recycled id) at the same
+        # addresses: their shapes and dtypes cannot have changed either
+        return all(r() is t and t.data_ptr() == p for r, t, p in zip(self.refs, tensors, self.ptrs))
+
+
+_marshalled: Dict[Tuple, _Marshalled] = {}
+
+
+def _marshal_list(tensors: list) -> _Marshalled:
+    """Marshalling a list of hundreds of tensors costs milliseconds of Python; a training loop passes
+    the same tensors every step, so the last marshalling of every distinct list is kept."""
+    key = tuple(map(id, tensors))
+    m = _marshalled.get(key)
+    if m is None or not m.still_describes(tensors):
+        if len(_marshalled) >= 8:
+            _marshalled.clear()
+        m = _marshalled[key] = _Marshalled(tensors)
+    return m
 
 
 def _sig(t: torch.Tensor):
@@ -117,10 +162,10 @@ def sgd_multi_mixed(tensor_list: Sequence[torch.Tensor], learning_rate, mu):
 def _sgd_multi(mixed, tensor_list, learning_rate, mu):
     lib = _lib.dialect()
     tensor_list = list(tensor_list)
-    keep: list = []
     n = len(tensor_list)
-    descs = (TensorDesc * max(n, 1))(*[_desc(t, keep) for t in tensor_list])
-    key = ("sgd_multi", mixed, tuple(_sig(t) for t in tensor_list), float(learning_rate), float(mu))
+    m = _marshal_list(tensor_list)
+    descs = m.descs
+    key = ("sgd_multi", mixed, m.sig, float(learning_rate), float(mu))
     env = _env_cache.get(key)
     if env is None:
         h = c_void_p(None)
@@ -157,11 +202,12 @@ def _lans(op_name, tensor_list, step, learning_rate, beta1, beta2, eps, bias_cor
     tensor_list = list(tensor_list)
     keep: list = []
     n4 = len(tensor_list)
-    descs = (TensorDesc * max(n4, 1))(*[_desc(t, keep) for t in tensor_list])
+    m = _marshal_list(tensor_list)
+    descs = m.descs
     dstep = _desc(step, keep)
     hp = (float(learning_rate), float(beta1), float(beta2), float(eps), int(bias_correction),
           float(weight_decay), int(grad_averaging), int(mode), int(bool(normalize_grad)))
-    key = (op_name, tuple(_sig(t) for t in tensor_list), _sig(step), hp, get_lans_grad_unscale())
+    key = (op_name, m.sig, _sig(step), hp, get_lans_grad_unscale())
     env = _env_cache.get(key)
     if env is None:
         h = c_void_p(None)
@@ -172,8 +218,6 @@ def _lans(op_name, tensor_list, step, learning_rate, beta1, beta2, eps, bias_cor
     ws = _workspace(env, tensor_list[0], stream) if env.workspace_bytes > 0 else None
     check_raf(lib.rafhip_raf_lans_execute(env.handle, n4, descs, dstep, ws.data if ws else None,
                                           env.workspace_bytes, stream))
-    if ws:
-        ws.close()  # stream-ordered: the memory goes back to the pool after the step's kernels
     return tensor_list
 
 
@@ -211,8 +255,6 @@ def l2norm(x: torch.Tensor) -> torch.Tensor:
     ws = _workspace(env, x, _stream(x)) if env.workspace_bytes else None
     check_raf(lib.rafhip_raf_l2norm_execute(env.handle, dx, _desc(out, keep), ws.data if ws else None,
                                             env.workspace_bytes, _stream(x)))
-    if ws:
-        ws.close()
     return out
 
 

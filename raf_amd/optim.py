@@ -81,6 +81,10 @@ class LANS:
         self.normalize_grad = normalize_grad
         self.params = []
         self._step = 1  # lans.py:66
+        # The step also lives on the device and is advanced there, like the traced optimizer's
+        # `step` array (lans.py:228, :240): making a fresh device scalar from the host every step
+        # would block on the previous step's kernels.
+        self._step_dev = None
         params = list(params)
         halves = {x.dtype for x in params if isinstance(x, torch.Tensor)} & {torch.float16, torch.bfloat16}
         self.mixed = bool(halves)
@@ -104,9 +108,11 @@ class LANS:
             v_list.append(v)
             p_list.append(x.data)
         if not x_list:
-            self._step += 1
+            self._advance()
             return
-        step = torch.tensor(float(self._step), dtype=torch.float32, device=x_list[0].device)
+        if self._step_dev is None or self._step_dev.device != x_list[0].device:
+            self._step_dev = torch.tensor(float(self._step), dtype=torch.float32, device=x_list[0].device)
+        step = self._step_dev
         tensor_list = g_list + x_list + m_list + v_list  # lans.py:89
         hyper = (self.lr, self.beta1, self.beta2, self.eps, self.bias_correction, self.weight_decay,
                  self.grad_averaging, self.mode, self.normalize_grad)
@@ -114,4 +120,9 @@ class LANS:
             _op.lans_mixed(tensor_list + p_list, step, *hyper)
         else:
             _op.lans(tensor_list, step, *hyper)
+        self._advance()
+
+    def _advance(self):
         self._step += 1
+        if self._step_dev is not None:
+            self._step_dev.add_(1.0)
