@@ -82,6 +82,15 @@ struct GradIO<float> {
   static __device__ __forceinline__ float load1(const void* g, int64_t i, float us) {
     return ((const RAFHIP_GLOBAL float*)g)[i] * us;
   }
+  // The same split in two, so that a load can be issued well before its value is needed.
+  typedef f32x4 Raw4;
+  template <bool kNT>
+  static __device__ __forceinline__ Raw4 load_raw4(const void* g, int64_t i4) {
+    return ldg<kNT>((const RAFHIP_GLOBAL f32x4*)g + i4);
+  }
+  static __device__ __forceinline__ f32x4 widen4(const Raw4& r, float us) {
+    return f32x4{r.x * us, r.y * us, r.z * us, r.w * us};
+  }
 };
 
 template <>
@@ -101,6 +110,14 @@ struct GradIO<_Float16> {
   }
   static __device__ __forceinline__ float load1(const void* g, int64_t i, float us) {
     return (float)((const RAFHIP_GLOBAL _Float16*)g)[i] * us;
+  }
+  typedef f16x4 Raw4;
+  template <bool kNT>
+  static __device__ __forceinline__ Raw4 load_raw4(const void* g, int64_t i4) {
+    return ldg<kNT>((const RAFHIP_GLOBAL f16x4*)g + i4);
+  }
+  static __device__ __forceinline__ f32x4 widen4(const Raw4& r, float us) {
+    return f32x4{(float)r.x * us, (float)r.y * us, (float)r.z * us, (float)r.w * us};
   }
 };
 
@@ -122,6 +139,15 @@ struct GradIO<Bf16> {
   }
   static __device__ __forceinline__ float load1(const void* g, int64_t i, float us) {
     return bf16_widen(((const RAFHIP_GLOBAL unsigned short*)g)[i]) * us;
+  }
+  typedef u16x4 Raw4;
+  template <bool kNT>
+  static __device__ __forceinline__ Raw4 load_raw4(const void* g, int64_t i4) {
+    return ldg<kNT>((const RAFHIP_GLOBAL u16x4*)g + i4);
+  }
+  static __device__ __forceinline__ f32x4 widen4(const Raw4& r, float us) {
+    return f32x4{bf16_widen(r.x) * us, bf16_widen(r.y) * us, bf16_widen(r.z) * us,
+                 bf16_widen(r.w) * us};
   }
 };
 

@@ -33,6 +33,7 @@ constexpr CachePolicy kPhasedPolicy = {true, false, true, false, true, true};
 // of the group reads them another round later; pass C reads non-temporally (a hit is consumed, not
 // kept) and writes non-temporally.  Measured best of nine combinations.
 constexpr CachePolicy kPipelinedPolicy = {false, true, false, true, true, true};
+constexpr bool kPipelinedAhead = true;  // issue the next trip's loads before evaluating this one
 // Lists whose whole working set fits in the cache (a few million elements) are better off cached.
 constexpr CachePolicy kResidentPolicy = {false, false, false, false, false, false};
 
@@ -265,18 +266,20 @@ __device__ __forceinline__ double chunk_sum_g(const ChunkView& cv, float unscale
 
 // ------------------------------------------------------------------ passes B and C: shared loads
 // One trip's worth of the four arrays for one lane: kUnroll groups of 4 consecutive elements.
+// The gradient stays as loaded (widening it would wait for the load) until the trip is evaluated.
+template <typename G>
 struct Batch {
-  f32x4 g[kUnroll], w[kUnroll], m[kUnroll], v[kUnroll];
+  typename GradIO<G>::Raw4 g[kUnroll];
+  f32x4 w[kUnroll], m[kUnroll], v[kUnroll];
 };
 
 template <typename G, bool kGradNT, bool kNT>
-__device__ __forceinline__ void load_batch(Batch& b, const ChunkView& cv, int i0, int n4,
-                                           float unscale) {
+__device__ __forceinline__ void load_batch(Batch<G>& b, const ChunkView& cv, int i0, int n4) {
 #pragma unroll
   for (int u = 0; u < kUnroll; ++u) {
     const int i = i0 + u * kLansBlock;
     if (i < n4) {
-      b.g[u] = GradIO<G>::template load4<kGradNT>(cv.g, i, unscale);
+      b.g[u] = GradIO<G>::template load_raw4<kGradNT>(cv.g, i);
       b.w[u] = ldg<kNT>((gc_float4*)cv.w + i);
       b.m[u] = ldg<kNT>((gc_float4*)cv.m + i);
       b.v[u] = ldg<kNT>((gc_float4*)cv.v + i);
@@ -284,37 +287,58 @@ __device__ __forceinline__ void load_batch(Batch& b, const ChunkView& cv, int i0
   }
 }
 
+// Walks the 4-element groups of a chunk trip by trip and hands each loaded trip to `body`.  With
+// kAhead the loads of trip i+1 are issued before trip i is evaluated: one more trip of registers
+// (32 VGPRs), which the persistent kernel has to spare at three workgroups per CU.
+template <typename G, bool kGradNT, bool kNT, bool kAhead, typename Body>
+__device__ __forceinline__ void for_each_trip(const ChunkView& cv, int n4, Body&& body) {
+  constexpr int kStride = kLansBlock * kUnroll;
+  if constexpr (kAhead) {
+    Batch<G> nxt;
+    load_batch<G, kGradNT, kNT>(nxt, cv, (int)threadIdx.x, n4);
+    for (int i0 = threadIdx.x; i0 < n4; i0 += kStride) {
+      const Batch<G> cur = nxt;
+      load_batch<G, kGradNT, kNT>(nxt, cv, i0 + kStride, n4);  // guarded per lane by i < n4
+      body(cur, i0);
+    }
+  } else {
+    for (int i0 = threadIdx.x; i0 < n4; i0 += kStride) {
+      Batch<G> cur;
+      load_batch<G, kGradNT, kNT>(cur, cv, i0, n4);
+      body(cur, i0);
+    }
+  }
+}
+
 // ------------------------------------------------------------------ pass B on one chunk
 // Per-thread contributions to sum u_m^2, sum u_g^2 and sum w^2.  `get_inv_gdiv` supplies the
 // tensor's gradient divisor (the pipelined schedule may have to wait for it).
-// (Issuing trip i+1's loads before evaluating trip i was tried: the extra registers cost a wave of
-// occupancy and the kernels got slower.)
-template <typename G, bool kGradNT, bool kNT, typename GetInvGdiv>
+// (In the one-launch-per-pass kernels, issuing trip i+1's loads before evaluating trip i costs a
+// wave of occupancy and makes them slower; the persistent kernel has the registers to spare.)
+template <typename G, bool kGradNT, bool kNT, bool kAhead = false, typename GetInvGdiv>
 __device__ __forceinline__ void chunk_sums_u(const ChunkView& cv, float unscale,
                                              const StepScalars& k, GetInvGdiv&& get_inv_gdiv,
                                              double (&sums)[3]) {
   double am = 0.0, au = 0.0, aw = 0.0;
   if (cv.vec_ok) {
     const int n4 = cv.len >> 2;
-    constexpr int kStride = kLansBlock * kUnroll;
     const double inv_gdiv = get_inv_gdiv();
-    for (int i0 = threadIdx.x; i0 < n4; i0 += kStride) {
-      Batch cur;
-      load_batch<G, kGradNT, kNT>(cur, cv, i0, n4, unscale);
+    for_each_trip<G, kGradNT, kNT, kAhead>(cv, n4, [&](const Batch<G>& cur, int i0) {
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
         if (i0 + u * kLansBlock < n4) {
-          const Directions d0 = lans_directions(cur.g[u].x, cur.w[u].x, cur.m[u].x, cur.v[u].x, inv_gdiv, k);
-          const Directions d1 = lans_directions(cur.g[u].y, cur.w[u].y, cur.m[u].y, cur.v[u].y, inv_gdiv, k);
-          const Directions d2 = lans_directions(cur.g[u].z, cur.w[u].z, cur.m[u].z, cur.v[u].z, inv_gdiv, k);
-          const Directions d3 = lans_directions(cur.g[u].w, cur.w[u].w, cur.m[u].w, cur.v[u].w, inv_gdiv, k);
+          const f32x4 g = GradIO<G>::widen4(cur.g[u], unscale);
+          const Directions d0 = lans_directions(g.x, cur.w[u].x, cur.m[u].x, cur.v[u].x, inv_gdiv, k);
+          const Directions d1 = lans_directions(g.y, cur.w[u].y, cur.m[u].y, cur.v[u].y, inv_gdiv, k);
+          const Directions d2 = lans_directions(g.z, cur.w[u].z, cur.m[u].z, cur.v[u].z, inv_gdiv, k);
+          const Directions d3 = lans_directions(g.w, cur.w[u].w, cur.m[u].w, cur.v[u].w, inv_gdiv, k);
           am += (d0.um * d0.um + d1.um * d1.um) + (d2.um * d2.um + d3.um * d3.um);
           au += (d0.ug * d0.ug + d1.ug * d1.ug) + (d2.ug * d2.ug + d3.ug * d3.ug);
           aw += ((double)cur.w[u].x * (double)cur.w[u].x + (double)cur.w[u].y * (double)cur.w[u].y) +
                 ((double)cur.w[u].z * (double)cur.w[u].z + (double)cur.w[u].w * (double)cur.w[u].w);
         }
       }
-    }
+    });
     const int tail = (n4 << 2) + threadIdx.x;
     if (tail < cv.len) {
       const double wx = ((gc_float*)cv.w)[tail];
@@ -362,24 +386,22 @@ __device__ __forceinline__ Applied apply_one(double g, double w, double m, doubl
 }
 
 // `get_params` supplies the tensor's divisor and trust ratios.
-template <typename G, bool kGradNT, bool kNT, bool kStoreNT, typename GetParams>
+template <typename G, bool kGradNT, bool kNT, bool kStoreNT, bool kAhead = false, typename GetParams>
 __device__ __forceinline__ void chunk_apply(const ChunkView& cv, float unscale, bool p_is_bf16,
                                             const StepScalars& k, GetParams&& get_params) {
   if (cv.vec_ok) {
     const int n4 = cv.len >> 2;
-    constexpr int kStride = kLansBlock * kUnroll;
     const ApplyParams p = get_params();
-    for (int i0 = threadIdx.x; i0 < n4; i0 += kStride) {
-      Batch cur;
-      load_batch<G, kGradNT, kNT>(cur, cv, i0, n4, unscale);
+    for_each_trip<G, kGradNT, kNT, kAhead>(cv, n4, [&](const Batch<G>& cur, int i0) {
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
         const int i = i0 + u * kLansBlock;
         if (i < n4) {
-          const Applied a0 = apply_one(cur.g[u].x, cur.w[u].x, cur.m[u].x, cur.v[u].x, p, k);
-          const Applied a1 = apply_one(cur.g[u].y, cur.w[u].y, cur.m[u].y, cur.v[u].y, p, k);
-          const Applied a2 = apply_one(cur.g[u].z, cur.w[u].z, cur.m[u].z, cur.v[u].z, p, k);
-          const Applied a3 = apply_one(cur.g[u].w, cur.w[u].w, cur.m[u].w, cur.v[u].w, p, k);
+          const f32x4 g = GradIO<G>::widen4(cur.g[u], unscale);
+          const Applied a0 = apply_one(g.x, cur.w[u].x, cur.m[u].x, cur.v[u].x, p, k);
+          const Applied a1 = apply_one(g.y, cur.w[u].y, cur.m[u].y, cur.v[u].y, p, k);
+          const Applied a2 = apply_one(g.z, cur.w[u].z, cur.m[u].z, cur.v[u].z, p, k);
+          const Applied a3 = apply_one(g.w, cur.w[u].w, cur.m[u].w, cur.v[u].w, p, k);
           stg<kStoreNT>((g_float4*)cv.w + i, f32x4{a0.w, a1.w, a2.w, a3.w});
           stg<kStoreNT>((g_float4*)cv.m + i, f32x4{a0.m, a1.m, a2.m, a3.m});
           stg<kStoreNT>((g_float4*)cv.v + i, f32x4{a0.v, a1.v, a2.v, a3.v});
@@ -389,7 +411,7 @@ __device__ __forceinline__ void chunk_apply(const ChunkView& cv, float unscale, 
                                 narrow16(a2.w, p_is_bf16), narrow16(a3.w, p_is_bf16)});
         }
       }
-    }
+    });
     const int tail = (n4 << 2) + threadIdx.x;
     if (tail < cv.len) {
       const Applied o = apply_one(GradIO<G>::load1(cv.g, tail, unscale), ((gc_float*)cv.w)[tail],
@@ -676,7 +698,7 @@ __global__ __launch_bounds__(kLansBlock) void lans_pipelined(LansDeviceArgs a) {
       if (threadIdx.x == 0) stats_after_a(st, tot[0], k);
     } else if (phase == kPhaseB) {
       double s[3];
-      chunk_sums_u<G, kPipelinedPolicy.b_g, kPipelinedPolicy.b_wmv>(cv, a.unscale, k,
+      chunk_sums_u<G, kPipelinedPolicy.b_g, kPipelinedPolicy.b_wmv, kPipelinedAhead>(cv, a.unscale, k,
                       [&] { return wait_published(&st->inv_grad_div, a.sync); }, s);
       block_sum<3>(s, red);
       if (threadIdx.x == 0) {
@@ -689,7 +711,7 @@ __global__ __launch_bounds__(kLansBlock) void lans_pipelined(LansDeviceArgs a) {
       tensor_totals<3, true>(tensor_part, 1, n_chunks, 1, tot, red, a.sync);
       if (threadIdx.x == 0) stats_after_b(st, tot, k, r0, r1);
     } else if (phase == kPhaseC) {
-      chunk_apply<G, kPipelinedPolicy.c_g, kPipelinedPolicy.c_wmv, kPipelinedPolicy.c_stores>(
+      chunk_apply<G, kPipelinedPolicy.c_g, kPipelinedPolicy.c_wmv, kPipelinedPolicy.c_stores, kPipelinedAhead>(
           cv, a.unscale, a.p_is_bf16 != 0, k, [&] {
         const double* const words[3] = {&st->inv_grad_div, &st->ratio_m, &st->ratio_g};
         double val[3];
