@@ -128,7 +128,8 @@ struct TensorStats {  // 64 bytes = 8 words, one per tensor; "not ready" pattern
 struct SyncHeader {
   uint32_t ticket;  // next work item
   uint32_t error;   // 1 if a bounded wait ran out
-  uint32_t pad[2];
+  uint32_t spin_limit;  // polls a wait may take before it gives up
+  uint32_t pad;
 };
 
 struct HParamsPod {
@@ -145,6 +146,7 @@ struct LansDeviceArgs {
   int64_t n_items_a;
   uint32_t n_items;       // pipelined work-list length
   const WorkItem* pipeline_items;
+  uint32_t spin_limit;    // pipelined: bound of every wait, in polls
   float unscale;
   int32_t p_is_bf16;      // dtype of the optional 16-bit weight copies: 0 binary16, 1 bfloat16
   StepScalars* scalars;

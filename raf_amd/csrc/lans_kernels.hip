@@ -82,7 +82,6 @@ __device__ __forceinline__ void st_dev(double* p, double v) {
 }
 
 constexpr uint64_t kNotReady = 0xFFFFFFFFFFFFFFFFull;
-constexpr uint32_t kSpinLimit = 1u << 22;  // bounded wait: far beyond any real dependency latency
 
 __device__ __forceinline__ uint64_t ld_bits(const double* p) {
   return __hip_atomic_load(reinterpret_cast<const uint64_t*>(p), __ATOMIC_RELAXED,
@@ -102,7 +101,7 @@ __device__ __forceinline__ double wait_published(const double* word, SyncHeader*
   uint64_t bits = ld_bits(word);
   uint32_t spins = 0;
   while (bits == kNotReady) {
-    if (++spins > kSpinLimit) {
+    if (++spins > sync->spin_limit) {
       __hip_atomic_store(&sync->error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       break;
     }
@@ -489,6 +488,7 @@ __device__ __forceinline__ void write_step_scalars(const LansDeviceArgs& a, cons
                                                    int32_t step_host, const HParamsPod& hp) {
   a.sync->ticket = 0u;
   a.sync->error = 0u;
+  a.sync->spin_limit = a.spin_limit;
   const int step = step_dev ? (int)(*step_dev) : step_host;
   float bc1 = 1.0f, bc2 = 1.0f;
   if (hp.bias_correction == 1) {  // double pow, then one rounding to fp32 (lans.cc:103-104)

@@ -111,6 +111,17 @@ int64_t group_elems_setting() {
   return kDefaultGroupElems;
 }
 
+// Polls a wait of the pipelined kernel may take before it gives up and raises the error word:
+// with a sleep of a few hundred cycles per poll the default is seconds, far beyond any real
+// dependency latency.  RAFHIP_LANS_SPIN_LIMIT overrides it (tests force a time-out with 0).
+uint32_t spin_limit_setting() {
+  if (const char* e = std::getenv("RAFHIP_LANS_SPIN_LIMIT")) {
+    const long long v = std::atoll(e);
+    if (v >= 0 && v <= 0xFFFFFFFFll) return (uint32_t)v;
+  }
+  return 1u << 22;
+}
+
 int schedule_setting(int64_t total_elements) {
   if (const char* e = std::getenv("RAFHIP_LANS_SCHEDULE")) {
     if (!std::strcmp(e, "phased")) return RAFHIP_LANS_PHASED;
@@ -129,6 +140,7 @@ struct rafhip_lans_plan {
   int32_t schedule = RAFHIP_LANS_PHASED;
   int64_t n_chunks = 0;
   int64_t total_elements = 0;
+  uint32_t spin_limit = 1u << 22;
   bool short_tensors_only = false;  // no tensor has more than kInlineFinishChunks chunks
   uint32_t n_pipeline_items = 0;
   unsigned pipeline_grid = 0;
@@ -271,6 +283,7 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
   p->n_chunks = chunks;
   p->total_elements = total;
   p->schedule = schedule_setting(total);
+  p->spin_limit = spin_limit_setting();
   p->ws = make_layout(n_tensors, chunks);
 
   if (hipGetDevice(&p->device) != hipSuccess) {
@@ -449,6 +462,7 @@ int rafhip_lans_step_mixed(rafhip_lans_plan* plan, const void* const* g, float* 
   a.n_items = plan->n_pipeline_items;
   a.pipeline_items = plan->d_pipeline;
   a.unscale = hp->grad_unscale;
+  a.spin_limit = plan->spin_limit;
   a.p_is_bf16 = p_dtype == RAFHIP_BF16 ? 1 : 0;
   a.scalars = reinterpret_cast<StepScalars*>(ws + plan->ws.scalars_off);
   a.stats = reinterpret_cast<TensorStats*>(ws + plan->ws.stats_off);

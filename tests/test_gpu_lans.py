@@ -364,3 +364,33 @@ def test_same_tensors_on_another_stream(native_libs):
     torch.cuda.synchronize()
     _assert_close([t.cpu().numpy() for t in tw], ow, TOL_1, "w")
     plan.close()
+
+
+def test_a_wait_that_runs_out_is_reported_not_hung(native_libs, monkeypatch):
+    """Every wait of the persistent kernel is bounded.  With the bound forced to zero polls from the
+    host, waits give up at once: the kernel still drains, the step's results are declared invalid by
+    rafhip_lans_read_norms, and the next plan (default bound) works as usual."""
+    from raf_amd import kernels
+
+    sizes = [1 << 22, 3 << 20, 70001]
+    g, w, m, v = lans_inputs(sizes, cfg=87)
+    hp = LansHParams()
+    monkeypatch.setenv("RAFHIP_LANS_SPIN_LIMIT", "0")
+    tg, tw, tm, tv = _to_dev(g), _to_dev(w), _to_dev(m), _to_dev(v)
+    plan = kernels.LansPlan(sizes, torch.float32, DEV)
+    plan.set_schedule("pipelined")
+    plan.step(tg, tw, tm, tv, 1, _khp(hp))
+    torch.cuda.synchronize()  # returns: no workgroup is left waiting
+    with pytest.raises(native_libs.RafHipError, match="bounded wait"):
+        plan.read_norms()
+    plan.close()
+    monkeypatch.delenv("RAFHIP_LANS_SPIN_LIMIT")
+    tg, tw, tm, tv = _to_dev(g), _to_dev(w), _to_dev(m), _to_dev(v)
+    plan = kernels.LansPlan(sizes, torch.float32, DEV)
+    plan.set_schedule("pipelined")
+    plan.step(tg, tw, tm, tv, 1, _khp(hp))
+    torch.cuda.synchronize()
+    ow, _, _, on = lans_f64.lans_step(g, w, m, v, 1, hp)
+    _assert_norms(plan.read_norms(), on)
+    _assert_close([t.cpu().numpy() for t in tw], ow, TOL_1, "w")
+    plan.close()
