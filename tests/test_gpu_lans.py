@@ -394,3 +394,37 @@ def test_a_wait_that_runs_out_is_reported_not_hung(native_libs, monkeypatch):
     _assert_norms(plan.read_norms(), on)
     _assert_close([t.cpu().numpy() for t in tw], ow, TOL_1, "w")
     plan.close()
+
+
+@pytest.mark.parametrize("bad", [np.inf, np.nan])
+def test_overflowed_gradient_poisons_only_its_tensor(native_libs, bad):
+    """A loss-scale overflow leaves inf / NaN in a half gradient.  The rule then turns that tensor's
+    w, m, v into NaN (as the reference's arithmetic would); the other tensors are untouched by it,
+    both schedules agree on where the NaNs are, and the persistent kernel's waits are not confused
+    by NaN partial sums (its 'not ready' pattern is itself a NaN)."""
+    from raf_amd import kernels
+
+    sizes = [30000, 70001, 9000]
+    hp = LansHParams(grad_unscale=1 / 1024)
+    g, w, m, v = lans_inputs(sizes, cfg=88, g16=True)
+    g[1][12345] = np.float16(bad)
+    ow, om, ov, on = lans_f64.lans_step(g, w, m, v, 2, hp)
+    assert np.isnan(ow[1]).all() and not np.isnan(ow[0]).any() and not np.isnan(ow[2]).any()
+    outs = {}
+    for schedule in ("phased", "pipelined"):
+        tg, tw, tm, tv = _to_dev(g), _to_dev(w), _to_dev(m), _to_dev(v)
+        plan = kernels.LansPlan(sizes, torch.float16, DEV)
+        plan.set_schedule(schedule)
+        plan.step(tg, tw, tm, tv, 2, _khp(hp))
+        torch.cuda.synchronize()
+        norms = plan.read_norms()
+        outs[schedule] = [t.cpu().numpy() for t in tw + tm + tv]
+        plan.close()
+        for q, want in zip((0, 3, 6), (ow, om, ov)):
+            got = outs[schedule][q:q + 3]
+            assert np.array_equal(np.isnan(got[1]), np.isnan(want[1]))
+            _assert_close([got[0], got[2]], [want[0], want[2]], TOL_1, schedule)
+        assert np.isnan(norms[1][0]) or np.isinf(norms[1][0])
+        _assert_norms(norms[[0, 2]], on[[0, 2]])
+    for a, b in zip(outs["phased"], outs["pipelined"]):
+        assert np.array_equal(a, b, equal_nan=True)
