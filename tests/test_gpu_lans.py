@@ -428,3 +428,33 @@ def test_overflowed_gradient_poisons_only_its_tensor(native_libs, bad):
         _assert_norms(norms[[0, 2]], on[[0, 2]])
     for a, b in zip(outs["phased"], outs["pipelined"]):
         assert np.array_equal(a, b, equal_nan=True)
+
+
+def test_two_persistent_kernels_side_by_side(native_libs):
+    """Two plans stepping on two streams at once share the CUs.  A waiting workgroup only ever
+    depends on items with earlier tickets, which running workgroups hold, so neither kernel needs
+    all of its workgroups resident; both must finish and match the oracle."""
+    from raf_amd import kernels
+
+    hp = LansHParams()
+    lists = [[1 << 22, 3 << 20, 70001, 1 << 21], [5 << 20, 1 << 20, 9, 1 << 22]]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    state = []
+    for cfg, sizes in enumerate(lists):
+        g, w, m, v = lans_inputs(sizes, cfg=89 + cfg)
+        plan = kernels.LansPlan(sizes, torch.float32, DEV)
+        plan.set_schedule("pipelined")
+        state.append((g, w, m, v, plan, _to_dev(g), _to_dev(w), _to_dev(m), _to_dev(v)))
+    torch.cuda.synchronize()
+    for step in (1, 2, 3):
+        for (g, w, m, v, plan, tg, tw, tm, tv), s in zip(state, streams):
+            with torch.cuda.stream(s):
+                plan.step(tg, tw, tm, tv, step, _khp(hp))
+    torch.cuda.synchronize()
+    for g, w, m, v, plan, tg, tw, tm, tv in state:
+        ow, om, ov = w, m, v
+        for step in (1, 2, 3):
+            ow, om, ov, on = lans_f64.lans_step(g, ow, om, ov, step, hp)
+        _assert_norms(plan.read_norms(), on)
+        _assert_close([t.cpu().numpy() for t in tw], ow, TOL_1, "w")
+        plan.close()
