@@ -73,6 +73,8 @@ def workloads():
                                     zero_state=True, step0=1),
         "sgd_4m_fp32": dict(kind="sgd", n=4_194_304),
         "sgd_multi_bert_large_fp32": dict(kind="sgd_multi", sizes=shapes.numels(shapes.bert_large_shapes())),
+        # the traced optimizer's per-parameter op sequence after dialect fusion: one fused call per parameter
+        "traced_sgd_fused_bert_large_fp32": dict(kind="traced_sgd", sizes=shapes.numels(shapes.bert_large_shapes())),
         # neighbours of the optimizer step that reuse its machinery
         "l2norm_bert_large_flat_fp32": dict(kind="l2norm", n=sum(shapes.numels(shapes.bert_large_shapes()))),
         "fuse_bert_large_fp32": dict(kind="fuse", sizes=shapes.numels(shapes.bert_large_shapes()), gather=True),
@@ -452,6 +454,40 @@ def bench_copy(name, wl, args):
                          "traffic": None, "bytes_per_launch": moved, "avg_launch_ms": round(dev_ms, 4)}}
 
 
+def bench_traced_sgd(name, wl, args):
+    """One step = the traced SGD update of every parameter, each parameter's add/multiply/subtract
+    sequence fused by the dialect pass into one primitive function and run as one launch."""
+    import torch
+
+    from raf_amd import op
+
+    dev = torch.device("cuda:0")
+    sizes = wl["sizes"]
+    total = sum(sizes)
+    gen = torch.Generator(dev).manual_seed(2024)
+    x = [torch.randn(n, device=dev, generator=gen) * 0.02 for n in sizes]
+    dx = [torch.randn(n, device=dev, generator=gen) * 1e-3 for n in sizes]
+    v = [torch.zeros(n, device=dev) for n in sizes]
+
+    updates = [op.TracedSgdUpdate(w_, d_, v_, 0.01, 0.9) for w_, d_, v_ in zip(x, dx, v)]
+
+    def step(_):
+        for upd in updates:
+            upd()
+
+    wall_ms, dev_ms = _timed(step, args)
+    res = _line("traced SGD update after dialect fusion, achieved HBM bandwidth (algorithmic bytes / step time)",
+                name, "f32", total * SGD_BYTES_PER_ELT, wall_ms, dev_ms, "sgd_vec4_kernel", args,
+                {"tensors": len(sizes), "elements": total, "bytes_per_element": SGD_BYTES_PER_ELT,
+                 "launches_per_step": len(sizes), "unfused_kernels_per_step": 4 * len(sizes)})
+    # the roofline object is about one launch of the dominant kernel; here a step is many launches of
+    # different sizes, so the step as a whole stands in for it
+    res["roofline"]["note"] = "whole step (one launch per parameter), not a single launch"
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline_sgd(1 << 24)
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -480,7 +516,7 @@ def main():
     _lib.optim()  # fails loudly if the HIP library is not built
     wl = table[args.workload]
     fn = {"lans": bench_lans, "sgd": bench_sgd, "copy": bench_copy, "l2norm": bench_l2norm,
-          "fuse": bench_fuse, "sgd_multi": bench_sgd_multi}[wl["kind"]]
+          "fuse": bench_fuse, "sgd_multi": bench_sgd_multi, "traced_sgd": bench_traced_sgd}[wl["kind"]]
     out = fn(args.workload, wl, args)
     print(json.dumps(out), flush=True)
 

@@ -157,6 +157,26 @@ int rafhip_raf_pool_info(int32_t device_type, int32_t device_id, char* name_buf,
 /* Memory::GetAllocBytes: what a request of nbytes really takes from the pool; -1 on error. */
 int64_t rafhip_raf_pool_alloc_bytes(int32_t device_type, int32_t device_id, int64_t nbytes);
 
+/* Dialect fusion.  The reference's traced SGD optimizer emits, per parameter,
+ *     new_v = add(multiply(momentum, v), dx, out=v)
+ *     new_w = subtract(w, multiply(learning_rate, new_v), out=w)
+ * with a cast(dx, "float32") in front for 16-bit gradients (python/raf/optim/sgd.py:192-200).
+ * rafhip_raf_traced_sgd_make builds that graph for one parameter from the descriptors' types, runs
+ * the FuseDialect pass (src/pass/fuse_dialect.cc:179-198) for their device type with the `hip`
+ * dialect's "sgd_update" pattern, and dispatches the fused function the way
+ * DispatchFusedOp does (src/impl/op.cc:182-203: maker raf.op.hip._fused_op).  If nothing fuses
+ * (other device, other dtypes) it fails like a dispatch with no backend, and *env_out still
+ * holds the graphs for rafhip_raf_env_ir_text.  _execute runs the fused function IN PLACE on w
+ * and v (that is what out= means) as one kernel launch.
+ * rafhip_raf_env_ir_text copies the text of the graph before (fused = 0) or after the pass. */
+int rafhip_raf_traced_sgd_make(const rafhip_tensor_desc* w, const rafhip_tensor_desc* dx,
+                               const rafhip_tensor_desc* v, double learning_rate, double momentum,
+                               rafhip_raf_env** env_out);
+int rafhip_raf_traced_sgd_execute(rafhip_raf_env* env, const rafhip_tensor_desc* w,
+                                  const rafhip_tensor_desc* dx, const rafhip_tensor_desc* v,
+                                  void* stream);
+int rafhip_raf_env_ir_text(const rafhip_raf_env* env, int32_t fused, char* buf, int32_t buflen);
+
 /* Total bytes of the OpEnv's workspace requests (each rounded up to 256). */
 int64_t rafhip_raf_env_workspace_bytes(const rafhip_raf_env* env);
 /* OpEnv::name() and the dialect op the dispatcher picked; pointers stay valid until destroy. */

@@ -167,6 +167,10 @@ DIALECT_SYMBOLS = {
     "rafhip_raf_pool_info": (c_int, [c_int32, c_int32, c_char_p, c_int32, POINTER(c_float), POINTER(c_float)]),
     "rafhip_raf_pool_alloc_bytes": (c_int64, [c_int32, c_int32, c_int64]),
     "rafhip_raf_env_workspace_bytes": (c_int64, [c_void_p]),
+    "rafhip_raf_traced_sgd_make": (c_int, [POINTER(TensorDesc), POINTER(TensorDesc), POINTER(TensorDesc),
+                                           c_double, c_double, POINTER(c_void_p)]),
+    "rafhip_raf_traced_sgd_execute": (c_int, [c_void_p] + [POINTER(TensorDesc)] * 3 + [c_void_p]),
+    "rafhip_raf_env_ir_text": (c_int, [c_void_p, c_int32, c_char_p, c_int32]),
     "rafhip_raf_env_name": (c_char_p, [c_void_p]),
     "rafhip_raf_env_op": (c_char_p, [c_void_p]),
     "rafhip_raf_env_destroy": (c_int, [c_void_p]),

@@ -31,7 +31,7 @@ HIP_FLAGS = [
 OPTIM_SOURCES = ["status.hip", "sgd.hip", "lans_kernels.hip", "lans_plan.hip", "l2norm.hip", "fuse_tensor.hip",
                  "device_rt.hip"]
 DIALECT_SOURCES = ["dialect/registry.cc", "dialect/device_api.cc", "dialect/memory_pool.cc", "dialect/hip_dialect.cc",
-                   "dialect/c_api.cc"]
+                   "dialect/raf_ir.cc", "dialect/hip_fusion.cc", "dialect/c_api.cc"]
 
 
 def hipcc() -> str:

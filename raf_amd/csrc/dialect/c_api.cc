@@ -7,6 +7,7 @@
 #include "hip_dialect.h"
 #include "memory_pool.h"
 #include "raf_iface.h"
+#include "raf_ir.h"
 #include "rafhip_dialect.h"
 
 using namespace raf;
@@ -21,6 +22,10 @@ struct rafhip_raf_env {
   CallValues call;
   std::string name;
   std::string op;
+  // Only for an env made from a graph (rafhip_raf_traced_sgd_make): the graph before and after
+  // the FuseDialect pass and the variables to bind at Execute time.
+  ir::Expr traced, fused;
+  std::vector<ir::Expr> vars;
 };
 
 namespace {
@@ -525,6 +530,74 @@ int64_t rafhip_raf_env_workspace_bytes(const rafhip_raf_env* env) {
   int64_t need = 0;
   for (const auto& r : env->env->workspace_requests()) need += RoundUp(r.nbytes);
   return need;
+}
+
+int rafhip_raf_traced_sgd_make(const rafhip_tensor_desc* w, const rafhip_tensor_desc* dx,
+                               const rafhip_tensor_desc* v, double learning_rate, double momentum,
+                               rafhip_raf_env** env_out) {
+  return Guard([&] {
+    if (!env_out) throw Error("rafhip_raf_traced_sgd_make: env_out is NULL");
+    *env_out = nullptr;
+    const rafhip_tensor_desc* descs[3] = {w, dx, v};
+    const char* names[3] = {"w", "dx", "v"};
+    std::unique_ptr<rafhip_raf_env> h(new rafhip_raf_env());
+    std::map<const ir::ExprNode*, value::Value> bindings;
+    for (int i = 0; i < 3; ++i) {
+      value::TensorValue t = FromDesc(descs[i], names[i]);
+      ir::TensorType ty;
+      ty.defined = true;
+      ty.shape = t->tensor.shape;
+      ty.dtype = t->tensor.dtype;
+      h->vars.push_back(ir::MakeVar(names[i], ty));
+      bindings[h->vars.back().get()] = t;
+    }
+    const Device device = value::AsTensor(bindings[h->vars[0].get()])->tensor.device;
+    h->traced = hip::TracedSgdUpdate(h->vars[0], h->vars[1], h->vars[2], learning_rate, momentum);
+    h->fused = pass::FuseDialect(h->traced, device.device_type());
+    const auto* call = ir::AsCall(h->fused);
+    if (!call || !ir::AsFunction(call->op)) {
+      // Nothing was fused; the element-wise base ops have no backend in this library.
+      *env_out = h.release();
+      throw Error("Cannot find a valid dispatch for op " + ir::AsOp(ir::AsCall((*env_out)->traced)->op)->name +
+                  ": no fuse pattern matched on device type " + device.device_type().c_str());
+    }
+    h->call = BindCall(h->fused, bindings, device);
+    h->env = Dispatch(h->call);
+    h->name = h->env->name();
+    h->op = "raf.op." + ir::AsFunction(call->op)->attrs.at(ir::kDialect) + "._fused_op";
+    *env_out = h.release();
+  });
+}
+
+int rafhip_raf_traced_sgd_execute(rafhip_raf_env* env, const rafhip_tensor_desc* w,
+                                  const rafhip_tensor_desc* dx, const rafhip_tensor_desc* v,
+                                  void* stream) {
+  return Guard([&] {
+    if (!env || !env->env || env->vars.size() != 3)
+      throw Error("rafhip_raf_traced_sgd_execute: env was not made by rafhip_raf_traced_sgd_make");
+    std::map<const ir::ExprNode*, value::Value> bindings;
+    value::TensorValue wt = FromDesc(w, "w");
+    bindings[env->vars[0].get()] = wt;
+    bindings[env->vars[1].get()] = FromDesc(dx, "dx");
+    bindings[env->vars[2].get()] = FromDesc(v, "v");
+    CallValues call = BindCall(env->fused, bindings, env->call->device);
+    call->out = wt;  // out=w: the result shares w's memory (src/op/declare/binary.cc:52-55)
+    OpEnv::SetStreamForAllBackends(call->device, stream);
+    WorkspaceBinding bind(env->env.get(), nullptr, 0);
+    // the executors hand a fused function all of its arguments (arg_indices covers them all)
+    env->env->Execute(call->args_as<schema::ListArgs>()->args, call->out);
+  });
+}
+
+int rafhip_raf_env_ir_text(const rafhip_raf_env* env, int32_t fused, char* buf, int32_t buflen) {
+  return Guard([&] {
+    if (!env || !buf || buflen <= 0) throw Error("rafhip_raf_env_ir_text: bad arguments");
+    const ir::Expr& e = fused ? env->fused : env->traced;
+    if (!e) throw Error("rafhip_raf_env_ir_text: env was not made from a graph");
+    std::string s = ir::AsText(e);
+    if ((int64_t)s.size() >= (int64_t)buflen) throw Error("rafhip_raf_env_ir_text: buffer too small");
+    std::memcpy(buf, s.c_str(), s.size() + 1);
+  });
 }
 
 const char* rafhip_raf_env_name(const rafhip_raf_env* env) { return env ? env->name.c_str() : ""; }

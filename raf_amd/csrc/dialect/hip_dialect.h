@@ -1,6 +1,10 @@
 // Knobs of the `hip` dialect that have no field in the reference's schemas.
 #pragma once
 
+#include <string>
+
+#include "raf_ir.h"
+
 namespace raf {
 namespace op {
 namespace hip {
@@ -10,6 +14,26 @@ namespace hip {
 // has no such field: there, gradients are cast and unscaled by separate ops before LANS runs.
 void SetLansGradUnscale(float factor);
 float GetLansGradUnscale();
+
+// The per-parameter update of the reference's traced SGD optimizer
+// (python/raf/optim/sgd.py:192-200) as a dataflow pattern, with handles on its leaves:
+//     subtract(w, multiply(lr, add(multiply(mu, v), dx | cast(dx_half, "float32"), v, null)), w, null)
+// `op_prefix` is "raf.op." for the pattern registered with the FuseDialect pass and
+// "raf.op.hip." for the body of the fused function.  Inside the function every outside value
+// (constants included) is a parameter of its own, so there the leaves are all wildcards and the
+// `out` arguments are separate leaves.
+struct SgdUpdatePattern {
+  ir::DFPattern root;
+  ir::DFPattern w, w_out, v, v_out, dx, dx_half, lr, mu, null_v, null_w, cast_dtype;
+};
+SgdUpdatePattern MakeSgdUpdatePattern(const std::string& op_prefix, bool inside_function);
+constexpr const char* kSgdUpdatePatternName = "sgd_update";
+constexpr int kSgdUpdatePatternPlevel = 60;  // above every pattern of the reference (8..55)
+
+// The expression the traced optimizer emits for one parameter (w, v float32; dx float32, or a
+// 16-bit float that is cast first); the result is new_w.
+ir::Expr TracedSgdUpdate(const ir::Expr& w, const ir::Expr& dx, const ir::Expr& v,
+                         double learning_rate, double momentum);
 
 }  // namespace hip
 }  // namespace op

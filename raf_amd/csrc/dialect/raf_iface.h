@@ -33,6 +33,10 @@
 
 namespace raf {
 
+namespace ir {
+struct ExprNode;  // raf_ir.h
+}
+
 class Error : public std::runtime_error {
  public:
   explicit Error(const std::string& what) : std::runtime_error(what) {}
@@ -223,6 +227,9 @@ struct DefuseTensorArgs : ArgsBase {  // def_schema.py:836-841
 // ---------------------------------------------------------------------------------- CallValues
 struct CallValuesNode {
   std::string callee;  // operator name, e.g. "raf.op.lans" or "raf.op.hip.lans"
+  // Set instead of `callee` when a fused (primitive) function is called: the reference's
+  // ClosureValue callee (src/impl/op.cc:182-185).  `args` is then a schema::ListArgs.
+  std::shared_ptr<const ir::ExprNode> closure;
   std::shared_ptr<schema::ArgsBase> args;
   value::Value out;
   Device device;
@@ -330,6 +337,9 @@ class OpDialect {
   // Highest-plevel enabled dialect op, skipping `skip_dialects`; "" if none.
   static std::string Dispatch(const std::string& base_op, DevType device_type,
                               const std::vector<std::string>& skip_dialects = {});
+  // The op that `dialect` registered for `base_op`, whatever the device; "" if none
+  // (src/impl/dialect.cc:204-214).
+  static std::string Lower(const std::string& base_op, const std::string& dialect);
   std::string name;
 
  private:

@@ -409,6 +409,14 @@ std::string OpDialect::Dispatch(const std::string& base_op, DevType device_type,
   return "";
 }
 
+std::string OpDialect::Lower(const std::string& base_op, const std::string& dialect) {
+  OpDialect& od = OpDialects().get_or_add(base_op);
+  std::lock_guard<std::mutex> lock(od.mu_);
+  for (const auto& e : od.dialect_ops_)
+    if (e.dialect == dialect) return e.dialect_op;
+  return "";
+}
+
 DialectPreference::DialectPreference(std::vector<std::string> dialects)
     : dialects_(std::move(dialects)), prev_(g_preference) {
   g_preference = &dialects_;

@@ -146,6 +146,64 @@ def sgd(x, dx, v, learning_rate, mu):
     return v1, x1
 
 
+class TracedSgdUpdate:
+    """The per-parameter update of the reference's traced SGD optimizer,
+    ``add(multiply(momentum, v), dx, out=v)`` then ``subtract(w, multiply(learning_rate, new_v),
+    out=w)`` with ``cast(dx, "float32")`` in front for a 16-bit gradient
+    (python/raf/optim/sgd.py:192-200), taken through the dialect fusion pass: the graph is built,
+    the ``hip`` dialect's ``sgd_update`` pattern turns it into one primitive function, and every
+    call of this object runs that function as one kernel launch, in place on ``w`` and ``v``.
+    The tensors are bound once, as a traced model binds its parameters; ``ir_before`` / ``ir_after``
+    hold the text of the graph on either side of the pass."""
+
+    def __init__(self, w, dx, v, learning_rate, momentum):
+        lib = _lib.dialect()
+        self._keep: list = [w, dx, v]
+        self._descs = (_desc(w, self._keep), _desc(dx, self._keep), _desc(v, self._keep))
+        self.w = w
+        key = ("traced_sgd", _sig(w), _sig(dx), _sig(v), float(learning_rate), float(momentum))
+        env = _env_cache.get(key)
+        if env is None:
+            h = c_void_p(None)
+            status = lib.rafhip_raf_traced_sgd_make(*self._descs, float(learning_rate), float(momentum),
+                                                    ctypes.byref(h))
+            made = _Env(h) if h.value else None  # also set when nothing fused: it then holds the graphs
+            check_raf(status)
+            env = _env_cache[key] = made
+        self._env = env
+        self._execute = lib.rafhip_raf_traced_sgd_execute
+
+    def __call__(self):
+        check_raf(self._execute(self._env.handle, *self._descs, _stream(self.w)))
+        return self.w
+
+    def _text(self, fused: int) -> str:
+        buf = ctypes.create_string_buffer(1 << 14)
+        check_raf(_lib.dialect().rafhip_raf_env_ir_text(self._env.handle, fused, buf, len(buf)))
+        return buf.value.decode()
+
+    @property
+    def ir_before(self) -> str:
+        return self._text(0)
+
+    @property
+    def ir_after(self) -> str:
+        return self._text(1)
+
+    @property
+    def op(self) -> str:
+        return self._env.op
+
+
+def traced_sgd_update(w, dx, v, learning_rate, momentum, return_ir=False):
+    """One fused traced update (see ``TracedSgdUpdate``) of ``w`` and ``v`` in place; returns ``w``
+    (the traced ``new_w`` shares its memory), with ``return_ir`` also the graph text before and
+    after the pass."""
+    upd = TracedSgdUpdate(w, dx, v, learning_rate, momentum)
+    upd()
+    return (w, upd.ir_before, upd.ir_after) if return_ir else w
+
+
 def sgd_multi(tensor_list: Sequence[torch.Tensor], learning_rate, mu):
     """Extension op: momentum SGD over a parameter list ``[x..., dx..., v...]`` in place (x and v
     are updated, the list is returned), one launch; per element the four roundings of ``sgd``."""

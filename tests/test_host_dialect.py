@@ -24,6 +24,32 @@ def test_cpp_registry_dispatch_declare(native_libs, tmp_path):
     assert "ALL OK" in r.stdout
 
 
+def test_cpp_ir_patterns_fuse_dialect_pass(native_libs, tmp_path):
+    """Graph IR, dataflow patterns, the fuse-pattern registry, the FuseDialect pass on the traced SGD
+    update and the dispatch of fused functions (tests/cpp/test_fuse_dialect.cc)."""
+    exe = tmp_path / "test_fuse_dialect"
+    d = ROOT / "raf_amd" / "csrc" / "dialect"
+    subprocess.run(["g++", "-O1", "-std=c++17", "-Wall", f"-I{d}", f"-I{ROOT / 'include'}",
+                    str(ROOT / "tests" / "cpp" / "test_fuse_dialect.cc"),
+                    str(d / "registry.cc"), str(d / "raf_ir.cc"), str(d / "hip_fusion.cc"),
+                    str(d / "hip_dialect.cc"), str(d / "device_api.cc"), str(d / "memory_pool.cc"),
+                    f"-L{native_libs.LIB_DIR}", "-lraf_hip_optim", f"-Wl,-rpath,{native_libs.LIB_DIR}",
+                    "-o", str(exe)], check=True)
+    r = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "ALL OK" in r.stdout
+
+
+def test_traced_update_needs_a_rocm_device(native_libs):
+    import torch
+    from raf_amd import op
+    from raf_amd._lib import RafError
+
+    w = torch.zeros(8)
+    with pytest.raises(RafError, match="no fuse pattern matched on device type cpu"):
+        op.traced_sgd_update(w, torch.ones(8), torch.zeros(8), 0.1, 0.9)
+
+
 def test_dispatch_lists_seen_from_python(native_libs):
     from raf_amd import op
 
