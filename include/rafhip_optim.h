@@ -41,7 +41,8 @@ typedef enum rafhip_status {
   RAFHIP_ERR_UNSUPPORTED = 2, /* dtype or size the kernels do not handle                       */
   RAFHIP_ERR_WORKSPACE = 3,   /* workspace missing, too small or misaligned                    */
   RAFHIP_ERR_HIP = 4,         /* a HIP runtime call failed; message carries hipGetErrorString  */
-  RAFHIP_ERR_NO_DEVICE = 5    /* no usable gfx950 device in this process                       */
+  RAFHIP_ERR_NO_DEVICE = 5,   /* no usable gfx950 device in this process                       */
+  RAFHIP_ERR_HOST = 6         /* host side: out of memory or an unexpected C++ exception       */
 } rafhip_status;
 
 typedef enum rafhip_dtype {

@@ -20,6 +20,7 @@ RAFHIP_ERR_UNSUPPORTED = 2
 RAFHIP_ERR_WORKSPACE = 3
 RAFHIP_ERR_HIP = 4
 RAFHIP_ERR_NO_DEVICE = 5
+RAFHIP_ERR_HOST = 6
 
 RAFHIP_F32 = 0
 RAFHIP_F16 = 1

@@ -17,6 +17,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <memory>
 #include <new>
 #include <vector>
 
@@ -142,24 +143,26 @@ int run(rafhip_fuse_plan* plan, const char* what, void* const* parts, void* flat
   if (!plan) return fail(RAFHIP_ERR_INVALID_ARG, "%s: plan is NULL", what);
   if (plan->n_items == 0) return RAFHIP_OK;  // nothing to move
   if (!parts || !flat) return fail(RAFHIP_ERR_INVALID_ARG, "%s: null pointer argument", what);
-  std::vector<Segment> segs((size_t)plan->n);
-  for (int32_t i = 0; i < plan->n; ++i) {
-    if (plan->nbytes[i] > 0 && !parts[i])
-      return fail(RAFHIP_ERR_INVALID_ARG, "%s: tensor %d has a null data pointer", what, i);
-    segs[i] = Segment{static_cast<char*>(parts[i]), plan->offset[i], plan->nbytes[i], 0};
-  }
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  RAFHIP_HIP_TRY(plan->segments.sync(segs, s));
-  const int64_t cap = streaming_grid_cap();
-  const unsigned grid = (unsigned)(plan->n_items < cap ? plan->n_items : cap);
-  if (plan->total_bytes > kStreamFromBytes)
-    hipLaunchKernelGGL(fuse_copy<true>, dim3(grid), dim3(kCopyBlock), 0, s, plan->d_segments,
-                       plan->d_items, plan->n_items, static_cast<char*>(flat), gather ? 1 : 0);
-  else
-    hipLaunchKernelGGL(fuse_copy<false>, dim3(grid), dim3(kCopyBlock), 0, s, plan->d_segments,
-                       plan->d_items, plan->n_items, static_cast<char*>(flat), gather ? 1 : 0);
-  RAFHIP_HIP_TRY(hipGetLastError());
-  return RAFHIP_OK;
+  return guarded(what, [&]() -> int {
+    std::vector<Segment> segs((size_t)plan->n);
+    for (int32_t i = 0; i < plan->n; ++i) {
+      if (plan->nbytes[i] > 0 && !parts[i])
+        return fail(RAFHIP_ERR_INVALID_ARG, "%s: tensor %d has a null data pointer", what, i);
+      segs[i] = Segment{static_cast<char*>(parts[i]), plan->offset[i], plan->nbytes[i], 0};
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    RAFHIP_HIP_TRY(plan->segments.sync(segs, s));
+    const int64_t cap = streaming_grid_cap();
+    const unsigned grid = (unsigned)(plan->n_items < cap ? plan->n_items : cap);
+    if (plan->total_bytes > kStreamFromBytes)
+      hipLaunchKernelGGL(fuse_copy<true>, dim3(grid), dim3(kCopyBlock), 0, s, plan->d_segments,
+                         plan->d_items, plan->n_items, static_cast<char*>(flat), gather ? 1 : 0);
+    else
+      hipLaunchKernelGGL(fuse_copy<false>, dim3(grid), dim3(kCopyBlock), 0, s, plan->d_segments,
+                         plan->d_items, plan->n_items, static_cast<char*>(flat), gather ? 1 : 0);
+    RAFHIP_HIP_TRY(hipGetLastError());
+    return RAFHIP_OK;
+  });
 }
 
 }  // namespace
@@ -172,52 +175,45 @@ int rafhip_fuse_plan_create(int32_t n_tensors, const int64_t* nbytes, rafhip_fus
   *out_plan = nullptr;
   if (n_tensors < 0 || (n_tensors > 0 && !nbytes))
     return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_fuse_plan_create: bad tensor list");
-  rafhip_fuse_plan* p = new (std::nothrow) rafhip_fuse_plan();
-  if (!p) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_fuse_plan_create: out of host memory");
-  p->n = n_tensors;
-  std::vector<CopyItem> items;
-  for (int32_t i = 0; i < n_tensors; ++i) {
-    if (nbytes[i] < 0) {
-      free_plan(p);
-      return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_fuse_plan_create: nbytes[%d] = %lld < 0", i,
-                  (long long)nbytes[i]);
+  return guarded("rafhip_fuse_plan_create", [&]() -> int {
+    std::unique_ptr<rafhip_fuse_plan, void (*)(rafhip_fuse_plan*)> p(new rafhip_fuse_plan(), free_plan);
+    p->n = n_tensors;
+    std::vector<CopyItem> items;
+    for (int32_t i = 0; i < n_tensors; ++i) {
+      if (nbytes[i] < 0)
+        return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_fuse_plan_create: nbytes[%d] = %lld < 0", i,
+                    (long long)nbytes[i]);
+      const int64_t chunks = (nbytes[i] + kCopyChunk - 1) / kCopyChunk;
+      if (chunks > INT32_MAX)
+        return fail(RAFHIP_ERR_UNSUPPORTED, "rafhip_fuse_plan_create: tensor %d is too large", i);
+      p->nbytes.push_back(nbytes[i]);
+      p->offset.push_back(p->total_bytes);
+      p->total_bytes += nbytes[i];
+      for (int64_t c = 0; c < chunks; ++c) items.push_back(CopyItem{i, (int32_t)c});
     }
-    const int64_t chunks = (nbytes[i] + kCopyChunk - 1) / kCopyChunk;
-    if (chunks > INT32_MAX) {
-      free_plan(p);
-      return fail(RAFHIP_ERR_UNSUPPORTED, "rafhip_fuse_plan_create: tensor %d is too large", i);
+    p->n_items = (int64_t)items.size();
+    if (p->n_items == 0) {  // an empty list or only empty tensors: valid, nothing to launch
+      *out_plan = p.release();
+      return RAFHIP_OK;
     }
-    p->nbytes.push_back(nbytes[i]);
-    p->offset.push_back(p->total_bytes);
-    p->total_bytes += nbytes[i];
-    for (int64_t c = 0; c < chunks; ++c) items.push_back(CopyItem{i, (int32_t)c});
-  }
-  p->n_items = (int64_t)items.size();
-  if (p->n_items == 0) {  // an empty list or only empty tensors: valid, nothing to launch
-    *out_plan = p;
+    if (hipGetDevice(&p->device) != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(RAFHIP_ERR_NO_DEVICE, "rafhip_fuse_plan_create: no HIP device available");
+    }
+    const size_t seg_bytes = (sizeof(Segment) * (size_t)n_tensors + 255) / 256 * 256;
+    hipError_t e = hipMalloc(&p->d_tables, seg_bytes + sizeof(CopyItem) * items.size());
+    if (e == hipSuccess) {
+      p->d_segments = static_cast<Segment*>(p->d_tables);
+      p->d_items = reinterpret_cast<CopyItem*>(static_cast<char*>(p->d_tables) + seg_bytes);
+      e = p->segments.init(p->d_segments, (size_t)n_tensors);
+    }
+    if (e == hipSuccess) {
+      e = hipMemcpy(p->d_items, items.data(), sizeof(CopyItem) * items.size(), hipMemcpyHostToDevice);
+    }
+    if (e != hipSuccess) return fail(RAFHIP_ERR_HIP, "rafhip_fuse_plan_create: %s", hipGetErrorString(e));
+    *out_plan = p.release();
     return RAFHIP_OK;
-  }
-  if (hipGetDevice(&p->device) != hipSuccess) {
-    (void)hipGetLastError();
-    free_plan(p);
-    return fail(RAFHIP_ERR_NO_DEVICE, "rafhip_fuse_plan_create: no HIP device available");
-  }
-  const size_t seg_bytes = (sizeof(Segment) * (size_t)n_tensors + 255) / 256 * 256;
-  hipError_t e = hipMalloc(&p->d_tables, seg_bytes + sizeof(CopyItem) * items.size());
-  if (e == hipSuccess) {
-    p->d_segments = static_cast<Segment*>(p->d_tables);
-    p->d_items = reinterpret_cast<CopyItem*>(static_cast<char*>(p->d_tables) + seg_bytes);
-    e = p->segments.init(p->d_segments, (size_t)n_tensors);
-  }
-  if (e == hipSuccess) {
-    e = hipMemcpy(p->d_items, items.data(), sizeof(CopyItem) * items.size(), hipMemcpyHostToDevice);
-  }
-  if (e != hipSuccess) {
-    free_plan(p);
-    return fail(RAFHIP_ERR_HIP, "rafhip_fuse_plan_create: %s", hipGetErrorString(e));
-  }
-  *out_plan = p;
-  return RAFHIP_OK;
+  });
 }
 
 int rafhip_fuse_plan_destroy(rafhip_fuse_plan* plan) {

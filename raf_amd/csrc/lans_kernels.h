@@ -128,8 +128,7 @@ struct TensorStats {  // 64 bytes = 8 words, one per tensor; "not ready" pattern
 struct SyncHeader {
   uint32_t ticket;  // next work item
   uint32_t error;   // 1 if a bounded wait ran out
-  uint32_t spin_limit;  // polls a wait may take before it gives up
-  uint32_t pad;
+  uint32_t pad[2];
 };
 
 struct HParamsPod {

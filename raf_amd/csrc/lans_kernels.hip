@@ -97,12 +97,19 @@ __device__ __forceinline__ uint64_t ld_bits(const double* p) {
 __device__ __forceinline__ void publish(double* p, double v) {
   st_dev(p, v != v ? __builtin_nan("") : v);
 }
-__device__ __forceinline__ double wait_published(const double* word, SyncHeader* sync) {
+// The bound of a wait travels in registers (a kernel argument): a poll loop must not touch the
+// cache line of the ticket, which every workgroup hammers with atomics (reading the bound from
+// there made the whole step 12 % slower).
+struct WaitCtx {
+  uint32_t* error;  // set to 1 when a wait runs out
+  uint32_t limit;   // polls a wait may take
+};
+__device__ __forceinline__ double wait_published(const double* word, const WaitCtx& wc) {
   uint64_t bits = ld_bits(word);
   uint32_t spins = 0;
   while (bits == kNotReady) {
-    if (++spins > sync->spin_limit) {
-      __hip_atomic_store(&sync->error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (++spins > wc.limit) {
+      __hip_atomic_store(wc.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       break;
     }
     __builtin_amdgcn_s_sleep(8);
@@ -115,14 +122,14 @@ __device__ __forceinline__ double wait_published(const double* word, SyncHeader*
 // read again.
 template <int N>
 __device__ __forceinline__ void wait_published_n(const double* const (&words)[N], double (&out)[N],
-                                                 SyncHeader* sync) {
+                                                 const WaitCtx& wc) {
   uint64_t bits[N];
 #pragma unroll
   for (int j = 0; j < N; ++j) bits[j] = ld_bits(words[j]);
 #pragma unroll
   for (int j = 0; j < N; ++j)
     out[j] = bits[j] != kNotReady ? __longlong_as_double((long long)bits[j])
-                                  : wait_published(words[j], sync);
+                                  : wait_published(words[j], wc);
 }
 
 // A tensor's totals from its chunk partials (kPartialSlots doubles per chunk, N of them starting
@@ -132,7 +139,7 @@ __device__ __forceinline__ void wait_published_n(const double* const (&words)[N]
 template <int N, bool kWait>
 __device__ __forceinline__ void tensor_totals(const double* partials, int slot, int64_t n_units,
                                               int chunks_per_unit, double (&tot)[N],
-                                              double (*red)[kLansWaves], SyncHeader* sync) {
+                                              double (*red)[kLansWaves], const WaitCtx& wc) {
 #pragma unroll
   for (int j = 0; j < N; ++j) tot[j] = 0.0;
   for (int64_t i = threadIdx.x; i < n_units; i += kLansBlock) {
@@ -142,7 +149,7 @@ __device__ __forceinline__ void tensor_totals(const double* partials, int slot, 
       double val[N];
 #pragma unroll
       for (int j = 0; j < N; ++j) words[j] = p + j;
-      wait_published_n<N>(words, val, sync);
+      wait_published_n<N>(words, val, wc);
 #pragma unroll
       for (int j = 0; j < N; ++j) tot[j] += val[j];
     } else {
@@ -488,7 +495,6 @@ __device__ __forceinline__ void write_step_scalars(const LansDeviceArgs& a, cons
                                                    int32_t step_host, const HParamsPod& hp) {
   a.sync->ticket = 0u;
   a.sync->error = 0u;
-  a.sync->spin_limit = a.spin_limit;
   const int step = step_dev ? (int)(*step_dev) : step_host;
   float bc1 = 1.0f, bc2 = 1.0f;
   if (hp.bias_correction == 1) {  // double pow, then one rounding to fp32 (lans.cc:103-104)
@@ -564,11 +570,11 @@ __global__ __launch_bounds__(kLansBlock) void lans_finish(LansDeviceArgs a, int 
   const StepScalars k = *a.scalars;
   if (after_b) {
     double tot[3], r0, r1;
-    tensor_totals<3, false>(part, 1, chunks_of(tr), 1, tot, red, nullptr);
+    tensor_totals<3, false>(part, 1, chunks_of(tr), 1, tot, red, WaitCtx{nullptr, 0});
     if (threadIdx.x == 0) stats_after_b(&a.stats[t], tot, k, r0, r1);
   } else {
     double tot[1];
-    tensor_totals<1, false>(part, 0, units_a_of(tr), kChunksPerA, tot, red, nullptr);
+    tensor_totals<1, false>(part, 0, units_a_of(tr), kChunksPerA, tot, red, WaitCtx{nullptr, 0});
     if (threadIdx.x == 0) stats_after_a(&a.stats[t], tot[0], k);
   }
 }
@@ -590,7 +596,7 @@ __global__ __launch_bounds__(kLansBlock) void lans_norm_u(LansDeviceArgs a) {
     if constexpr (kMode == kModeResidentInline) {
       double tot[1];
       tensor_totals<1, false>(a.partials + kPartialSlots * (int64_t)tr.first_chunk, 0, units_a_of(tr),
-                              kChunksPerA, tot, red, nullptr);
+                              kChunksPerA, tot, red, WaitCtx{nullptr, 0});
       if (chunk == 0 && threadIdx.x == 0)  // one workgroup per tensor leaves the statistics
         inv_gdiv = stats_after_a(&a.stats[it.tensor], tot[0], k);
       else
@@ -623,7 +629,7 @@ __global__ __launch_bounds__(kLansBlock) void lans_apply(LansDeviceArgs a) {
     if constexpr (kMode == kModeResidentInline) {
       double tot[3];
       tensor_totals<3, false>(a.partials + kPartialSlots * (int64_t)tr.first_chunk, 1, chunks_of(tr), 1,
-                              tot, red, nullptr);
+                              tot, red, WaitCtx{nullptr, 0});
       p.inv_gdiv = a.stats[it.tensor].inv_grad_div;  // left by pass B
       if (chunk == 0 && threadIdx.x == 0)
         stats_after_b(&a.stats[it.tensor], tot, k, p.rm, p.rg);
@@ -644,6 +650,7 @@ __global__ __launch_bounds__(kLansBlock) void lans_pipelined(LansDeviceArgs a) {
   __shared__ double s_bcast[3];
   __shared__ uint32_t s_ticket;
   const StepScalars k = *a.scalars;
+  const WaitCtx wc{&a.sync->error, a.spin_limit};
 
   // Thread 0 draws tickets two items ahead, so an atomic's round trip is hidden behind a whole
   // item, and every thread reads the NEXT item's descriptor and tensor record while the current
@@ -694,12 +701,12 @@ __global__ __launch_bounds__(kLansBlock) void lans_pipelined(LansDeviceArgs a) {
       if (threadIdx.x == 0) publish(part, s[0]);
     } else if (phase == kPhaseFinishA) {
       double tot[1];
-      tensor_totals<1, true>(tensor_part, 0, units_a_of(tr), kChunksPerA, tot, red, a.sync);
+      tensor_totals<1, true>(tensor_part, 0, units_a_of(tr), kChunksPerA, tot, red, wc);
       if (threadIdx.x == 0) stats_after_a(st, tot[0], k);
     } else if (phase == kPhaseB) {
       double s[3];
       chunk_sums_u<G, kPipelinedPolicy.b_g, kPipelinedPolicy.b_wmv, kPipelinedAhead>(cv, a.unscale, k,
-                      [&] { return wait_published(&st->inv_grad_div, a.sync); }, s);
+                      [&] { return wait_published(&st->inv_grad_div, wc); }, s);
       block_sum<3>(s, red);
       if (threadIdx.x == 0) {
         publish(part + 1, s[0]);
@@ -708,14 +715,14 @@ __global__ __launch_bounds__(kLansBlock) void lans_pipelined(LansDeviceArgs a) {
       }
     } else if (phase == kPhaseFinishB) {
       double tot[3], r0, r1;
-      tensor_totals<3, true>(tensor_part, 1, n_chunks, 1, tot, red, a.sync);
+      tensor_totals<3, true>(tensor_part, 1, n_chunks, 1, tot, red, wc);
       if (threadIdx.x == 0) stats_after_b(st, tot, k, r0, r1);
     } else if (phase == kPhaseC) {
       chunk_apply<G, kPipelinedPolicy.c_g, kPipelinedPolicy.c_wmv, kPipelinedPolicy.c_stores, kPipelinedAhead>(
           cv, a.unscale, a.p_is_bf16 != 0, k, [&] {
         const double* const words[3] = {&st->inv_grad_div, &st->ratio_m, &st->ratio_g};
         double val[3];
-        wait_published_n<3>(words, val, a.sync);
+        wait_published_n<3>(words, val, wc);
         return ApplyParams{val[0], val[1], val[2]};
       });
     } else {

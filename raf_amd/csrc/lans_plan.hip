@@ -9,6 +9,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <limits>
+#include <memory>
 #include <new>
 #include <vector>
 
@@ -238,20 +239,22 @@ int rafhip_lans_pipeline_order(int32_t n_tensors, const int64_t* numel, int64_t 
   clear_error();
   if (int st = validate_list("rafhip_lans_pipeline_order", n_tensors, numel)) return st;
   if (!n_items_out) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_pipeline_order: n_items_out is NULL");
-  const std::vector<WorkItem> items =
-      build_pipeline(n_tensors, numel, group_elements > 0 ? group_elements : kDefaultGroupElems);
-  *n_items_out = (int64_t)items.size();
-  if (triples_out) {
-    if (capacity < (int64_t)items.size())
-      return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_pipeline_order: capacity %lld < %zu items",
-                  (long long)capacity, items.size());
-    for (size_t i = 0; i < items.size(); ++i) {
-      triples_out[3 * i + 0] = (int32_t)(items[i].chunk_phase >> kPhaseShift);
-      triples_out[3 * i + 1] = items[i].tensor;
-      triples_out[3 * i + 2] = (int32_t)(items[i].chunk_phase & kChunkMask);
+  return guarded("rafhip_lans_pipeline_order", [&]() -> int {
+    const std::vector<WorkItem> items =
+        build_pipeline(n_tensors, numel, group_elements > 0 ? group_elements : kDefaultGroupElems);
+    *n_items_out = (int64_t)items.size();
+    if (triples_out) {
+      if (capacity < (int64_t)items.size())
+        return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_pipeline_order: capacity %lld < %zu items",
+                    (long long)capacity, items.size());
+      for (size_t i = 0; i < items.size(); ++i) {
+        triples_out[3 * i + 0] = (int32_t)(items[i].chunk_phase >> kPhaseShift);
+        triples_out[3 * i + 1] = items[i].tensor;
+        triples_out[3 * i + 2] = (int32_t)(items[i].chunk_phase & kChunkMask);
+      }
     }
-  }
-  return RAFHIP_OK;
+    return RAFHIP_OK;
+  });
 }
 
 int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t grad_dtype,
@@ -266,96 +269,92 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
                 "gradients may be fp32, fp16 or bf16)",
                 grad_dtype);
 
-  rafhip_lans_plan* p = new (std::nothrow) rafhip_lans_plan();
-  if (!p) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_plan_create: out of host memory");
-  p->n_tensors = n_tensors;
-  p->grad_dtype = grad_dtype;
-  p->numel.assign(numel, numel + n_tensors);
-  p->first_chunk.resize(n_tensors);
-  int64_t chunks = 0, total = 0, longest = 0;
-  for (int32_t t = 0; t < n_tensors; ++t) {
-    p->first_chunk[t] = (int32_t)chunks;
-    chunks += chunks_of(numel[t]);
-    longest = std::max(longest, chunks_of(numel[t]));
-    total += numel[t];
-  }
-  p->short_tensors_only = longest <= kInlineFinishChunks;
-  p->n_chunks = chunks;
-  p->total_elements = total;
-  p->schedule = schedule_setting(total);
-  p->spin_limit = spin_limit_setting();
-  p->ws = make_layout(n_tensors, chunks);
-
-  if (hipGetDevice(&p->device) != hipSuccess) {
-    (void)hipGetLastError();
-    free_plan(p);
-    return fail(RAFHIP_ERR_NO_DEVICE, "rafhip_lans_plan_create: no HIP device available");
-  }
-  int cus = 0;
-  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, p->device) == hipSuccess &&
-      cus > 0)
-    p->n_cus = cus;
-
-  if (n_tensors > 0) {
-    std::vector<WorkItem> phased((size_t)chunks);
-    size_t k = 0;
-    for (int32_t t = 0; t < n_tensors; ++t)
-      for (int64_t c = 0; c < chunks_of(numel[t]); ++c) phased[k++] = make_item(t, kPhaseA, c);
-    std::vector<WorkItem> phased_a;
-    for (int32_t t = 0; t < n_tensors; ++t)
-      for (int64_t u = 0; u < units_a_of(numel[t]); ++u) phased_a.push_back(make_item(t, kPhaseA, u));
-    p->n_items_a = (int64_t)phased_a.size();
-    const std::vector<WorkItem> pipeline = build_pipeline(n_tensors, numel, group_elems_setting());
-    p->n_pipeline_items = (uint32_t)pipeline.size();
-    // Resident workgroups per CU: never more than fit (every workgroup must be running), and by
-    // default three: a larger window of in-flight items measured slower on MI355X (it crowds the
-    // Infinity Cache).  RAFHIP_LANS_BLOCKS_PER_CU overrides the default downwards or up to the fit.
-    const int fit = pipelined_blocks_per_cu(grad_dtype);
-    int per_cu = fit > 0 ? (fit < 3 ? fit : 3) : 2;
-    if (const char* e = std::getenv("RAFHIP_LANS_BLOCKS_PER_CU")) {
-      const int want = std::atoi(e);
-      if (want > 0) per_cu = (fit > 0 && want > fit) ? fit : want;
+  return guarded("rafhip_lans_plan_create", [&]() -> int {
+    std::unique_ptr<rafhip_lans_plan, void (*)(rafhip_lans_plan*)> p(new rafhip_lans_plan(), free_plan);
+    p->n_tensors = n_tensors;
+    p->grad_dtype = grad_dtype;
+    p->numel.assign(numel, numel + n_tensors);
+    p->first_chunk.resize(n_tensors);
+    int64_t chunks = 0, total = 0, longest = 0;
+    for (int32_t t = 0; t < n_tensors; ++t) {
+      p->first_chunk[t] = (int32_t)chunks;
+      chunks += chunks_of(numel[t]);
+      longest = std::max(longest, chunks_of(numel[t]));
+      total += numel[t];
     }
-    p->pipeline_grid = (unsigned)(p->n_cus * per_cu);
-    if (p->pipeline_grid > p->n_pipeline_items) p->pipeline_grid = p->n_pipeline_items;
+    p->short_tensors_only = longest <= kInlineFinishChunks;
+    p->n_chunks = chunks;
+    p->total_elements = total;
+    p->schedule = schedule_setting(total);
+    p->spin_limit = spin_limit_setting();
+    p->ws = make_layout(n_tensors, chunks);
 
-    const size_t tensors_bytes = (size_t)align_up((int64_t)sizeof(TensorRec) * n_tensors);
-    const size_t phased_bytes = (size_t)align_up((int64_t)sizeof(WorkItem) * (int64_t)phased.size());
-    const size_t pipe_bytes = (size_t)align_up((int64_t)sizeof(WorkItem) * (int64_t)pipeline.size());
-    const size_t a_bytes = (size_t)align_up((int64_t)sizeof(WorkItem) * (int64_t)phased_a.size());
-    hipError_t e =
-        hipMalloc(&p->d_tables, tensors_bytes + phased_bytes + pipe_bytes + a_bytes + kAlign);
-    if (e == hipSuccess)
-      e = p->tensors.init(static_cast<TensorRec*>(p->d_tables), (size_t)n_tensors);
-    if (e != hipSuccess) {
-      free_plan(p);
-      return fail(RAFHIP_ERR_HIP, "rafhip_lans_plan_create: allocation failed: %s",
-                  hipGetErrorString(e));
+    if (hipGetDevice(&p->device) != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(RAFHIP_ERR_NO_DEVICE, "rafhip_lans_plan_create: no HIP device available");
     }
-    char* base = static_cast<char*>(p->d_tables);
-    p->d_tensors = reinterpret_cast<TensorRec*>(base);
-    p->d_items = reinterpret_cast<WorkItem*>(base + tensors_bytes);
-    p->d_pipeline = reinterpret_cast<WorkItem*>(base + tensors_bytes + phased_bytes);
-    p->d_items_a = reinterpret_cast<WorkItem*>(base + tensors_bytes + phased_bytes + pipe_bytes);
-    if (!phased_a.empty())
-      e = hipMemcpy(p->d_items_a, phased_a.data(), sizeof(WorkItem) * phased_a.size(),
-                    hipMemcpyHostToDevice);
-    if (e == hipSuccess && !phased.empty())
-      e = hipMemcpy(p->d_items, phased.data(), sizeof(WorkItem) * phased.size(),
-                    hipMemcpyHostToDevice);
-    if (e == hipSuccess && !pipeline.empty())
-      e = hipMemcpy(p->d_pipeline, pipeline.data(), sizeof(WorkItem) * pipeline.size(),
-                    hipMemcpyHostToDevice);
-    if (e == hipSuccess && std::getenv("RAFHIP_LANS_TRACE") && !pipeline.empty())
-      e = hipMalloc(reinterpret_cast<void**>(&p->d_trace), 32 * pipeline.size());
-    if (e != hipSuccess) {
-      free_plan(p);
-      return fail(RAFHIP_ERR_HIP, "rafhip_lans_plan_create: work list upload failed: %s",
-                  hipGetErrorString(e));
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, p->device) == hipSuccess &&
+        cus > 0)
+      p->n_cus = cus;
+
+    if (n_tensors > 0) {
+      std::vector<WorkItem> phased((size_t)chunks);
+      size_t k = 0;
+      for (int32_t t = 0; t < n_tensors; ++t)
+        for (int64_t c = 0; c < chunks_of(numel[t]); ++c) phased[k++] = make_item(t, kPhaseA, c);
+      std::vector<WorkItem> phased_a;
+      for (int32_t t = 0; t < n_tensors; ++t)
+        for (int64_t u = 0; u < units_a_of(numel[t]); ++u) phased_a.push_back(make_item(t, kPhaseA, u));
+      p->n_items_a = (int64_t)phased_a.size();
+      const std::vector<WorkItem> pipeline = build_pipeline(n_tensors, numel, group_elems_setting());
+      p->n_pipeline_items = (uint32_t)pipeline.size();
+      // Resident workgroups per CU: never more than fit (every workgroup must be running), and by
+      // default three: a larger window of in-flight items measured slower on MI355X (it crowds the
+      // Infinity Cache).  RAFHIP_LANS_BLOCKS_PER_CU overrides the default downwards or up to the fit.
+      const int fit = pipelined_blocks_per_cu(grad_dtype);
+      int per_cu = fit > 0 ? (fit < 3 ? fit : 3) : 2;
+      if (const char* e = std::getenv("RAFHIP_LANS_BLOCKS_PER_CU")) {
+        const int want = std::atoi(e);
+        if (want > 0) per_cu = (fit > 0 && want > fit) ? fit : want;
+      }
+      p->pipeline_grid = (unsigned)(p->n_cus * per_cu);
+      if (p->pipeline_grid > p->n_pipeline_items) p->pipeline_grid = p->n_pipeline_items;
+
+      const size_t tensors_bytes = (size_t)align_up((int64_t)sizeof(TensorRec) * n_tensors);
+      const size_t phased_bytes = (size_t)align_up((int64_t)sizeof(WorkItem) * (int64_t)phased.size());
+      const size_t pipe_bytes = (size_t)align_up((int64_t)sizeof(WorkItem) * (int64_t)pipeline.size());
+      const size_t a_bytes = (size_t)align_up((int64_t)sizeof(WorkItem) * (int64_t)phased_a.size());
+      hipError_t e =
+          hipMalloc(&p->d_tables, tensors_bytes + phased_bytes + pipe_bytes + a_bytes + kAlign);
+      if (e == hipSuccess)
+        e = p->tensors.init(static_cast<TensorRec*>(p->d_tables), (size_t)n_tensors);
+      if (e != hipSuccess)
+        return fail(RAFHIP_ERR_HIP, "rafhip_lans_plan_create: allocation failed: %s",
+                    hipGetErrorString(e));
+      char* base = static_cast<char*>(p->d_tables);
+      p->d_tensors = reinterpret_cast<TensorRec*>(base);
+      p->d_items = reinterpret_cast<WorkItem*>(base + tensors_bytes);
+      p->d_pipeline = reinterpret_cast<WorkItem*>(base + tensors_bytes + phased_bytes);
+      p->d_items_a = reinterpret_cast<WorkItem*>(base + tensors_bytes + phased_bytes + pipe_bytes);
+      if (!phased_a.empty())
+        e = hipMemcpy(p->d_items_a, phased_a.data(), sizeof(WorkItem) * phased_a.size(),
+                      hipMemcpyHostToDevice);
+      if (e == hipSuccess && !phased.empty())
+        e = hipMemcpy(p->d_items, phased.data(), sizeof(WorkItem) * phased.size(),
+                      hipMemcpyHostToDevice);
+      if (e == hipSuccess && !pipeline.empty())
+        e = hipMemcpy(p->d_pipeline, pipeline.data(), sizeof(WorkItem) * pipeline.size(),
+                      hipMemcpyHostToDevice);
+      if (e == hipSuccess && std::getenv("RAFHIP_LANS_TRACE") && !pipeline.empty())
+        e = hipMalloc(reinterpret_cast<void**>(&p->d_trace), 32 * pipeline.size());
+      if (e != hipSuccess)
+        return fail(RAFHIP_ERR_HIP, "rafhip_lans_plan_create: work list upload failed: %s",
+                    hipGetErrorString(e));
     }
-  }
-  *out_plan = p;
-  return RAFHIP_OK;
+    *out_plan = p.release();
+    return RAFHIP_OK;
+  });
 }
 
 int rafhip_lans_plan_destroy(rafhip_lans_plan* plan) {
@@ -414,92 +413,94 @@ int rafhip_lans_step_mixed(rafhip_lans_plan* plan, const void* const* g, float* 
   if (n == 0 || plan->n_chunks == 0) return RAFHIP_OK;  // nothing to update
   if (!g || !w || !m || !v)
     return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_step: null pointer list");
-  if (!workspace || workspace_bytes < plan->ws.total)
-    return fail(RAFHIP_ERR_WORKSPACE, "rafhip_lans_step: workspace %p of %lld bytes, need %lld",
-                workspace, (long long)workspace_bytes, (long long)plan->ws.total);
-  if (!aligned_to(workspace, kAlign))
-    return fail(RAFHIP_ERR_WORKSPACE, "rafhip_lans_step: workspace %p is not 256-byte aligned",
-                workspace);
+  return guarded("rafhip_lans_step", [&]() -> int {
+    if (!workspace || workspace_bytes < plan->ws.total)
+      return fail(RAFHIP_ERR_WORKSPACE, "rafhip_lans_step: workspace %p of %lld bytes, need %lld",
+                  workspace, (long long)workspace_bytes, (long long)plan->ws.total);
+    if (!aligned_to(workspace, kAlign))
+      return fail(RAFHIP_ERR_WORKSPACE, "rafhip_lans_step: workspace %p is not 256-byte aligned",
+                  workspace);
 
-  // Build this call's tensor table; 4-byte (fp16 g: 2-byte) alignment is the hard requirement,
-  // 16-byte alignment of all four selects the vector path.
-  const uintptr_t g_elem = plan->grad_dtype == RAFHIP_F32 ? 4 : 2;
-  const uintptr_t g_vec = 16;  // pass A reads the gradient with 16-byte lane accesses
-  std::vector<TensorRec> recs((size_t)n);
-  for (int32_t t = 0; t < n; ++t) {
-    TensorRec& r = recs[t];
-    r.g = g[t];
-    r.w = w[t];
-    r.m = m[t];
-    r.v = v[t];
-    r.p = p ? p[t] : nullptr;
-    r.numel = plan->numel[t];
-    r.first_chunk = plan->first_chunk[t];
-    r.vec_ok = 0;
-    r.chunk_shift = chunk_shift_for(r.numel);
-    r.reserved = 0;
-    if (r.numel == 0) continue;
-    if (!r.g || !r.w || !r.m || !r.v)
-      return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_step: tensor %d has a null data pointer", t);
-    if (!aligned_to(r.g, g_elem) || !aligned_to(r.w, 4) || !aligned_to(r.m, 4) ||
-        !aligned_to(r.v, 4) || !aligned_to(r.p, 2))
-      return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_step: tensor %d is not element-aligned", t);
-    r.vec_ok = aligned_to(r.g, g_vec) && aligned_to(r.w, 16) && aligned_to(r.m, 16) &&
-               aligned_to(r.v, 16) && aligned_to(r.p, 8);
-  }
+    // Build this call's tensor table; 4-byte (fp16 g: 2-byte) alignment is the hard requirement,
+    // 16-byte alignment of all four selects the vector path.
+    const uintptr_t g_elem = plan->grad_dtype == RAFHIP_F32 ? 4 : 2;
+    const uintptr_t g_vec = 16;  // pass A reads the gradient with 16-byte lane accesses
+    std::vector<TensorRec> recs((size_t)n);
+    for (int32_t t = 0; t < n; ++t) {
+      TensorRec& r = recs[t];
+      r.g = g[t];
+      r.w = w[t];
+      r.m = m[t];
+      r.v = v[t];
+      r.p = p ? p[t] : nullptr;
+      r.numel = plan->numel[t];
+      r.first_chunk = plan->first_chunk[t];
+      r.vec_ok = 0;
+      r.chunk_shift = chunk_shift_for(r.numel);
+      r.reserved = 0;
+      if (r.numel == 0) continue;
+      if (!r.g || !r.w || !r.m || !r.v)
+        return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_step: tensor %d has a null data pointer", t);
+      if (!aligned_to(r.g, g_elem) || !aligned_to(r.w, 4) || !aligned_to(r.m, 4) ||
+          !aligned_to(r.v, 4) || !aligned_to(r.p, 2))
+        return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_step: tensor %d is not element-aligned", t);
+      r.vec_ok = aligned_to(r.g, g_vec) && aligned_to(r.w, 16) && aligned_to(r.m, 16) &&
+                 aligned_to(r.v, 16) && aligned_to(r.p, 8);
+    }
 
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  RAFHIP_HIP_TRY(plan->tensors.sync(recs, s));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    RAFHIP_HIP_TRY(plan->tensors.sync(recs, s));
 
-  char* ws = static_cast<char*>(workspace);
-  LansDeviceArgs a;
-  a.tensors = plan->d_tensors;
-  a.n_tensors = n;
-  a.items = plan->d_items;
-  a.n_chunks = plan->n_chunks;
-  a.items_a = plan->d_items_a;
-  a.n_items_a = plan->n_items_a;
-  a.n_items = plan->n_pipeline_items;
-  a.pipeline_items = plan->d_pipeline;
-  a.unscale = hp->grad_unscale;
-  a.spin_limit = plan->spin_limit;
-  a.p_is_bf16 = p_dtype == RAFHIP_BF16 ? 1 : 0;
-  a.scalars = reinterpret_cast<StepScalars*>(ws + plan->ws.scalars_off);
-  a.stats = reinterpret_cast<TensorStats*>(ws + plan->ws.stats_off);
-  a.partials = reinterpret_cast<double*>(ws + plan->ws.partials_off);
-  a.sync = reinterpret_cast<SyncHeader*>(ws + plan->ws.sync_off);
-  a.trace = plan->d_trace;
+    char* ws = static_cast<char*>(workspace);
+    LansDeviceArgs a;
+    a.tensors = plan->d_tensors;
+    a.n_tensors = n;
+    a.items = plan->d_items;
+    a.n_chunks = plan->n_chunks;
+    a.items_a = plan->d_items_a;
+    a.n_items_a = plan->n_items_a;
+    a.n_items = plan->n_pipeline_items;
+    a.pipeline_items = plan->d_pipeline;
+    a.unscale = hp->grad_unscale;
+    a.spin_limit = plan->spin_limit;
+    a.p_is_bf16 = p_dtype == RAFHIP_BF16 ? 1 : 0;
+    a.scalars = reinterpret_cast<StepScalars*>(ws + plan->ws.scalars_off);
+    a.stats = reinterpret_cast<TensorStats*>(ws + plan->ws.stats_off);
+    a.partials = reinterpret_cast<double*>(ws + plan->ws.partials_off);
+    a.sync = reinterpret_cast<SyncHeader*>(ws + plan->ws.sync_off);
+    a.trace = plan->d_trace;
 
-  HParamsPod pod;
-  pod.learning_rate = hp->learning_rate;
-  pod.beta1 = hp->beta1;
-  pod.beta2 = hp->beta2;
-  pod.eps = hp->eps;
-  pod.weight_decay = hp->weight_decay;
-  pod.bias_correction = hp->bias_correction;
-  pod.grad_averaging = hp->grad_averaging;
-  pod.mode = hp->mode;
-  pod.normalize_grad = hp->normalize_grad ? 1 : 0;
+    HParamsPod pod;
+    pod.learning_rate = hp->learning_rate;
+    pod.beta1 = hp->beta1;
+    pod.beta2 = hp->beta2;
+    pod.eps = hp->eps;
+    pod.weight_decay = hp->weight_decay;
+    pod.bias_correction = hp->bias_correction;
+    pod.grad_averaging = hp->grad_averaging;
+    pod.mode = hp->mode;
+    pod.normalize_grad = hp->normalize_grad ? 1 : 0;
 
-  hipEvent_t* marks = nullptr;
-  if (!plan->timing.empty())
-    marks = plan->timing[plan->steps_done % (int64_t)plan->timing.size()].data();
+    hipEvent_t* marks = nullptr;
+    if (!plan->timing.empty())
+      marks = plan->timing[plan->steps_done % (int64_t)plan->timing.size()].data();
 
-  if (plan->schedule == RAFHIP_LANS_PIPELINED) {
-    if (marks) RAFHIP_HIP_TRY(hipEventRecord(marks[0], s));
-    launch_prepare(s, a, step_dev, step_host, pod);
-    if (marks) RAFHIP_HIP_TRY(hipEventRecord(marks[1], s));
-    launch_pipelined(plan->grad_dtype, plan->pipeline_grid, s, a);
-    if (marks)
-      for (int i = 2; i < 6; ++i) RAFHIP_HIP_TRY(hipEventRecord(marks[i], s));
-  } else {
-    const int64_t bytes_per_elt = plan->grad_dtype == RAFHIP_F32 ? 16 : 14;
-    launch_phased(plan->grad_dtype, plan->total_elements * bytes_per_elt > kResidentBytes,
-                  plan->short_tensors_only, s, a, step_dev, step_host, pod, marks);
-  }
-  RAFHIP_HIP_TRY(hipGetLastError());
-  plan->steps_done++;
-  return RAFHIP_OK;
+    if (plan->schedule == RAFHIP_LANS_PIPELINED) {
+      if (marks) RAFHIP_HIP_TRY(hipEventRecord(marks[0], s));
+      launch_prepare(s, a, step_dev, step_host, pod);
+      if (marks) RAFHIP_HIP_TRY(hipEventRecord(marks[1], s));
+      launch_pipelined(plan->grad_dtype, plan->pipeline_grid, s, a);
+      if (marks)
+        for (int i = 2; i < 6; ++i) RAFHIP_HIP_TRY(hipEventRecord(marks[i], s));
+    } else {
+      const int64_t bytes_per_elt = plan->grad_dtype == RAFHIP_F32 ? 16 : 14;
+      launch_phased(plan->grad_dtype, plan->total_elements * bytes_per_elt > kResidentBytes,
+                    plan->short_tensors_only, s, a, step_dev, step_host, pod, marks);
+    }
+    RAFHIP_HIP_TRY(hipGetLastError());
+    plan->steps_done++;
+    return RAFHIP_OK;
+  });
 }
 
 int rafhip_lans_read_norms(const rafhip_lans_plan* plan, const void* workspace, double* host_out,
@@ -509,29 +510,31 @@ int rafhip_lans_read_norms(const rafhip_lans_plan* plan, const void* workspace, 
     return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_read_norms: null argument");
   const int32_t n = plan->n_tensors;
   if (n == 0) return RAFHIP_OK;
-  std::vector<TensorStats> st((size_t)n);
-  SyncHeader sync{};
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  const char* ws = static_cast<const char*>(workspace);
-  RAFHIP_HIP_TRY(hipMemcpyAsync(st.data(), ws + plan->ws.stats_off, sizeof(TensorStats) * (size_t)n,
-                                hipMemcpyDeviceToHost, s));
-  RAFHIP_HIP_TRY(hipMemcpyAsync(&sync, ws + plan->ws.sync_off, sizeof(sync), hipMemcpyDeviceToHost, s));
-  RAFHIP_HIP_TRY(hipStreamSynchronize(s));
-  for (int32_t t = 0; t < n; ++t) {
-    if (plan->numel[t] == 0) {  // no chunks, nothing was computed: an empty tensor has zero norms
-      for (int q = 0; q < 4; ++q) host_out[4 * t + q] = 0.0;
-      continue;
+  return guarded("rafhip_lans_read_norms", [&]() -> int {
+    std::vector<TensorStats> st((size_t)n);
+    SyncHeader sync{};
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const char* ws = static_cast<const char*>(workspace);
+    RAFHIP_HIP_TRY(hipMemcpyAsync(st.data(), ws + plan->ws.stats_off, sizeof(TensorStats) * (size_t)n,
+                                  hipMemcpyDeviceToHost, s));
+    RAFHIP_HIP_TRY(hipMemcpyAsync(&sync, ws + plan->ws.sync_off, sizeof(sync), hipMemcpyDeviceToHost, s));
+    RAFHIP_HIP_TRY(hipStreamSynchronize(s));
+    for (int32_t t = 0; t < n; ++t) {
+      if (plan->numel[t] == 0) {  // no chunks, nothing was computed: an empty tensor has zero norms
+        for (int q = 0; q < 4; ++q) host_out[4 * t + q] = 0.0;
+        continue;
+      }
+      host_out[4 * t + 0] = st[t].grad_norm;
+      host_out[4 * t + 1] = st[t].param_norm;
+      host_out[4 * t + 2] = st[t].um_norm;
+      host_out[4 * t + 3] = st[t].ug_norm;
     }
-    host_out[4 * t + 0] = st[t].grad_norm;
-    host_out[4 * t + 1] = st[t].param_norm;
-    host_out[4 * t + 2] = st[t].um_norm;
-    host_out[4 * t + 3] = st[t].ug_norm;
-  }
-  if (plan->n_chunks > 0 && sync.error != 0)
-    return fail(RAFHIP_ERR_HIP,
-                "rafhip_lans_read_norms: the last pipelined step ran out of a bounded wait; its "
-                "results are invalid");
-  return RAFHIP_OK;
+    if (plan->n_chunks > 0 && sync.error != 0)
+      return fail(RAFHIP_ERR_HIP,
+                  "rafhip_lans_read_norms: the last pipelined step ran out of a bounded wait; its "
+                  "results are invalid");
+    return RAFHIP_OK;
+  });
 }
 
 int rafhip_lans_debug_trace(rafhip_lans_plan* plan, uint64_t* words_out, int64_t capacity_items,
@@ -553,20 +556,22 @@ int rafhip_lans_timing_enable(rafhip_lans_plan* plan, int32_t slots) {
   if (!plan) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_timing_enable: plan is NULL");
   if (slots < 0 || slots > 4096)
     return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_timing_enable: slots = %d", slots);
-  destroy_timing(plan);
-  plan->steps_done = 0;
-  plan->timing.resize((size_t)slots);
-  for (auto& slot : plan->timing) slot.fill(nullptr);
-  for (auto& slot : plan->timing)
-    for (auto& e : slot) {
-      hipError_t err = hipEventCreate(&e);
-      if (err != hipSuccess) {
-        destroy_timing(plan);
-        return fail(RAFHIP_ERR_HIP, "rafhip_lans_timing_enable: hipEventCreate: %s",
-                    hipGetErrorString(err));
+  return guarded("rafhip_lans_timing_enable", [&]() -> int {
+    destroy_timing(plan);
+    plan->steps_done = 0;
+    plan->timing.resize((size_t)slots);
+    for (auto& slot : plan->timing) slot.fill(nullptr);
+    for (auto& slot : plan->timing)
+      for (auto& e : slot) {
+        hipError_t err = hipEventCreate(&e);
+        if (err != hipSuccess) {
+          destroy_timing(plan);
+          return fail(RAFHIP_ERR_HIP, "rafhip_lans_timing_enable: hipEventCreate: %s",
+                      hipGetErrorString(err));
+        }
       }
-    }
-  return RAFHIP_OK;
+    return RAFHIP_OK;
+  });
 }
 
 int rafhip_lans_timing_read(rafhip_lans_plan* plan, int32_t slot, float* ms_out5) {

@@ -20,6 +20,7 @@
 // (python/raf/optim/sgd.py:187-215) -- and for the one-op-call-per-parameter loop of its imperative
 // optimizer (sgd.py:51-58).
 #include <cstdint>
+#include <memory>
 #include <new>
 #include <vector>
 
@@ -264,52 +265,45 @@ extern "C" int rafhip_sgd_plan_create(int32_t n_tensors, const int64_t* numel, i
   if (grad_dtype != RAFHIP_F32 && grad_dtype != RAFHIP_F16 && grad_dtype != RAFHIP_BF16)
     return fail(RAFHIP_ERR_UNSUPPORTED,
                 "rafhip_sgd_plan_create: gradient dtype %d (fp32, fp16 or bf16)", grad_dtype);
-  rafhip_sgd_plan* p = new (std::nothrow) rafhip_sgd_plan();
-  if (!p) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_sgd_plan_create: out of host memory");
-  p->n = n_tensors;
-  p->grad_dtype = grad_dtype;
-  std::vector<SgdItem> items;
-  for (int32_t t = 0; t < n_tensors; ++t) {
-    if (numel[t] < 0) {
-      free_sgd_plan(p);
-      return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_sgd_plan_create: numel[%d] = %lld < 0", t,
-                  (long long)numel[t]);
+  return guarded("rafhip_sgd_plan_create", [&]() -> int {
+    std::unique_ptr<rafhip_sgd_plan, void (*)(rafhip_sgd_plan*)> p(new rafhip_sgd_plan(), free_sgd_plan);
+    p->n = n_tensors;
+    p->grad_dtype = grad_dtype;
+    std::vector<SgdItem> items;
+    for (int32_t t = 0; t < n_tensors; ++t) {
+      if (numel[t] < 0)
+        return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_sgd_plan_create: numel[%d] = %lld < 0", t,
+                    (long long)numel[t]);
+      const int64_t chunks = (numel[t] + kSgdChunk - 1) / kSgdChunk;
+      if (chunks > INT32_MAX)
+        return fail(RAFHIP_ERR_UNSUPPORTED, "rafhip_sgd_plan_create: tensor %d is too large", t);
+      p->numel.push_back(numel[t]);
+      p->total_elements += numel[t];
+      for (int64_t c = 0; c < chunks; ++c) items.push_back(SgdItem{t, (int32_t)c});
     }
-    const int64_t chunks = (numel[t] + kSgdChunk - 1) / kSgdChunk;
-    if (chunks > INT32_MAX) {
-      free_sgd_plan(p);
-      return fail(RAFHIP_ERR_UNSUPPORTED, "rafhip_sgd_plan_create: tensor %d is too large", t);
+    p->n_items = (int64_t)items.size();
+    if (p->n_items == 0) {  // nothing to update: valid, nothing to launch
+      *out_plan = p.release();
+      return RAFHIP_OK;
     }
-    p->numel.push_back(numel[t]);
-    p->total_elements += numel[t];
-    for (int64_t c = 0; c < chunks; ++c) items.push_back(SgdItem{t, (int32_t)c});
-  }
-  p->n_items = (int64_t)items.size();
-  if (p->n_items == 0) {  // nothing to update: valid, nothing to launch
-    *out_plan = p;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(RAFHIP_ERR_NO_DEVICE, "rafhip_sgd_plan_create: no HIP device available");
+    }
+    const size_t rec_bytes = (sizeof(SgdRec) * (size_t)n_tensors + 255) / 256 * 256;
+    hipError_t e = hipMalloc(&p->d_tables, rec_bytes + sizeof(SgdItem) * items.size());
+    if (e == hipSuccess) {
+      p->d_recs = static_cast<SgdRec*>(p->d_tables);
+      p->d_items = reinterpret_cast<SgdItem*>(static_cast<char*>(p->d_tables) + rec_bytes);
+      e = p->recs.init(p->d_recs, (size_t)n_tensors);
+    }
+    if (e == hipSuccess)
+      e = hipMemcpy(p->d_items, items.data(), sizeof(SgdItem) * items.size(), hipMemcpyHostToDevice);
+    if (e != hipSuccess) return fail(RAFHIP_ERR_HIP, "rafhip_sgd_plan_create: %s", hipGetErrorString(e));
+    *out_plan = p.release();
     return RAFHIP_OK;
-  }
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) {
-    (void)hipGetLastError();
-    free_sgd_plan(p);
-    return fail(RAFHIP_ERR_NO_DEVICE, "rafhip_sgd_plan_create: no HIP device available");
-  }
-  const size_t rec_bytes = (sizeof(SgdRec) * (size_t)n_tensors + 255) / 256 * 256;
-  hipError_t e = hipMalloc(&p->d_tables, rec_bytes + sizeof(SgdItem) * items.size());
-  if (e == hipSuccess) {
-    p->d_recs = static_cast<SgdRec*>(p->d_tables);
-    p->d_items = reinterpret_cast<SgdItem*>(static_cast<char*>(p->d_tables) + rec_bytes);
-    e = p->recs.init(p->d_recs, (size_t)n_tensors);
-  }
-  if (e == hipSuccess)
-    e = hipMemcpy(p->d_items, items.data(), sizeof(SgdItem) * items.size(), hipMemcpyHostToDevice);
-  if (e != hipSuccess) {
-    free_sgd_plan(p);
-    return fail(RAFHIP_ERR_HIP, "rafhip_sgd_plan_create: %s", hipGetErrorString(e));
-  }
-  *out_plan = p;
-  return RAFHIP_OK;
+  });
 }
 
 extern "C" int rafhip_sgd_plan_destroy(rafhip_sgd_plan* plan) {
@@ -329,34 +323,36 @@ extern "C" int rafhip_sgd_multi_step(rafhip_sgd_plan* plan, float* const* x, con
                 "rafhip_sgd_multi_step: weight-copy dtype %d (binary16 or bfloat16)", p_dtype);
   if (plan->n_items == 0) return RAFHIP_OK;
   if (!x || !dx || !v) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_sgd_multi_step: null pointer list");
-  const uintptr_t g_elem = plan->grad_dtype == RAFHIP_F32 ? 4 : 2;
-  std::vector<SgdRec> recs((size_t)plan->n);
-  for (int32_t t = 0; t < plan->n; ++t) {
-    SgdRec& r = recs[t];
-    r = SgdRec{x[t], dx[t], v[t], p ? p[t] : nullptr, plan->numel[t], 0, 0};
-    if (r.numel == 0) continue;
-    if (!r.x || !r.dx || !r.v)
-      return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_sgd_multi_step: tensor %d has a null data pointer", t);
-    if (!aligned_to(r.x, 4) || !aligned_to(r.v, 4) || !aligned_to(r.dx, g_elem) || !aligned_to(r.p, 2))
-      return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_sgd_multi_step: tensor %d is not element-aligned", t);
-    r.vec_ok = aligned_to(r.x, 16) && aligned_to(r.v, 16) && aligned_to(r.dx, 4 * g_elem) &&
-               aligned_to(r.p, 8);
-  }
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  RAFHIP_HIP_TRY(plan->recs.sync(recs, s));
-  // One rounding double -> fp32, as for the single-tensor op.
-  const float lr32 = static_cast<float>(learning_rate);
-  const float mu32 = static_cast<float>(mu);
-  const int64_t cap = streaming_grid_cap();
-  const unsigned grid = (unsigned)(plan->n_items < cap ? plan->n_items : cap);
-  const bool nt = plan->total_elements * (int64_t)(8 + g_elem) > kSgdStreamFromBytes;
-  const int bf = p_dtype == RAFHIP_BF16 ? 1 : 0;
-  if (plan->grad_dtype == RAFHIP_F16)
-    launch_sgd_multi<_Float16>(nt, grid, s, plan->d_recs, plan->d_items, plan->n_items, lr32, mu32, bf);
-  else if (plan->grad_dtype == RAFHIP_BF16)
-    launch_sgd_multi<Bf16>(nt, grid, s, plan->d_recs, plan->d_items, plan->n_items, lr32, mu32, bf);
-  else
-    launch_sgd_multi<float>(nt, grid, s, plan->d_recs, plan->d_items, plan->n_items, lr32, mu32, bf);
-  RAFHIP_HIP_TRY(hipGetLastError());
-  return RAFHIP_OK;
+  return guarded("rafhip_sgd_multi_step", [&]() -> int {
+    const uintptr_t g_elem = plan->grad_dtype == RAFHIP_F32 ? 4 : 2;
+    std::vector<SgdRec> recs((size_t)plan->n);
+    for (int32_t t = 0; t < plan->n; ++t) {
+      SgdRec& r = recs[t];
+      r = SgdRec{x[t], dx[t], v[t], p ? p[t] : nullptr, plan->numel[t], 0, 0};
+      if (r.numel == 0) continue;
+      if (!r.x || !r.dx || !r.v)
+        return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_sgd_multi_step: tensor %d has a null data pointer", t);
+      if (!aligned_to(r.x, 4) || !aligned_to(r.v, 4) || !aligned_to(r.dx, g_elem) || !aligned_to(r.p, 2))
+        return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_sgd_multi_step: tensor %d is not element-aligned", t);
+      r.vec_ok = aligned_to(r.x, 16) && aligned_to(r.v, 16) && aligned_to(r.dx, 4 * g_elem) &&
+                 aligned_to(r.p, 8);
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    RAFHIP_HIP_TRY(plan->recs.sync(recs, s));
+    // One rounding double -> fp32, as for the single-tensor op.
+    const float lr32 = static_cast<float>(learning_rate);
+    const float mu32 = static_cast<float>(mu);
+    const int64_t cap = streaming_grid_cap();
+    const unsigned grid = (unsigned)(plan->n_items < cap ? plan->n_items : cap);
+    const bool nt = plan->total_elements * (int64_t)(8 + g_elem) > kSgdStreamFromBytes;
+    const int bf = p_dtype == RAFHIP_BF16 ? 1 : 0;
+    if (plan->grad_dtype == RAFHIP_F16)
+      launch_sgd_multi<_Float16>(nt, grid, s, plan->d_recs, plan->d_items, plan->n_items, lr32, mu32, bf);
+    else if (plan->grad_dtype == RAFHIP_BF16)
+      launch_sgd_multi<Bf16>(nt, grid, s, plan->d_recs, plan->d_items, plan->n_items, lr32, mu32, bf);
+    else
+      launch_sgd_multi<float>(nt, grid, s, plan->d_recs, plan->d_items, plan->n_items, lr32, mu32, bf);
+    RAFHIP_HIP_TRY(hipGetLastError());
+    return RAFHIP_OK;
+  });
 }

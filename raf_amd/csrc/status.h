@@ -4,6 +4,8 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <exception>
+#include <new>
 
 #include "rafhip_optim.h"
 
@@ -12,6 +14,21 @@ namespace rafhip {
 // Stores a printf-style message for rafhip_last_error() and returns `code`.
 int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 void clear_error();
+
+// No C++ exception may cross the C boundary: entry points that allocate host memory (work lists,
+// tables) run their body through this and report a failure as RAFHIP_ERR_HOST instead.
+template <typename F>
+int guarded(const char* who, F&& body) noexcept {
+  try {
+    return body();
+  } catch (const std::bad_alloc&) {
+    return fail(RAFHIP_ERR_HOST, "%s: out of host memory", who);
+  } catch (const std::exception& e) {
+    return fail(RAFHIP_ERR_HOST, "%s: %s", who, e.what());
+  } catch (...) {
+    return fail(RAFHIP_ERR_HOST, "%s: unknown C++ exception", who);
+  }
+}
 
 }  // namespace rafhip
 

@@ -43,6 +43,14 @@ def test_dialect_header_symbols_all_exported_and_bound(native_libs):
     assert sorted(native_libs.DIALECT_SYMBOLS) == names
 
 
+def test_status_and_dtype_codes_match_the_header(native_libs):
+    text = (ROOT / "include" / "rafhip_optim.h").read_text()
+    codes = dict(re.findall(r"\b(RAFHIP_(?:OK|ERR_[A-Z_]+|F16|F32|F64|BF16))\s*=\s*(\d+)", text))
+    assert len([k for k in codes if k.startswith("RAFHIP_ERR_")]) == 6
+    for name, value in codes.items():
+        assert getattr(native_libs, name) == int(value), name
+
+
 def test_abi_version_and_struct_layout(native_libs):
     lib = native_libs.optim()
     assert lib.rafhip_abi_version() == 1
