@@ -43,7 +43,7 @@ SGD_BYTES_PER_ELT = 20  # read x, dx, v; write v1, x1
 # runs scaled by a plain 1 GiB copy (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); figures and commands are in
 # profiles/.  Workloads not listed were not measured (null).
 MEASURED_TRAFFIC = {
-    ("lans_bert_large_fp16grad", "lans_pipelined"): 14_089_400_000,
+    ("lans_bert_large_fp16grad", "lans_pipelined"): 14_088_700_000,
     ("lans_bert_large_fp16grad", "lans_apply"): 8_716_600_000,
     ("sgd_4m_fp32", "sgd_vec4_kernel"): 83_925_600,
     ("lans_bert_large_mixed_fp16", "lans_pipelined"): 14_759_300_000,
