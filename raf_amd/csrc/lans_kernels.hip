@@ -296,18 +296,23 @@ __device__ __forceinline__ void load_batch(Batch<G>& b, const ChunkView& cv, int
 // Walks the 4-element groups of a chunk trip by trip and hands each loaded trip to `body`.  With
 // kAhead the loads of trip i+1 are issued before trip i is evaluated: one more trip of registers
 // (32 VGPRs), which the persistent kernel has to spare at three workgroups per CU.
-template <typename G, bool kGradNT, bool kNT, bool kAhead, typename Body>
-__device__ __forceinline__ void for_each_trip(const ChunkView& cv, int n4, Body&& body) {
+// `pre` runs once before the first trip is evaluated -- with kAhead after that trip's loads have
+// been issued, so that whatever it waits for (the tensor's statistics, read past the L2 in the
+// pipelined schedule) is in flight together with the data instead of ahead of it.
+template <typename G, bool kGradNT, bool kNT, bool kAhead, typename Pre, typename Body>
+__device__ __forceinline__ void for_each_trip(const ChunkView& cv, int n4, Pre&& pre, Body&& body) {
   constexpr int kStride = kLansBlock * kUnroll;
   if constexpr (kAhead) {
     Batch<G> nxt;
     load_batch<G, kGradNT, kNT>(nxt, cv, (int)threadIdx.x, n4);
+    pre();
     for (int i0 = threadIdx.x; i0 < n4; i0 += kStride) {
       const Batch<G> cur = nxt;
       load_batch<G, kGradNT, kNT>(nxt, cv, i0 + kStride, n4);  // guarded per lane by i < n4
       body(cur, i0);
     }
   } else {
+    pre();
     for (int i0 = threadIdx.x; i0 < n4; i0 += kStride) {
       Batch<G> cur;
       load_batch<G, kGradNT, kNT>(cur, cv, i0, n4);
@@ -328,8 +333,9 @@ __device__ __forceinline__ void chunk_sums_u(const ChunkView& cv, float unscale,
   double am = 0.0, au = 0.0, aw = 0.0;
   if (cv.vec_ok) {
     const int n4 = cv.len >> 2;
-    const double inv_gdiv = get_inv_gdiv();
-    for_each_trip<G, kGradNT, kNT, kAhead>(cv, n4, [&](const Batch<G>& cur, int i0) {
+    double inv_gdiv = 1.0;
+    for_each_trip<G, kGradNT, kNT, kAhead>(cv, n4, [&] { inv_gdiv = get_inv_gdiv(); },
+                                           [&](const Batch<G>& cur, int i0) {
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
         if (i0 + u * kLansBlock < n4) {
@@ -397,8 +403,9 @@ __device__ __forceinline__ void chunk_apply(const ChunkView& cv, float unscale, 
                                             const StepScalars& k, GetParams&& get_params) {
   if (cv.vec_ok) {
     const int n4 = cv.len >> 2;
-    const ApplyParams p = get_params();
-    for_each_trip<G, kGradNT, kNT, kAhead>(cv, n4, [&](const Batch<G>& cur, int i0) {
+    ApplyParams p{1.0, 0.0, 0.0};
+    for_each_trip<G, kGradNT, kNT, kAhead>(cv, n4, [&] { p = get_params(); },
+                                           [&](const Batch<G>& cur, int i0) {
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
         const int i = i0 + u * kLansBlock;
