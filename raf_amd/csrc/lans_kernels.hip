@@ -321,6 +321,27 @@ __device__ __forceinline__ void for_each_trip(const ChunkView& cv, int n4, Pre&&
   }
 }
 
+// One trip's contribution to a lane's sums of u_m^2, u_g^2 and w^2 (pass B).
+template <typename G>
+__device__ __forceinline__ void sums_of_trip(const Batch<G>& cur, int i0, int n4, float unscale,
+                                             double inv_gdiv, const StepScalars& k, double& am,
+                                             double& au, double& aw) {
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    if (i0 + u * kLansBlock < n4) {
+      const f32x4 g = GradIO<G>::widen4(cur.g[u], unscale);
+      const Directions d0 = lans_directions(g.x, cur.w[u].x, cur.m[u].x, cur.v[u].x, inv_gdiv, k);
+      const Directions d1 = lans_directions(g.y, cur.w[u].y, cur.m[u].y, cur.v[u].y, inv_gdiv, k);
+      const Directions d2 = lans_directions(g.z, cur.w[u].z, cur.m[u].z, cur.v[u].z, inv_gdiv, k);
+      const Directions d3 = lans_directions(g.w, cur.w[u].w, cur.m[u].w, cur.v[u].w, inv_gdiv, k);
+      am += (d0.um * d0.um + d1.um * d1.um) + (d2.um * d2.um + d3.um * d3.um);
+      au += (d0.ug * d0.ug + d1.ug * d1.ug) + (d2.ug * d2.ug + d3.ug * d3.ug);
+      aw += ((double)cur.w[u].x * (double)cur.w[u].x + (double)cur.w[u].y * (double)cur.w[u].y) +
+            ((double)cur.w[u].z * (double)cur.w[u].z + (double)cur.w[u].w * (double)cur.w[u].w);
+    }
+  }
+}
+
 // ------------------------------------------------------------------ pass B on one chunk
 // Per-thread contributions to sum u_m^2, sum u_g^2 and sum w^2.  `get_inv_gdiv` supplies the
 // tensor's gradient divisor (the pipelined schedule may have to wait for it).
@@ -336,20 +357,7 @@ __device__ __forceinline__ void chunk_sums_u(const ChunkView& cv, float unscale,
     double inv_gdiv = 1.0;
     for_each_trip<G, kGradNT, kNT, kAhead>(cv, n4, [&] { inv_gdiv = get_inv_gdiv(); },
                                            [&](const Batch<G>& cur, int i0) {
-#pragma unroll
-      for (int u = 0; u < kUnroll; ++u) {
-        if (i0 + u * kLansBlock < n4) {
-          const f32x4 g = GradIO<G>::widen4(cur.g[u], unscale);
-          const Directions d0 = lans_directions(g.x, cur.w[u].x, cur.m[u].x, cur.v[u].x, inv_gdiv, k);
-          const Directions d1 = lans_directions(g.y, cur.w[u].y, cur.m[u].y, cur.v[u].y, inv_gdiv, k);
-          const Directions d2 = lans_directions(g.z, cur.w[u].z, cur.m[u].z, cur.v[u].z, inv_gdiv, k);
-          const Directions d3 = lans_directions(g.w, cur.w[u].w, cur.m[u].w, cur.v[u].w, inv_gdiv, k);
-          am += (d0.um * d0.um + d1.um * d1.um) + (d2.um * d2.um + d3.um * d3.um);
-          au += (d0.ug * d0.ug + d1.ug * d1.ug) + (d2.ug * d2.ug + d3.ug * d3.ug);
-          aw += ((double)cur.w[u].x * (double)cur.w[u].x + (double)cur.w[u].y * (double)cur.w[u].y) +
-                ((double)cur.w[u].z * (double)cur.w[u].z + (double)cur.w[u].w * (double)cur.w[u].w);
-        }
-      }
+      sums_of_trip<G>(cur, i0, n4, unscale, inv_gdiv, k, am, au, aw);
     });
     const int tail = (n4 << 2) + threadIdx.x;
     if (tail < cv.len) {
@@ -397,6 +405,32 @@ __device__ __forceinline__ Applied apply_one(double g, double w, double m, doubl
   return o;
 }
 
+// One trip of pass C for a lane: the new w, m, v (and the optional 16-bit weight copy) of its
+// kUnroll groups of four elements.
+template <typename G, bool kStoreNT>
+__device__ __forceinline__ void apply_trip(const Batch<G>& cur, int i0, int n4, const ChunkView& cv,
+                                           float unscale, bool p_is_bf16, const ApplyParams& p,
+                                           const StepScalars& k) {
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    const int i = i0 + u * kLansBlock;
+    if (i < n4) {
+      const f32x4 g = GradIO<G>::widen4(cur.g[u], unscale);
+      const Applied a0 = apply_one(g.x, cur.w[u].x, cur.m[u].x, cur.v[u].x, p, k);
+      const Applied a1 = apply_one(g.y, cur.w[u].y, cur.m[u].y, cur.v[u].y, p, k);
+      const Applied a2 = apply_one(g.z, cur.w[u].z, cur.m[u].z, cur.v[u].z, p, k);
+      const Applied a3 = apply_one(g.w, cur.w[u].w, cur.m[u].w, cur.v[u].w, p, k);
+      stg<kStoreNT>((g_float4*)cv.w + i, f32x4{a0.w, a1.w, a2.w, a3.w});
+      stg<kStoreNT>((g_float4*)cv.m + i, f32x4{a0.m, a1.m, a2.m, a3.m});
+      stg<kStoreNT>((g_float4*)cv.v + i, f32x4{a0.v, a1.v, a2.v, a3.v});
+      if (cv.p)  // uniform over the workgroup
+        stg<kStoreNT>((g_u16x4*)cv.p + i,
+                      u16x4{narrow16(a0.w, p_is_bf16), narrow16(a1.w, p_is_bf16),
+                            narrow16(a2.w, p_is_bf16), narrow16(a3.w, p_is_bf16)});
+    }
+  }
+}
+
 // `get_params` supplies the tensor's divisor and trust ratios.
 template <typename G, bool kGradNT, bool kNT, bool kStoreNT, bool kAhead = false, typename GetParams>
 __device__ __forceinline__ void chunk_apply(const ChunkView& cv, float unscale, bool p_is_bf16,
@@ -406,24 +440,7 @@ __device__ __forceinline__ void chunk_apply(const ChunkView& cv, float unscale, 
     ApplyParams p{1.0, 0.0, 0.0};
     for_each_trip<G, kGradNT, kNT, kAhead>(cv, n4, [&] { p = get_params(); },
                                            [&](const Batch<G>& cur, int i0) {
-#pragma unroll
-      for (int u = 0; u < kUnroll; ++u) {
-        const int i = i0 + u * kLansBlock;
-        if (i < n4) {
-          const f32x4 g = GradIO<G>::widen4(cur.g[u], unscale);
-          const Applied a0 = apply_one(g.x, cur.w[u].x, cur.m[u].x, cur.v[u].x, p, k);
-          const Applied a1 = apply_one(g.y, cur.w[u].y, cur.m[u].y, cur.v[u].y, p, k);
-          const Applied a2 = apply_one(g.z, cur.w[u].z, cur.m[u].z, cur.v[u].z, p, k);
-          const Applied a3 = apply_one(g.w, cur.w[u].w, cur.m[u].w, cur.v[u].w, p, k);
-          stg<kStoreNT>((g_float4*)cv.w + i, f32x4{a0.w, a1.w, a2.w, a3.w});
-          stg<kStoreNT>((g_float4*)cv.m + i, f32x4{a0.m, a1.m, a2.m, a3.m});
-          stg<kStoreNT>((g_float4*)cv.v + i, f32x4{a0.v, a1.v, a2.v, a3.v});
-          if (cv.p)  // uniform over the workgroup
-            stg<kStoreNT>((g_u16x4*)cv.p + i,
-                          u16x4{narrow16(a0.w, p_is_bf16), narrow16(a1.w, p_is_bf16),
-                                narrow16(a2.w, p_is_bf16), narrow16(a3.w, p_is_bf16)});
-        }
-      }
+      apply_trip<G, kStoreNT>(cur, i0, n4, cv, unscale, p_is_bf16, p, k);
     });
     const int tail = (n4 << 2) + threadIdx.x;
     if (tail < cv.len) {
