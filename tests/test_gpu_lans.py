@@ -296,6 +296,48 @@ def test_pipelined_schedule_is_bitwise_equal_to_phased(native_libs, monkeypatch,
         _assert_norms(results["pipelined"][1], on)
 
 
+def test_random_lists_groupings_and_slicings_agree_bitwise(native_libs, monkeypatch):
+    """Whatever the list looks like and however the pipelined work list is cut (cache-group size,
+    slices per round, resident workgroups), the result is the phased schedule's, bit for bit, and no
+    bounded wait runs out."""
+    from raf_amd import kernels
+
+    rng = np.random.default_rng(9)
+    hp = LansHParams()
+    for case in range(24):
+        n = int(rng.integers(1, 40))
+        kinds = rng.integers(0, 4, n)
+        sizes = [int(x) for x in np.where(kinds == 0, rng.integers(0, 64, n),          # tiny, some empty
+                                 np.where(kinds == 1, rng.integers(1000, 9000, n),      # around one chunk
+                                 np.where(kinds == 2, rng.integers(20_000, 200_000, n),  # a few chunks
+                                          rng.integers(500_000, 1_500_000, n))))]       # large-chunk tensors
+        g, w, m, v = lans_inputs(sizes, cfg=200 + case, g16=bool(case % 2))
+        hp_case = LansHParams(grad_unscale=(1 / 1024 if case % 2 else 1.0), mode=int(case % 3 == 0))
+        outs = []
+        for schedule in ("phased", "pipelined"):
+            if schedule == "pipelined":
+                monkeypatch.setenv("RAFHIP_LANS_GROUP_ELEMS", str(int(rng.choice([1, 50_000, 400_000, 3_000_000]))))
+                monkeypatch.setenv("RAFHIP_LANS_ROUND_SLICES", str(int(rng.choice([1, 2, 8, 64, 4096]))))
+                monkeypatch.setenv("RAFHIP_LANS_BLOCKS_PER_CU", str(int(rng.choice([1, 2, 3]))))
+            tg, tw, tm, tv = _to_dev(g), _to_dev(w), _to_dev(m), _to_dev(v)
+            plan = kernels.LansPlan(sizes, tg[0].dtype, DEV)
+            plan.set_schedule(schedule)
+            for step in (1, 2):
+                plan.step(tg, tw, tm, tv, step, _khp(hp_case))
+            torch.cuda.synchronize()
+            norms = plan.read_norms()  # raises if a wait ran out
+            outs.append(([t.cpu().numpy() for t in tw + tm + tv], norms))
+            plan.close()
+        for a, b in zip(outs[0][0], outs[1][0]):
+            assert np.array_equal(a, b), (case, sizes)
+        assert np.array_equal(outs[0][1], outs[1][1]), (case, sizes)
+        if case < 6:  # and both are the oracle's
+            ow, om, ov = w, m, v
+            for step in (1, 2):
+                ow, om, ov, on = lans_f64.lans_step(g, ow, om, ov, step, hp_case)
+            _assert_close(outs[1][0], ow + om + ov, TOL_1, f"case {case}")
+
+
 # ------------------------------------------------------------------ graph capture
 @pytest.mark.parametrize("schedule", ["phased", "pipelined"])
 def test_step_can_be_captured_in_a_hip_graph(native_libs, schedule):
