@@ -177,6 +177,12 @@ int rafhip_raf_traced_sgd_execute(rafhip_raf_env* env, const rafhip_tensor_desc*
                                   void* stream);
 int rafhip_raf_env_ir_text(const rafhip_raf_env* env, int32_t fused, char* buf, int32_t buflen);
 
+/* hip-dialect extension for learning-rate schedules: moves the learning rate of an OpEnv made by
+ * the sgd, sgd_multi, lans or lans_mixed makers, so that a new value every step does not mean a
+ * new OpEnv (in the reference the learning rate is a schema constant and part of the OpEnv cache
+ * key, src/impl/vm/vm.cc:1012-1015).  Fails for any other OpEnv. */
+int rafhip_raf_env_set_learning_rate(rafhip_raf_env* env, double learning_rate);
+
 /* Total bytes of the OpEnv's workspace requests (each rounded up to 256). */
 int64_t rafhip_raf_env_workspace_bytes(const rafhip_raf_env* env);
 /* OpEnv::name() and the dialect op the dispatcher picked; pointers stay valid until destroy. */

@@ -172,6 +172,7 @@ DIALECT_SYMBOLS = {
                                            c_double, c_double, POINTER(c_void_p)]),
     "rafhip_raf_traced_sgd_execute": (c_int, [c_void_p] + [POINTER(TensorDesc)] * 3 + [c_void_p]),
     "rafhip_raf_env_ir_text": (c_int, [c_void_p, c_int32, c_char_p, c_int32]),
+    "rafhip_raf_env_set_learning_rate": (c_int, [c_void_p, c_double]),
     "rafhip_raf_env_name": (c_char_p, [c_void_p]),
     "rafhip_raf_env_op": (c_char_p, [c_void_p]),
     "rafhip_raf_env_destroy": (c_int, [c_void_p]),

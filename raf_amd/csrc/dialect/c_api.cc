@@ -600,6 +600,16 @@ int rafhip_raf_env_ir_text(const rafhip_raf_env* env, int32_t fused, char* buf, 
   });
 }
 
+int rafhip_raf_env_set_learning_rate(rafhip_raf_env* env, double learning_rate) {
+  return Guard([&] {
+    if (!env) throw Error("rafhip_raf_env_set_learning_rate: env is NULL");
+    if (!env->env) return;  // declared as a no-op: nothing to tell
+    auto* target = dynamic_cast<hip::HasLearningRate*>(env->env.get());
+    if (!target) throw Error("rafhip_raf_env_set_learning_rate: " + env->name + " has no learning rate");
+    target->SetLearningRate(learning_rate);
+  });
+}
+
 const char* rafhip_raf_env_name(const rafhip_raf_env* env) { return env ? env->name.c_str() : ""; }
 const char* rafhip_raf_env_op(const rafhip_raf_env* env) { return env ? env->op.c_str() : ""; }
 

@@ -53,7 +53,7 @@ void SetLansGradUnscale(float factor) { g_lans_grad_unscale = factor; }
 float GetLansGradUnscale() { return g_lans_grad_unscale; }
 
 // ----------------------------------------------------------------------------------------- SGD
-class SgdHipEnv : public OpEnv {
+class SgdHipEnv : public OpEnv, public HasLearningRate {
  public:
   explicit SgdHipEnv(const CallValues& cv) {
     const auto* args = cv->args_as<schema::SgdArgs>();
@@ -101,6 +101,9 @@ class SgdHipEnv : public OpEnv {
     if (st != RAFHIP_OK) throw Error(KernelError("rafhip_sgd_f32", st));
   }
 
+  void SetLearningRate(double learning_rate) override { learning_rate_ = learning_rate; }
+  double GetLearningRate() const override { return learning_rate_; }
+
   static OpEnv* make(const CallValues& cv) { return new SgdHipEnv(cv); }
 
  private:
@@ -113,7 +116,7 @@ class SgdHipEnv : public OpEnv {
 // Extension ops raf.op.sgd_multi / raf.op.sgd_multi_mixed: what the reference's traced optimizer
 // emits per parameter as cast, multiply, add(out=), multiply, subtract(out=), cast, add(out=)
 // (python/raf/optim/sgd.py:187-215), as one in-place launch over the whole list.
-class SgdMultiHipEnv : public OpEnv {
+class SgdMultiHipEnv : public OpEnv, public HasLearningRate {
  public:
   SgdMultiHipEnv(const CallValues& cv, bool mixed)
       : blocks_(mixed ? 4 : 3),
@@ -196,6 +199,9 @@ class SgdMultiHipEnv : public OpEnv {
     if (st != RAFHIP_OK) throw Error(KernelError("rafhip_sgd_multi_step", st));
   }
 
+  void SetLearningRate(double learning_rate) override { learning_rate_ = learning_rate; }
+  double GetLearningRate() const override { return learning_rate_; }
+
   static OpEnv* make(const CallValues& cv) { return new SgdMultiHipEnv(cv, false); }
   static OpEnv* make_mixed(const CallValues& cv) { return new SgdMultiHipEnv(cv, true); }
 
@@ -216,7 +222,7 @@ class SgdMultiHipEnv : public OpEnv {
 // new weights narrowed to 16 bits -- what the reference's traced optimizer does with a cast and a
 // copy after the op, python/raf/optim/lans.py:289-291, :303-305).  Half gradients are accepted by
 // both and widened in the kernel, replacing the group_cast in front of the op (lans.py:261-265).
-class LansHipEnv : public OpEnv {
+class LansHipEnv : public OpEnv, public HasLearningRate {
  public:
   LansHipEnv(const CallValues& cv, bool mixed)
       : blocks_(mixed ? 5 : 4),
@@ -331,6 +337,9 @@ class LansHipEnv : public OpEnv {
                                     workspace_bytes_, stream);
     if (st != RAFHIP_OK) throw Error(KernelError("rafhip_lans_step_mixed", st));
   }
+
+  void SetLearningRate(double learning_rate) override { hp_.learning_rate = (float)learning_rate; }
+  double GetLearningRate() const override { return hp_.learning_rate; }
 
   static OpEnv* make(const CallValues& cv) { return new LansHipEnv(cv, false); }
   static OpEnv* make_mixed(const CallValues& cv) { return new LansHipEnv(cv, true); }

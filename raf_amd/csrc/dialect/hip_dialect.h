@@ -15,6 +15,18 @@ namespace hip {
 void SetLansGradUnscale(float factor);
 float GetLansGradUnscale();
 
+// A learning-rate schedule changes one hyper-parameter every step.  The reference's schemas carry
+// the learning rate as a constant, so there every new value means a new OpEnv (the VM's cache key
+// holds the constants, src/impl/vm/vm.cc:1012-1015).  The hip OpEnvs of the optimizer ops
+// implement this interface instead: the executor that owns the OpEnv may move its learning rate
+// between two Execute calls and keep the OpEnv, its plan and its device tables.
+class HasLearningRate {
+ public:
+  virtual ~HasLearningRate() = default;
+  virtual void SetLearningRate(double learning_rate) = 0;
+  virtual double GetLearningRate() const = 0;
+};
+
 // The per-parameter update of the reference's traced SGD optimizer
 // (python/raf/optim/sgd.py:192-200) as a dataflow pattern, with handles on its leaves:
 //     subtract(w, multiply(lr, add(multiply(mu, v), dx | cast(dx_half, "float32"), v, null)), w, null)

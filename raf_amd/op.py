@@ -11,6 +11,7 @@ standing in for RAF's memory pool) and the current stream, nothing else.
 """
 from __future__ import annotations
 
+import collections
 import ctypes
 import weakref
 from ctypes import c_int64, c_void_p
@@ -61,6 +62,14 @@ class _Env:
         self.op = lib.rafhip_raf_env_op(handle).decode()
         self.workspace_bytes = lib.rafhip_raf_env_workspace_bytes(handle)
         self.workspaces = {}  # stream handle -> runtime.Memory
+        self.learning_rate = None  # what the OpEnv was made with or last told, if it has one
+
+    def set_learning_rate(self, learning_rate: float) -> None:
+        """A learning-rate schedule keeps its OpEnv: the hip optimizer OpEnvs take a new value between
+        two executions (a hip-dialect extension; the reference would build a new OpEnv)."""
+        if learning_rate != self.learning_rate:
+            check_raf(_lib.dialect().rafhip_raf_env_set_learning_rate(self.handle, learning_rate))
+            self.learning_rate = learning_rate
 
     def __del__(self):
         try:
@@ -83,7 +92,28 @@ def _workspace(env: "_Env", like: torch.Tensor, stream) -> runtime.Memory:
     return ws
 
 
-_env_cache: Dict[Tuple, _Env] = {}
+class _EnvCache(collections.OrderedDict):
+    """OpEnvs by call signature, the least recently used dropped beyond `capacity`: every OpEnv owns
+    device tables, pinned staging memory and a workspace per stream, and hyper-parameters other than
+    the learning rate are part of the signature, so an unbounded table would grow with every new
+    value a training script tries."""
+
+    capacity = 64
+
+    def get(self, key, default=None):
+        env = super().get(key, default)
+        if env is not default:
+            self.move_to_end(key)
+        return env
+
+    def __setitem__(self, key, env):
+        super().__setitem__(key, env)
+        self.move_to_end(key)
+        while len(self) > self.capacity:
+            self.popitem(last=False)
+
+
+_env_cache = _EnvCache()
 
 
 def clear_op_env_cache() -> None:
@@ -132,13 +162,15 @@ def sgd(x, dx, v, learning_rate, mu):
     lib = _lib.dialect()
     keep: list = []
     dx_, ddx, dv = _desc(x, keep), _desc(dx, keep), _desc(v, keep)
-    key = ("sgd", _sig(x), _sig(dx), _sig(v), float(learning_rate), float(mu))
+    key = ("sgd", _sig(x), _sig(dx), _sig(v), float(mu))
     env = _env_cache.get(key)
     if env is None:
         h = c_void_p(None)
         check_raf(lib.rafhip_raf_sgd_make(dx_, ddx, dv, float(learning_rate), float(mu),
                                           ctypes.byref(h)))
         env = _env_cache[key] = _Env(h)
+        env.learning_rate = float(learning_rate)
+    env.set_learning_rate(float(learning_rate))
     v1 = torch.empty_like(dx)  # the executor's AllocOutputBuffer (interpreter.cc:397-426)
     x1 = torch.empty_like(dx)
     check_raf(lib.rafhip_raf_sgd_execute(env.handle, dx_, ddx, dv, _desc(v1, keep), _desc(x1, keep),
@@ -223,13 +255,16 @@ def _sgd_multi(mixed, tensor_list, learning_rate, mu):
     n = len(tensor_list)
     m = _marshal_list(tensor_list)
     descs = m.descs
-    key = ("sgd_multi", mixed, m.sig, float(learning_rate), float(mu))
+    key = ("sgd_multi", mixed, m.sig, float(mu))
     env = _env_cache.get(key)
     if env is None:
         h = c_void_p(None)
         check_raf(lib.rafhip_raf_sgd_multi_make(int(mixed), n, descs, float(learning_rate), float(mu),
                                                 ctypes.byref(h)))
         env = _env_cache[key] = _Env(h)
+        env.learning_rate = float(learning_rate)
+    if n:
+        env.set_learning_rate(float(learning_rate))
     check_raf(lib.rafhip_raf_sgd_multi_execute(env.handle, n, descs, _stream(tensor_list[0]) if n else None))
     return tensor_list
 
@@ -265,13 +300,16 @@ def _lans(op_name, tensor_list, step, learning_rate, beta1, beta2, eps, bias_cor
     dstep = _desc(step, keep)
     hp = (float(learning_rate), float(beta1), float(beta2), float(eps), int(bias_correction),
           float(weight_decay), int(grad_averaging), int(mode), int(bool(normalize_grad)))
-    key = (op_name, m.sig, _sig(step), hp, get_lans_grad_unscale())
+    key = (op_name, m.sig, _sig(step), hp[1:], get_lans_grad_unscale())  # all but the learning rate
     env = _env_cache.get(key)
     if env is None:
         h = c_void_p(None)
         make = lib.rafhip_raf_lans_make if op_name == "lans" else lib.rafhip_raf_lans_mixed_make
         check_raf(make(n4, descs, dstep, *hp, ctypes.byref(h)))
         env = _env_cache[key] = _Env(h)
+        env.learning_rate = hp[0]
+    if n4:
+        env.set_learning_rate(hp[0])
     stream = _stream(tensor_list[0]) if n4 else None
     ws = _workspace(env, tensor_list[0], stream) if env.workspace_bytes > 0 else None
     check_raf(lib.rafhip_raf_lans_execute(env.handle, n4, descs, dstep, ws.data if ws else None,
