@@ -145,7 +145,7 @@ int32_t rafhip_lans_pass_a_unit_elements(int64_t numel);
  *   PIPELINED  set-up + ONE persistent launch whose work list interleaves the three passes of
  *              neighbouring cache-sized tensor groups, so that a group's second and third reads
  *              come from the 256 MB Infinity Cache instead of HBM.
- * A plan picks PIPELINED for lists of 128 Mi elements or more and PHASED below (short lists are
+ * A plan picks PIPELINED for lists of 64 Mi elements or more and PHASED below (short lists are
  * launch- and latency-bound); RAFHIP_LANS_SCHEDULE=phased|pipelined overrides that per process and
  * rafhip_lans_plan_set_schedule per plan.
  */

@@ -240,12 +240,12 @@ def test_workspace_and_argument_errors(native_libs):
 
 # ------------------------------------------------------------------ the two schedules
 def test_default_schedule_follows_list_length(native_libs, monkeypatch):
-    """Lists of 128 Mi elements or more run pipelined, shorter ones phased; the environment variable
+    """Lists of 64 Mi elements or more run pipelined, shorter ones phased; the environment variable
     and the per-plan setter override that."""
     from raf_amd import kernels
 
     monkeypatch.delenv("RAFHIP_LANS_SCHEDULE", raising=False)
-    for sizes, want in (([1000, 5], "phased"), ([(1 << 27) - 1], "phased"), ([1 << 26, 1 << 26], "pipelined")):
+    for sizes, want in (([1000, 5], "phased"), ([(1 << 26) - 1], "phased"), ([1 << 25, 1 << 25], "pipelined")):
         plan = kernels.LansPlan(sizes, torch.float32, DEV)
         assert plan.schedule == want, sizes
         plan.set_schedule("pipelined" if want == "phased" else "phased")
