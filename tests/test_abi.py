@@ -43,6 +43,14 @@ def test_dialect_header_symbols_all_exported_and_bound(native_libs):
     assert sorted(native_libs.DIALECT_SYMBOLS) == names
 
 
+def test_built_libraries_are_not_older_than_their_sources(native_libs):
+    """GPU runs load the in-tree libraries as they are: a source edited after the last build would be
+    tested and measured in its old form."""
+    from raf_amd import build
+
+    assert build.stale() == []
+
+
 def test_status_and_dtype_codes_match_the_header(native_libs):
     text = (ROOT / "include" / "rafhip_optim.h").read_text()
     codes = dict(re.findall(r"\b(RAFHIP_(?:OK|ERR_[A-Z_]+|F16|F32|F64|BF16))\s*=\s*(\d+)", text))
