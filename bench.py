@@ -175,22 +175,44 @@ def bench_lans(name, wl, args):
     plan.bind(g, w, m, v, hp, p=p16)
     step_t = torch.full((), float(wl["step0"]), dtype=torch.float32, device=dev)
 
-    for _ in range(args.warmup):
+    def one_step():
         plan.step_bound(step_t)
-        step_t.add_(1.0)
+        step_t.add_(1.0)  # the step counter lives on the device, as in the reference's traced optimizer
+
+    for _ in range(args.warmup):
+        one_step()
+    graph = None
+    if args.hip_graph:
+        # The launches of one step (and the counter's increment) recorded once and replayed: what a
+        # training loop captured in a HIP graph pays per step.  Per-kernel events stay outside.
+        args.no_kernel_events = True
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            one_step()
+        for _ in range(3):
+            graph.replay()
     if not args.no_kernel_events:
         plan.timing_enable(args.steps)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        plan.step_bound(step_t)
-        step_t.add_(1.0)  # the step counter lives on the device, as in the reference's traced optimizer
+        if graph is not None:
+            graph.replay()
+        else:
+            one_step()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
 
     a, b, c = lans_bytes_per_elt(2 if g16 else 4)
     ka, kb, kc = lans_kernel_bytes_per_elt(2 if g16 else 4)
+    # phased: five launches, or three when the list fits the cache and no tensor has more than 32 chunks
+    # (every workgroup then adds its tensor's few partial sums itself)
+    lib = _libs()
+    short = all(-(-n // lib.rafhip_lans_chunk_elements(n)) <= 32 for n in sizes if n)
+    cached = total * (14 if g16 else 16) <= (192 << 20)
+    launches = 2 if schedule == "pipelined" else (3 if short and cached else 5)
     if copy16:  # the third pass also writes the 2-byte copy of the new weight
         c, kc = c + 2, kc + 2
     bytes_step = total * (a + b + c)
@@ -209,7 +231,7 @@ def bench_lans(name, wl, args):
                    "bytes_per_element": a + b + c, "bytes_per_step": bytes_step,
                    "kernel_bytes_per_element": ka + kb + kc,
                    "pct_of_hbm_peak": round(100 * bytes_step / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
-                   "schedule": schedule, "launches_per_step": 5 if schedule == "phased" else 2},
+                   "schedule": schedule, "launches_per_step": launches, "hip_graph": bool(args.hip_graph)},
     }
     if not args.no_kernel_events:
         ts = np.array([plan.timing_read(i) for i in range(args.steps)], dtype=np.float64)
@@ -498,6 +520,8 @@ def main():
                     help="LANS launch schedule (bit-identical results); auto = the library's choice")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline leg")
     ap.add_argument("--no-kernel-events", action="store_true", help="do not record per-kernel HIP events")
+    ap.add_argument("--hip-graph", action="store_true",
+                    help="LANS workloads: capture one step in a HIP graph and time its replays")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this path is built and measured on ONE GPU (no collectives, no sharding); "
