@@ -38,6 +38,8 @@ class RecordUploader {
   }
 
   void release() {
+    // An upload that is still reading the staging buffer must finish before the buffer goes away.
+    if (staging_free_ && sent_once_) (void)hipEventSynchronize(staging_free_);
     if (staging_free_) (void)hipEventDestroy(staging_free_);
     if (staging_) (void)hipHostFree(staging_);
     staging_free_ = nullptr;
