@@ -106,3 +106,30 @@ def test_2d_shape_and_shape_mismatch(native_libs):
         kernels.sgd_f32(torch.zeros(4, device=DEV), torch.zeros(5, device=DEV), torch.zeros(4, device=DEV), .1, .9)
     with pytest.raises(TypeError):
         kernels.sgd_f32(*(torch.zeros(4, device=DEV, dtype=torch.float16),) * 3, .1, .9)
+
+
+@pytest.mark.parametrize("shape", [[4, 4]])
+@pytest.mark.parametrize("seed", range(6))
+def test_reference_style_closed_form(native_libs, shape, seed):
+    """The reference's own operator test (tests/python/op/tvm/test_tvm_loss.py:158-176), through the
+    operator front end: standard-normal inputs, a standard-normal momentum (negative ones included),
+    learning rate 0.01, checked as there against the float64 closed form at 1e-4 -- and, beyond the
+    reference, bit for bit against the fp32 oracle."""
+    from raf_amd import op
+
+    rng = np.random.default_rng(seed)
+    x0 = rng.standard_normal(shape).astype("float32")
+    dx = rng.standard_normal(shape).astype("float32")
+    v0 = rng.standard_normal(shape).astype("float32")
+    mu = float(rng.standard_normal(1)[0])
+    learning_rate = 0.01
+    n_v1 = mu * v0 + dx
+    n_x1 = x0 - learning_rate * n_v1
+    m_v1, m_x1 = op.sgd(torch.from_numpy(x0).to(DEV), torch.from_numpy(dx).to(DEV),
+                        torch.from_numpy(v0).to(DEV), learning_rate, mu)
+    np.testing.assert_allclose(m_v1.cpu().numpy(), n_v1, 1e-4, 1e-4)
+    np.testing.assert_allclose(m_x1.cpu().numpy(), n_x1, 1e-4, 1e-4)
+    ov, ox = sgd_f32.sgd_step(x0, dx, v0, learning_rate, mu)
+    assert m_v1.shape == tuple(shape) and m_x1.shape == tuple(shape)
+    _bits_equal(m_v1.reshape(-1), ov.reshape(-1))
+    _bits_equal(m_x1.reshape(-1), ox.reshape(-1))
