@@ -352,9 +352,24 @@ bool IsPrimitive(const FunctionNode* f) {
   return it != f->attrs.end() && it->second != "0";
 }
 
+// Every kCall node of a pattern.
+void CollectCallPatternNodes(const DFPattern& p, std::set<const DFPatternNode*>* seen,
+                             std::vector<const DFPatternNode*>* calls) {
+  if (!p || !seen->insert(p.get()).second) return;
+  if (p->kind == DFPatternNode::kCall) calls->push_back(p.get());
+  CollectCallPatternNodes(p->op, seen, calls);
+  for (const auto& a : p->args) CollectCallPatternNodes(a, seen, calls);
+  CollectCallPatternNodes(p->left, seen, calls);
+  CollectCallPatternNodes(p->right, seen, calls);
+  CollectCallPatternNodes(p->inner, seen, calls);
+}
+
 class Rewriter {
  public:
-  Rewriter(const DFPattern& pattern, const RewriteCallback& cb) : pattern_(pattern), cb_(cb) {}
+  Rewriter(const DFPattern& pattern, const RewriteCallback& cb, const Expr& root)
+      : pattern_(pattern), cb_(cb), call_patterns_(CallPatternsOf(pattern)) {
+    CountUses(root);
+  }
 
   Expr Mutate(const Expr& e) {
     auto it = memo_.find(e.get());
@@ -369,8 +384,10 @@ class Rewriter {
         changed = changed || args.back().get() != a.get();
       }
       if (changed) post = MakeCall(op, args, c->type);
+      origin_[post.get()] = e.get();
       NodeMap node_map;
-      if (MatchPattern(pattern_, post, &node_map)) post = cb_(e, post, node_map);
+      if (MatchPattern(pattern_, post, &node_map) && InteriorIsPrivate(post, node_map))
+        post = cb_(e, post, node_map);
     } else if (const auto* f = AsFunction(e)) {
       if (!IsPrimitive(f)) {
         Expr body = Mutate(f->body);
@@ -383,13 +400,60 @@ class Rewriter {
   }
 
  private:
+  // How many argument slots of the graph refer to each expression.
+  void CountUses(const Expr& e) {
+    if (!e || !counted_.insert(e.get()).second) return;
+    if (const auto* c = AsCall(e)) {
+      CountUses(c->op);
+      for (const auto& a : c->args) {
+        ++uses_[a.get()];
+        CountUses(a);
+      }
+    } else if (const auto* f = AsFunction(e)) {
+      ++uses_[f->body.get()];
+      CountUses(f->body);
+    }
+  }
+
+  // A match of several calls is replaced by its root alone, so the calls inside it must have no
+  // consumer outside it: such a consumer would keep the old call alive next to the fused one, and
+  // an operator with out= would then run twice.  (The reference leaves this to the pattern writer.)
+  bool InteriorIsPrivate(const Expr& root, const NodeMap& node_map) const {
+    std::vector<const CallNode*> matched;
+    for (const auto* cp : call_patterns_) {
+      auto it = node_map.find(cp);
+      if (it != node_map.end()) matched.push_back(AsCall(it->second));
+    }
+    for (const CallNode* inner : matched) {
+      if (inner == root.get()) continue;
+      size_t inside = 0;
+      for (const CallNode* user : matched)
+        for (const auto& a : user->args) inside += a.get() == inner;
+      auto org = origin_.find(inner);
+      auto total = uses_.find(org == origin_.end() ? inner : org->second);
+      if (total == uses_.end() || total->second != inside) return false;
+    }
+    return true;
+  }
+
   const DFPattern& pattern_;
   const RewriteCallback& cb_;
+  std::vector<const DFPatternNode*> call_patterns_;
+  std::set<const ExprNode*> counted_;
+  std::map<const ExprNode*, size_t> uses_;
+  std::map<const ExprNode*, const ExprNode*> origin_;  // rebuilt call -> the call it was made from
   std::map<const ExprNode*, Expr> memo_;
   std::vector<Expr> keep_alive_;
 };
 
 }  // namespace
+
+std::vector<const DFPatternNode*> CallPatternsOf(const DFPattern& pattern) {
+  std::set<const DFPatternNode*> seen;
+  std::vector<const DFPatternNode*> calls;
+  CollectCallPatternNodes(pattern, &seen, &calls);
+  return calls;
+}
 
 bool MatchPattern(const DFPattern& pattern, const Expr& expr, NodeMap* node_map) {
   Matcher m;
@@ -399,7 +463,7 @@ bool MatchPattern(const DFPattern& pattern, const Expr& expr, NodeMap* node_map)
 }
 
 Expr RewritePatterns(const DFPattern& pattern, const RewriteCallback& callback, const Expr& expr) {
-  return Rewriter(pattern, callback).Mutate(expr);
+  return Rewriter(pattern, callback, expr).Mutate(expr);
 }
 
 }  // namespace ir
@@ -516,17 +580,6 @@ namespace {
 
 using ir::Expr;
 
-void CollectCallPatterns(const ir::DFPattern& p, std::set<const ir::DFPatternNode*>* seen,
-                         std::vector<const ir::DFPatternNode*>* calls) {
-  if (!p || !seen->insert(p.get()).second) return;
-  if (p->kind == ir::DFPatternNode::kCall) calls->push_back(p.get());
-  CollectCallPatterns(p->op, seen, calls);
-  for (const auto& a : p->args) CollectCallPatterns(a, seen, calls);
-  CollectCallPatterns(p->left, seen, calls);
-  CollectCallPatterns(p->right, seen, calls);
-  CollectCallPatterns(p->inner, seen, calls);
-}
-
 class FuseMutator {
  public:
   FuseMutator(const std::string& dialect, const std::set<const ir::ExprNode*>& call_set,
@@ -596,9 +649,7 @@ ir::Expr FuseDialect(const ir::Expr& expr, DevType device_type) {
   const op::DialectFusePattern::PatternList patterns = *op::DialectFusePattern::Get();
   for (const auto& pat : patterns) {
     if (!op::Dialect::IsEnabled(pat.dialect, device_type)) continue;
-    std::set<const ir::DFPatternNode*> seen;
-    std::vector<const ir::DFPatternNode*> call_patterns;
-    CollectCallPatterns(pat.pattern, &seen, &call_patterns);
+    const std::vector<const ir::DFPatternNode*> call_patterns = ir::CallPatternsOf(pat.pattern);
     std::unordered_map<std::string, Expr> func_cache;
     auto callback = [&](const Expr& pre, const Expr& post, const ir::NodeMap& node_map) -> Expr {
       (void)pre;

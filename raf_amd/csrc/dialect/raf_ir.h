@@ -145,11 +145,14 @@ DFPattern has_dtype(const DType& dtype, DFPattern inner = nullptr);  // inner de
 // pattern node -> the expression it matched.  A pattern node that occurs several times in a
 // pattern must match one and the same expression everywhere.
 using NodeMap = std::map<const DFPatternNode*, Expr>;
+// Every call node of a pattern (the reference's CallPatternExtractor, src/pass/fuse_dialect.cc:27-43).
+std::vector<const DFPatternNode*> CallPatternsOf(const DFPattern& pattern);
 bool MatchPattern(const DFPattern& pattern, const Expr& expr, NodeMap* node_map = nullptr);
 
 // Rewrites bottom-up: every sub-expression (after its arguments were rewritten) that matches
 // `pattern` is replaced by callback(pre, post, node_map); the bodies of primitive functions are
-// left alone.
+// left alone.  A match whose inner calls have consumers outside the match is skipped: the
+// replacement keeps the root only, so those consumers would hold on to the old calls.
 using RewriteCallback = std::function<Expr(const Expr& pre, const Expr& post, const NodeMap&)>;
 Expr RewritePatterns(const DFPattern& pattern, const RewriteCallback& callback, const Expr& expr);
 

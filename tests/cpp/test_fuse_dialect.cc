@@ -202,6 +202,31 @@ int main() {
     EXPECT(pass::FuseDialect(sched, DevType::kROCM()).get() == sched.get());
   }
 
+  std::puts("no fusion when a value inside the match is also used outside it");
+  {
+    // new_v feeds the weight update and is returned as well: fusing would leave the old add(out=v)
+    // alive beside the fused function, and v would be updated twice
+    Expr mv = MakeCall(GetOp("raf.op.multiply"), {MakeFloat(0.9), v}, TypeOf(v));
+    Expr nv = MakeCall(GetOp("raf.op.add"), {mv, dx, v, MakeNull()}, TypeOf(v));
+    Expr st = MakeCall(GetOp("raf.op.multiply"), {MakeFloat(0.01), nv}, TypeOf(v));
+    Expr nw = MakeCall(GetOp("raf.op.subtract"), {w, st, w, MakeNull()}, TypeOf(w));
+    Expr both = MakeCall(GetOp("raf.op.tuple3"), {nw, nv, dx});
+    EXPECT(pass::FuseDialect(both, DevType::kROCM()).get() == both.get());
+    // the same update without the second consumer is fused, also below another call
+    Expr alone = MakeCall(GetOp("raf.op.tuple3"), {nw, dx, dx});
+    Expr fused = pass::FuseDialect(alone, DevType::kROCM());
+    EXPECT(fused.get() != alone.get() && AsFunction(AsCall(AsCall(fused)->args[0])->op) != nullptr);
+    // a shared dense: dense+relu may not swallow it, the one-call pattern still lowers it once
+    Expr x = MakeVar("x", Ty({10, 20})), k = MakeVar("k", Ty({30, 20}));
+    Expr dense = MakeCall(GetOp("raf.op.dense"), {x, k}, Ty({10, 30}));
+    Expr act = MakeCall(GetOp("raf.op.relu"), {dense}, Ty({10, 30}));
+    Expr shared = MakeCall(GetOp("raf.op.tuple3"), {act, dense, x});
+    Expr got = pass::FuseDialect(shared, DevType::kCPU());
+    Expr low = MakeCall(GetOp("raf.op.fakeblas.dense"), {x, k}, Ty({10, 30}));
+    Expr want = MakeCall(GetOp("raf.op.tuple3"), {MakeCall(GetOp("raf.op.relu"), {low}, Ty({10, 30})), low, x});
+    EXPECT(StructuralEqual(got, want));
+  }
+
   std::puts("updates of equal type share one fused function; another shape gets its own");
   {
     Expr w2 = MakeVar("w2", Ty({1024, 1024})), dx2 = MakeVar("dx2", Ty({1024, 1024})), v2 = MakeVar("v2", Ty({1024, 1024}));
