@@ -229,6 +229,9 @@ class SgdUpdateFusedEnv : public OpEnv {
   static OpEnv* make(const CallValues& cv) { return new SgdUpdateFusedEnv(cv); }
 
  private:
+  // A Python float reaches the traced graph as a float64 scalar constant
+  // (src/op/regs/ffi2expr.h:41-43); the kernel entry points round it to fp32 once, as raf.op.sgd
+  // does with tir.const(value, dtype) (python/raf/_tvm_op/sgd.py:18-19).
   static bool Scalar(const Value& v, double* out) {
     if (auto f = std::dynamic_pointer_cast<FloatValueObj>(v)) {
       *out = f->value;
