@@ -85,3 +85,27 @@ def test_unfusable_graphs_find_no_backend(native_libs):
     w32 = torch.zeros(16, device=DEV)
     with pytest.raises(RafError, match="differ in shape"):
         op.traced_sgd_update(w32, torch.zeros(1, device=DEV), w32.clone(), 0.1, 0.9)
+
+
+def test_traced_update_trains_like_torch_sgd(native_libs):
+    """The reference's test of its traced optimizer (tests/python/optim/test_sgd.py:151-172): a 2x2
+    parameter under relu, random output gradients, 32 steps of with_sgd(0.1, 0.01) against
+    torch.optim.SGD at 1e-4 -- here with the traced update taken through the fusion pass."""
+    from raf_amd import op
+
+    torch.manual_seed(0)
+    shape = (2, 2)
+    x_t = torch.nn.Parameter(torch.randn(*shape, device=DEV))
+    t_opt = torch.optim.SGD([x_t], lr=0.1, momentum=0.01)
+    x_m = x_t.detach().clone()
+    v_m = torch.zeros_like(x_m)
+    grad = torch.empty_like(x_m)
+    update = op.TracedSgdUpdate(x_m, grad, v_m, 0.1, 0.01)
+    for _ in range(32):
+        dy = torch.randn(*shape, device=DEV)
+        t_opt.zero_grad()
+        torch.relu(x_t).backward(dy)
+        t_opt.step()
+        grad.copy_(dy * (x_m > 0))  # relu's gradient at our own parameter
+        update()
+        np.testing.assert_allclose(x_m.cpu().numpy(), x_t.detach().cpu().numpy(), rtol=1e-4, atol=1e-4)
