@@ -195,6 +195,9 @@ int64_t rafhip_lans_plan_total_elements(const rafhip_lans_plan* plan);
  * Arithmetic: scalars are the fp32 schema values; everything per element and every norm is
  * evaluated in float64 and rounded once to fp32 on store.
  */
+/* A pipelined step whose bounded waits ran out (which no correct run does) leaves invalid results.
+ * The failure is reported by rafhip_lans_read_norms of that step, or else by the NEXT step call on
+ * the plan, which then returns RAFHIP_ERR_HIP without launching anything; either report clears it. */
 int rafhip_lans_step(rafhip_lans_plan* plan, const void* const* g, float* const* w,
                      float* const* m, float* const* v, const float* step_dev, int32_t step_host,
                      const rafhip_lans_hparams* hp, void* workspace, int64_t workspace_bytes,

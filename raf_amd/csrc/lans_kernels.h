@@ -146,6 +146,7 @@ struct LansDeviceArgs {
   uint32_t n_items;       // pipelined work-list length
   const WorkItem* pipeline_items;
   uint32_t spin_limit;    // pipelined: bound of every wait, in polls
+  uint32_t* host_error;   // pipelined: pinned host word raised together with sync->error, or nullptr
   float unscale;
   int32_t p_is_bf16;      // dtype of the optional 16-bit weight copies: 0 binary16, 1 bfloat16
   StepScalars* scalars;

@@ -101,8 +101,9 @@ __device__ __forceinline__ void publish(double* p, double v) {
 // cache line of the ticket, which every workgroup hammers with atomics (reading the bound from
 // there made the whole step 12 % slower).
 struct WaitCtx {
-  uint32_t* error;  // set to 1 when a wait runs out
-  uint32_t limit;   // polls a wait may take
+  uint32_t* error;       // set to 1 when a wait runs out
+  uint32_t limit;        // polls a wait may take
+  uint32_t* host_error;  // the same flag in pinned host memory, which the host can read without a copy
 };
 __device__ __forceinline__ double wait_published(const double* word, const WaitCtx& wc) {
   uint64_t bits = ld_bits(word);
@@ -110,6 +111,7 @@ __device__ __forceinline__ double wait_published(const double* word, const WaitC
   while (bits == kNotReady) {
     if (++spins > wc.limit) {
       __hip_atomic_store(wc.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (wc.host_error) __hip_atomic_store(wc.host_error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
       break;
     }
     __builtin_amdgcn_s_sleep(8);
@@ -594,11 +596,11 @@ __global__ __launch_bounds__(kLansBlock) void lans_finish(LansDeviceArgs a, int 
   const StepScalars k = *a.scalars;
   if (after_b) {
     double tot[3], r0, r1;
-    tensor_totals<3, false>(part, 1, chunks_of(tr), 1, tot, red, WaitCtx{nullptr, 0});
+    tensor_totals<3, false>(part, 1, chunks_of(tr), 1, tot, red, WaitCtx{nullptr, 0, nullptr});
     if (threadIdx.x == 0) stats_after_b(&a.stats[t], tot, k, r0, r1);
   } else {
     double tot[1];
-    tensor_totals<1, false>(part, 0, units_a_of(tr), kChunksPerA, tot, red, WaitCtx{nullptr, 0});
+    tensor_totals<1, false>(part, 0, units_a_of(tr), kChunksPerA, tot, red, WaitCtx{nullptr, 0, nullptr});
     if (threadIdx.x == 0) stats_after_a(&a.stats[t], tot[0], k);
   }
 }
@@ -620,7 +622,7 @@ __global__ __launch_bounds__(kLansBlock) void lans_norm_u(LansDeviceArgs a) {
     if constexpr (kMode == kModeResidentInline) {
       double tot[1];
       tensor_totals<1, false>(a.partials + kPartialSlots * (int64_t)tr.first_chunk, 0, units_a_of(tr),
-                              kChunksPerA, tot, red, WaitCtx{nullptr, 0});
+                              kChunksPerA, tot, red, WaitCtx{nullptr, 0, nullptr});
       if (chunk == 0 && threadIdx.x == 0)  // one workgroup per tensor leaves the statistics
         inv_gdiv = stats_after_a(&a.stats[it.tensor], tot[0], k);
       else
@@ -653,7 +655,7 @@ __global__ __launch_bounds__(kLansBlock) void lans_apply(LansDeviceArgs a) {
     if constexpr (kMode == kModeResidentInline) {
       double tot[3];
       tensor_totals<3, false>(a.partials + kPartialSlots * (int64_t)tr.first_chunk, 1, chunks_of(tr), 1,
-                              tot, red, WaitCtx{nullptr, 0});
+                              tot, red, WaitCtx{nullptr, 0, nullptr});
       p.inv_gdiv = a.stats[it.tensor].inv_grad_div;  // left by pass B
       if (chunk == 0 && threadIdx.x == 0)
         stats_after_b(&a.stats[it.tensor], tot, k, p.rm, p.rg);
@@ -674,7 +676,7 @@ __global__ __launch_bounds__(kLansBlock) void lans_pipelined(LansDeviceArgs a) {
   __shared__ double s_bcast[3];
   __shared__ uint32_t s_ticket;
   const StepScalars k = *a.scalars;
-  const WaitCtx wc{&a.sync->error, a.spin_limit};
+  const WaitCtx wc{&a.sync->error, a.spin_limit, a.host_error};
 
   // Thread 0 draws tickets two items ahead, so an atomic's round trip is hidden behind a whole
   // item, and every thread reads the NEXT item's descriptor and tensor record while the current

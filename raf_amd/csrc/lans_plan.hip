@@ -180,6 +180,10 @@ struct rafhip_lans_plan {
   int64_t n_items_a = 0;
   WorkItem* d_pipeline = nullptr;
   uint64_t* d_trace = nullptr;  // diagnostics, only with RAFHIP_LANS_TRACE=1
+  // One word of pinned, device-visible host memory: the persistent kernel raises it when a bounded
+  // wait runs out, and the next call on the plan reports it without any copy or synchronisation.
+  uint32_t* host_error = nullptr;
+  uint32_t* host_error_dev = nullptr;  // the device's address of the same word
 
   RecordUploader<TensorRec> tensors;  // a step whose pointers did not move sends nothing
 
@@ -203,6 +207,7 @@ void free_plan(rafhip_lans_plan* p) {
   p->tensors.release();
   if (p->d_tables) (void)hipFree(p->d_tables);
   if (p->d_trace) (void)hipFree(p->d_trace);
+  if (p->host_error) (void)hipHostFree(p->host_error);
   delete p;
 }
 
@@ -369,6 +374,12 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
       if (e == hipSuccess && !pipeline.empty())
         e = hipMemcpy(p->d_pipeline, pipeline.data(), sizeof(WorkItem) * pipeline.size(),
                       hipMemcpyHostToDevice);
+      if (e == hipSuccess)
+        e = hipHostMalloc(reinterpret_cast<void**>(&p->host_error), 64, hipHostMallocMapped);
+      if (e == hipSuccess) {
+        *p->host_error = 0u;
+        e = hipHostGetDevicePointer(reinterpret_cast<void**>(&p->host_error_dev), p->host_error, 0);
+      }
       if (e == hipSuccess && std::getenv("RAFHIP_LANS_TRACE") && !pipeline.empty())
         e = hipMalloc(reinterpret_cast<void**>(&p->d_trace), 32 * pipeline.size());
       if (e != hipSuccess)
@@ -434,6 +445,13 @@ int rafhip_lans_step_mixed(rafhip_lans_plan* plan, const void* const* g, float* 
                 hp->mode);
   const int32_t n = plan->n_tensors;
   if (n == 0 || plan->n_chunks == 0) return RAFHIP_OK;  // nothing to update
+  if (plan->host_error && __atomic_load_n(plan->host_error, __ATOMIC_RELAXED) != 0) {
+    // Raised by the persistent kernel of an earlier step; reported once, then the plan works on.
+    __atomic_store_n(plan->host_error, 0u, __ATOMIC_RELAXED);
+    return fail(RAFHIP_ERR_HIP,
+                "rafhip_lans_step: an earlier pipelined step on this plan ran out of a bounded wait; "
+                "its results are invalid (this call did nothing)");
+  }
   if (!g || !w || !m || !v)
     return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_step: null pointer list");
   return guarded("rafhip_lans_step", [&]() -> int {
@@ -486,6 +504,7 @@ int rafhip_lans_step_mixed(rafhip_lans_plan* plan, const void* const* g, float* 
     a.pipeline_items = plan->d_pipeline;
     a.unscale = hp->grad_unscale;
     a.spin_limit = plan->spin_limit;
+    a.host_error = plan->host_error_dev;
     a.p_is_bf16 = p_dtype == RAFHIP_BF16 ? 1 : 0;
     a.scalars = reinterpret_cast<StepScalars*>(ws + plan->ws.scalars_off);
     a.stats = reinterpret_cast<TensorStats*>(ws + plan->ws.stats_off);
@@ -552,10 +571,12 @@ int rafhip_lans_read_norms(const rafhip_lans_plan* plan, const void* workspace, 
       host_out[4 * t + 2] = st[t].um_norm;
       host_out[4 * t + 3] = st[t].ug_norm;
     }
-    if (plan->n_chunks > 0 && sync.error != 0)
+    if (plan->n_chunks > 0 && sync.error != 0) {
+      if (plan->host_error) __atomic_store_n(plan->host_error, 0u, __ATOMIC_RELAXED);  // reported here
       return fail(RAFHIP_ERR_HIP,
                   "rafhip_lans_read_norms: the last pipelined step ran out of a bounded wait; its "
                   "results are invalid");
+    }
     return RAFHIP_OK;
   });
 }

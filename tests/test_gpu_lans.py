@@ -425,6 +425,14 @@ def test_a_wait_that_runs_out_is_reported_not_hung(native_libs, monkeypatch):
     torch.cuda.synchronize()  # returns: no workgroup is left waiting
     with pytest.raises(native_libs.RafHipError, match="bounded wait"):
         plan.read_norms()
+    # a caller that never reads the norms learns of it from the next step on the plan, once
+    plan.step(tg, tw, tm, tv, 2, _khp(hp))  # the report above cleared the flag: this one runs (and times out)
+    torch.cuda.synchronize()
+    with pytest.raises(native_libs.RafHipError, match="earlier pipelined step .* bounded wait"):
+        plan.step(tg, tw, tm, tv, 3, _khp(hp))
+    plan.set_schedule("phased")
+    plan.step(tg, tw, tm, tv, 3, _khp(hp))  # reported once; the plan works on
+    torch.cuda.synchronize()
     plan.close()
     monkeypatch.delenv("RAFHIP_LANS_SPIN_LIMIT")
     tg, tw, tm, tv = _to_dev(g), _to_dev(w), _to_dev(m), _to_dev(v)
