@@ -142,6 +142,24 @@ template <int N, bool kWait>
 __device__ __forceinline__ void tensor_totals(const double* partials, int slot, int64_t n_units,
                                               int chunks_per_unit, double (&tot)[N],
                                               double (*red)[kLansWaves], const WaitCtx& wc) {
+  if (n_units == 1) {
+    // One unit: the total is that partial (0 + x, as the tree below would form it), which every
+    // thread can read for itself -- no trip through LDS and two barriers for the many one-chunk
+    // tensors of a list of small tensors.
+    const double* p = partials + slot;
+    if (kWait) {
+      const double* words[N];
+#pragma unroll
+      for (int j = 0; j < N; ++j) words[j] = p + j;
+      wait_published_n<N>(words, tot, wc);
+    } else {
+#pragma unroll
+      for (int j = 0; j < N; ++j) tot[j] = ld_dev(p + j);
+    }
+#pragma unroll
+    for (int j = 0; j < N; ++j) tot[j] = 0.0 + tot[j];
+    return;
+  }
 #pragma unroll
   for (int j = 0; j < N; ++j) tot[j] = 0.0;
   for (int64_t i = threadIdx.x; i < n_units; i += kLansBlock) {
