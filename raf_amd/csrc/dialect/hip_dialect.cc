@@ -16,6 +16,7 @@
 // arguments are reported through error_msgs so dispatch can fall through to another dialect.
 #include "hip_dialect.h"
 
+#include <atomic>
 #include <sstream>
 
 #include "raf_iface.h"
@@ -32,7 +33,7 @@ using value::Value;
 
 namespace {
 
-float g_lans_grad_unscale = 1.0f;
+std::atomic<float> g_lans_grad_unscale{1.0f};  // set by one thread, read by makers on any thread
 
 std::string KernelError(const char* what, int status) {
   std::ostringstream ss;
@@ -49,8 +50,8 @@ int32_t KernelDType(const DType& t) {
 
 }  // namespace
 
-void SetLansGradUnscale(float factor) { g_lans_grad_unscale = factor; }
-float GetLansGradUnscale() { return g_lans_grad_unscale; }
+void SetLansGradUnscale(float factor) { g_lans_grad_unscale.store(factor, std::memory_order_relaxed); }
+float GetLansGradUnscale() { return g_lans_grad_unscale.load(std::memory_order_relaxed); }
 
 // ----------------------------------------------------------------------------------------- SGD
 class SgdHipEnv : public OpEnv, public HasLearningRate {
