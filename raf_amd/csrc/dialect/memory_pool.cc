@@ -1,6 +1,7 @@
 // Pool manager and the two pool strategies declared in memory_pool.h.
 #include "memory_pool.h"
 
+#include <cstdio>
 #include <cstdlib>
 #include <list>
 #include <map>
@@ -56,6 +57,19 @@ void CheckAlignment(int64_t alignment) {  // src/impl/memory_pool.cc:83-87
 
 bool IsGpu(DevType t) { return t == DevType::kCUDA() || t == DevType::kROCM(); }
 
+// A destructor must not throw: a failed release (the device API reports failures as raf::Error)
+// is written to stderr and otherwise dropped.
+template <typename F>
+void Release(F&& free_it) noexcept {
+  try {
+    free_it();
+  } catch (const std::exception& e) {
+    std::fprintf(stderr, "raf memory pool: releasing memory failed: %s\n", e.what());
+  } catch (...) {
+    std::fprintf(stderr, "raf memory pool: releasing memory failed\n");
+  }
+}
+
 // ---------------------------------------------------------------------------------- chunks
 // Memory returned to the device API when the last reference goes.
 class NonOwnedMemory final : public Memory {
@@ -65,7 +79,7 @@ class NonOwnedMemory final : public Memory {
     device = dev;
   }
   ~NonOwnedMemory() override {
-    if (data != nullptr) api_->FreeMemory(data);
+    if (data != nullptr) Release([&] { api_->FreeMemory(data); });
   }
 
  private:
@@ -81,7 +95,7 @@ class NonOwnedAsyncMemory final : public Memory {
     device = dev;
   }
   ~NonOwnedAsyncMemory() override {
-    if (data != nullptr) api_->FreeMemoryAsync(data, stream_);
+    if (data != nullptr) Release([&] { api_->FreeMemoryAsync(data, stream_); });
   }
 
  private:
