@@ -142,6 +142,7 @@ int run(rafhip_fuse_plan* plan, const char* what, void* const* parts, void* flat
   clear_error();
   if (!plan) return fail(RAFHIP_ERR_INVALID_ARG, "%s: plan is NULL", what);
   if (plan->n_items == 0) return RAFHIP_OK;  // nothing to move
+  if (int st = check_plan_device(what, plan->device)) return st;
   if (!parts || !flat) return fail(RAFHIP_ERR_INVALID_ARG, "%s: null pointer argument", what);
   return guarded(what, [&]() -> int {
     std::vector<Segment> segs((size_t)plan->n);

@@ -445,6 +445,7 @@ int rafhip_lans_step_mixed(rafhip_lans_plan* plan, const void* const* g, float* 
                 hp->mode);
   const int32_t n = plan->n_tensors;
   if (n == 0 || plan->n_chunks == 0) return RAFHIP_OK;  // nothing to update
+  if (int st = check_plan_device("rafhip_lans_step", plan->device)) return st;
   if (plan->host_error && __atomic_load_n(plan->host_error, __ATOMIC_RELAXED) != 0) {
     // Raised by the persistent kernel of an earlier step; reported once, then the plan works on.
     __atomic_store_n(plan->host_error, 0u, __ATOMIC_RELAXED);

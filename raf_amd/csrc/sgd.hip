@@ -233,6 +233,7 @@ extern "C" int rafhip_sgd_f32(const float* x, const float* dx, const float* v, f
 struct rafhip_sgd_plan {
   int32_t n = 0;
   int32_t grad_dtype = RAFHIP_F32;
+  int device = 0;
   std::vector<int64_t> numel;
   int64_t total_elements = 0;
   int64_t n_items = 0;
@@ -286,8 +287,7 @@ extern "C" int rafhip_sgd_plan_create(int32_t n_tensors, const int64_t* numel, i
       *out_plan = p.release();
       return RAFHIP_OK;
     }
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) {
+    if (hipGetDevice(&p->device) != hipSuccess) {
       (void)hipGetLastError();
       return fail(RAFHIP_ERR_NO_DEVICE, "rafhip_sgd_plan_create: no HIP device available");
     }
@@ -322,6 +322,7 @@ extern "C" int rafhip_sgd_multi_step(rafhip_sgd_plan* plan, float* const* x, con
     return fail(RAFHIP_ERR_UNSUPPORTED,
                 "rafhip_sgd_multi_step: weight-copy dtype %d (binary16 or bfloat16)", p_dtype);
   if (plan->n_items == 0) return RAFHIP_OK;
+  if (int st = check_plan_device("rafhip_sgd_multi_step", plan->device)) return st;
   if (!x || !dx || !v) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_sgd_multi_step: null pointer list");
   return guarded("rafhip_sgd_multi_step", [&]() -> int {
     const uintptr_t g_elem = plan->grad_dtype == RAFHIP_F32 ? 4 : 2;

@@ -15,6 +15,20 @@ namespace rafhip {
 int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 void clear_error();
 
+// A plan's tables live on the device that was current when it was made; running it with another
+// device current would hand the kernels pointers into the wrong address space.
+inline int check_plan_device(const char* who, int plan_device) {
+  int now = -1;
+  if (hipGetDevice(&now) != hipSuccess) {
+    (void)hipGetLastError();
+    return fail(RAFHIP_ERR_NO_DEVICE, "%s: no HIP device available", who);
+  }
+  if (now != plan_device)
+    return fail(RAFHIP_ERR_INVALID_ARG, "%s: the plan was made on device %d, the current device is %d", who,
+                plan_device, now);
+  return RAFHIP_OK;
+}
+
 // No C++ exception may cross the C boundary: entry points that allocate host memory (work lists,
 // tables) run their body through this and report a failure as RAFHIP_ERR_HOST instead.
 template <typename F>
