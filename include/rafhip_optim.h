@@ -220,6 +220,26 @@ int rafhip_lans_step_mixed(rafhip_lans_plan* plan, const void* const* g, float* 
                            const rafhip_lans_hparams* hp, void* workspace,
                            int64_t workspace_bytes, void* stream);
 
+/*
+ * rafhip_lans_step_mixed without the workspace arguments, for callers that cannot allocate device
+ * memory and have no workspace to hand over: code running under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose executors
+ * allocate the requested workspaces around every call).  The step scalars, per-tensor statistics
+ * and chunk partial sums live in an array of RAFHIP_LANS_STATIC_SCRATCH_BYTES that is part of the
+ * library's device code: every GPU the library is used on holds its own copy until the process
+ * ends.  The call itself allocates nothing, on the device or on the host, and gives the same bits
+ * as rafhip_lans_step_mixed.  A plan whose rafhip_lans_workspace_bytes exceeds
+ * RAFHIP_LANS_STATIC_SCRATCH_BYTES (lists beyond roughly two billion elements or 80 000 tensors)
+ * is refused with RAFHIP_ERR_WORKSPACE.  All calls on one GPU share that GPU's array: two such
+ * steps that overlap in time on one GPU (different streams or threads) race; calls on one stream
+ * are ordered and safe.  p may be NULL.
+ */
+#define RAFHIP_LANS_STATIC_SCRATCH_BYTES (8 * 1024 * 1024)
+int rafhip_lans_step_noalloc(rafhip_lans_plan* plan, const void* const* g, float* const* w,
+                             float* const* m, float* const* v, void* const* p, int32_t p_dtype,
+                             const float* step_dev, int32_t step_host,
+                             const rafhip_lans_hparams* hp, void* stream);
+
 /* Copies the per-tensor norms left in the workspace by the last step on `stream`
  * (4 doubles per tensor: ||g||, ||w||, ||u_m||, ||u_g||) to host memory; synchronises `stream`. */
 int rafhip_lans_read_norms(const rafhip_lans_plan* plan, const void* workspace, double* host_out,

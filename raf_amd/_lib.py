@@ -29,6 +29,7 @@ RAFHIP_F64 = 3
 
 RAFHIP_LANS_PHASED = 0
 RAFHIP_LANS_PIPELINED = 1
+RAFHIP_LANS_STATIC_SCRATCH_BYTES = 8 * 1024 * 1024
 
 
 class RafHipError(RuntimeError):
@@ -86,6 +87,9 @@ OPTIM_SYMBOLS = {
     "rafhip_lans_step_mixed": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
                                        POINTER(c_void_p), POINTER(c_void_p), c_int32, c_void_p, c_int32,
                                        POINTER(LansHParams), c_void_p, c_int64, c_void_p]),
+    "rafhip_lans_step_noalloc": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
+                                         POINTER(c_void_p), POINTER(c_void_p), c_int32, c_void_p, c_int32,
+                                         POINTER(LansHParams), c_void_p]),
     "rafhip_sgd_plan_create": (c_int, [c_int32, POINTER(c_int64), c_int32, POINTER(c_void_p)]),
     "rafhip_sgd_plan_destroy": (c_int, [c_void_p]),
     "rafhip_sgd_multi_step": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),

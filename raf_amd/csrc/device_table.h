@@ -34,6 +34,9 @@ class RecordUploader {
                                  hipHostMallocDefault);
     if (e == hipSuccess) e = hipEventCreateWithFlags(&staging_free_, hipEventDisableTiming);
     if (e != hipSuccess) release();
+    // Its final size from the start: sync() swaps it with the caller's vector, so neither side
+    // ever has to grow (a step allocates nothing, host memory included).
+    if (e == hipSuccess) last_sent_.assign(count, Rec{});
     return e;
   }
 

@@ -10,6 +10,7 @@
 #include <cstring>
 #include <limits>
 #include <memory>
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -18,6 +19,13 @@
 #include "status.h"
 
 using namespace rafhip;
+
+// Scratch memory of rafhip_lans_step_noalloc, the step for callers that cannot allocate: the
+// step scalars, per-tensor statistics, chunk partial sums and ticket words that the other step
+// entry points find in the caller's workspace.  Every GPU the library runs on holds its own copy
+// of the array, at its own address, until the process ends.  In host code the name below is only
+// a handle for hipGetSymbolAddress; the kernels receive the resolved address as an argument.
+static __device__ __align__(256) unsigned char scratch[RAFHIP_LANS_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -154,6 +162,32 @@ int schedule_setting(int64_t total_elements) {
   return total_elements >= kPipelinedFromElems ? RAFHIP_LANS_PIPELINED : RAFHIP_LANS_PHASED;
 }
 
+// The address of `scratch` on a device, resolved once per device with that device current.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// `device` must be the current device.  Returns nullptr (and leaves the reason in *err) on failure.
+void* static_scratch_of(int device, hipError_t* err) {
+  *err = hipSuccess;
+  if (device < 0 || device >= kMaxDevices) {
+    *err = hipErrorInvalidDevice;
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[device]) {
+    void* ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      (void)hipGetLastError();
+      *err = e != hipSuccess ? e : hipErrorInvalidSymbol;
+      return nullptr;
+    }
+    g_scratch_ptr[device] = ptr;
+  }
+  return g_scratch_ptr[device];
+}
+
 }  // namespace
 
 struct rafhip_lans_plan {
@@ -186,6 +220,12 @@ struct rafhip_lans_plan {
   uint32_t* host_error_dev = nullptr;  // the device's address of the same word
 
   RecordUploader<TensorRec> tensors;  // a step whose pointers did not move sends nothing
+  std::vector<TensorRec> recs;        // this call's records, built in place: a step allocates nothing
+
+  // This device's address of the static scratch array (rafhip_lans_step_noalloc), resolved when the
+  // plan is made; nullptr with the reason in static_scratch_error if that failed.
+  void* static_scratch = nullptr;
+  hipError_t static_scratch_error = hipSuccess;
 
   // Optional per-kernel timing: slots x 6 events.
   std::vector<std::array<hipEvent_t, 6>> timing;
@@ -228,6 +268,11 @@ int validate_list(const char* who, int32_t n_tensors, const int64_t* numel) {
   }
   return RAFHIP_OK;
 }
+
+int lans_step_impl(rafhip_lans_plan* plan, const void* const* g, float* const* w, float* const* m,
+                   float* const* v, void* const* p, int32_t p_dtype, const float* step_dev,
+                   int32_t step_host, const rafhip_lans_hparams* hp, void* workspace,
+                   int64_t workspace_bytes, void* stream);
 
 }  // namespace
 
@@ -325,6 +370,8 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, p->device) == hipSuccess &&
         cus > 0)
       p->n_cus = cus;
+    p->static_scratch = static_scratch_of(p->device, &p->static_scratch_error);
+    p->recs.resize((size_t)n_tensors);
 
     if (n_tensors > 0) {
       std::vector<WorkItem> phased((size_t)chunks);
@@ -436,6 +483,39 @@ int rafhip_lans_step_mixed(rafhip_lans_plan* plan, const void* const* g, float* 
                            int64_t workspace_bytes, void* stream) {
   clear_error();
   if (!plan) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_step: plan is NULL");
+  return lans_step_impl(plan, g, w, m, v, p, p_dtype, step_dev, step_host, hp, workspace,
+                        workspace_bytes, stream);
+}
+
+int rafhip_lans_step_noalloc(rafhip_lans_plan* plan, const void* const* g, float* const* w,
+                             float* const* m, float* const* v, void* const* p, int32_t p_dtype,
+                             const float* step_dev, int32_t step_host,
+                             const rafhip_lans_hparams* hp, void* stream) {
+  clear_error();
+  if (!plan) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_step_noalloc: plan is NULL");
+  if (plan->ws.total > (int64_t)RAFHIP_LANS_STATIC_SCRATCH_BYTES)
+    return fail(RAFHIP_ERR_WORKSPACE,
+                "rafhip_lans_step_noalloc: this tensor list needs %lld bytes of scratch, the static "
+                "buffer holds %lld; use rafhip_lans_step with a workspace of your own",
+                (long long)plan->ws.total, (long long)RAFHIP_LANS_STATIC_SCRATCH_BYTES);
+  if (plan->n_tensors > 0 && plan->n_chunks > 0 && !plan->static_scratch)
+    return fail(RAFHIP_ERR_HIP,
+                "rafhip_lans_step_noalloc: the static scratch array could not be located on device "
+                "%d when the plan was made: %s",
+                plan->device, hipGetErrorString(plan->static_scratch_error));
+  return lans_step_impl(plan, g, w, m, v, p, p_dtype, step_dev, step_host, hp, plan->static_scratch,
+                        (int64_t)RAFHIP_LANS_STATIC_SCRATCH_BYTES, stream);
+}
+
+}  // extern "C"
+
+namespace {
+
+// The step behind rafhip_lans_step, _mixed and _noalloc.  Allocates neither device nor host memory.
+int lans_step_impl(rafhip_lans_plan* plan, const void* const* g, float* const* w, float* const* m,
+                   float* const* v, void* const* p, int32_t p_dtype, const float* step_dev,
+                   int32_t step_host, const rafhip_lans_hparams* hp, void* workspace,
+                   int64_t workspace_bytes, void* stream) {
   if (p && p_dtype != RAFHIP_F16 && p_dtype != RAFHIP_BF16)
     return fail(RAFHIP_ERR_UNSUPPORTED,
                 "rafhip_lans_step: weight-copy dtype %d (binary16 or bfloat16)", p_dtype);
@@ -467,7 +547,8 @@ int rafhip_lans_step_mixed(rafhip_lans_plan* plan, const void* const* g, float* 
     // 16-byte alignment of all four selects the vector path.
     const uintptr_t g_elem = plan->grad_dtype == RAFHIP_F32 ? 4 : 2;
     const uintptr_t g_vec = 16;  // pass A reads the gradient with 16-byte lane accesses
-    std::vector<TensorRec> recs((size_t)n);
+    std::vector<TensorRec>& recs = plan->recs;
+    recs.resize((size_t)n);  // its size already: no allocation
     for (int32_t t = 0; t < n; ++t) {
       TensorRec& r = recs[t];
       r.g = g[t];
@@ -545,6 +626,10 @@ int rafhip_lans_step_mixed(rafhip_lans_plan* plan, const void* const* g, float* 
     return RAFHIP_OK;
   });
 }
+
+}  // namespace
+
+extern "C" {
 
 int rafhip_lans_read_norms(const rafhip_lans_plan* plan, const void* workspace, double* host_out,
                            void* stream) {

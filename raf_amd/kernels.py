@@ -309,6 +309,23 @@ class LansPlan:
                                               ctypes.byref(hp), ws.data_ptr(), ws.numel(),
                                               _current_stream(self.device)))
 
+    def step_noalloc(self, g, w, m, v, step, hp: LansHParams, p: Optional[Sequence] = None):
+        """``rafhip_lans_step_noalloc``: the same step on the library's static scratch array instead
+        of a workspace; no device memory is allocated by the call."""
+        pp, p_code = self._model_ptrs(p)
+        gp = self._ptrs(g, self.grad_dtype, "g")
+        wp = self._ptrs(w, torch.float32, "w")
+        mp = self._ptrs(m, torch.float32, "m")
+        vp = self._ptrs(v, torch.float32, "v")
+        if isinstance(step, torch.Tensor):
+            if step.dtype != torch.float32 or step.numel() != 1 or not step.is_cuda:
+                raise TypeError("step tensor must be a 0-d float32 GPU tensor")
+            step_dev, step_host = step.data_ptr(), 0
+        else:
+            step_dev, step_host = None, int(step)
+        check(self.lib.rafhip_lans_step_noalloc(self._h, gp, wp, mp, vp, pp, p_code, step_dev, step_host,
+                                                ctypes.byref(hp), _current_stream(self.device)))
+
     def bind(self, g, w, m, v, hp: LansHParams, workspace: Optional[torch.Tensor] = None, p=None):
         """Marshal the pointer lists once for tensors that stay where they are; ``step_bound`` then
         costs one foreign call per step (a training loop updates the same buffers every step)."""
