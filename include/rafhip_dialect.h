@@ -43,9 +43,6 @@ int rafhip_raf_dispatch_list(const char* base_op, int32_t device_type, char* buf
  * ','; pass NULL or "" to clear. */
 int rafhip_raf_set_dialect_preference(const char* dialects_csv);
 
-/* hip-dialect extension: factor applied to LANS gradients, captured by the next LANS make. */
-int rafhip_raf_set_lans_grad_unscale(float factor);
-
 /* raf.op.sgd(x, dx, v, learning_rate, mu) -> (v1, x1); python/raf/optim/sgd.py:56 */
 int rafhip_raf_sgd_make(const rafhip_tensor_desc* x, const rafhip_tensor_desc* dx,
                         const rafhip_tensor_desc* v, double learning_rate, double mu,
@@ -182,6 +179,17 @@ int rafhip_raf_env_ir_text(const rafhip_raf_env* env, int32_t fused, char* buf, 
  * new OpEnv (in the reference the learning rate is a schema constant and part of the OpEnv cache
  * key, src/impl/vm/vm.cc:1012-1015).  Fails for any other OpEnv. */
 int rafhip_raf_env_set_learning_rate(rafhip_raf_env* env, double learning_rate);
+
+/* hip-dialect extensions for loss scaling, on an OpEnv made by the lans or lans_mixed makers (the
+ * reference's LansArgs has no such field; its optimizers unscale with graph ops in front of the
+ * op).  _set_grad_unscale: every gradient element is multiplied by `factor` first (1 by default).
+ * _set_dynamic_scale: device-resident one-element float32 tensors holding that factor (the
+ * reciprocal of the current loss scale) and an overflow flag; the kernels read them when they
+ * start, and a non-zero flag turns the step into a no-op.  Either descriptor may be NULL.  None
+ * of this identifies the OpEnv: a scale change keeps the OpEnv, its plan and its tables. */
+int rafhip_raf_env_set_grad_unscale(rafhip_raf_env* env, float factor);
+int rafhip_raf_env_set_dynamic_scale(rafhip_raf_env* env, const rafhip_tensor_desc* grad_unscale,
+                                     const rafhip_tensor_desc* found_inf);
 
 /* Total bytes of the OpEnv's workspace requests (each rounded up to 256). */
 int64_t rafhip_raf_env_workspace_bytes(const rafhip_raf_env* env);

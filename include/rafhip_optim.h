@@ -173,8 +173,9 @@ int rafhip_lans_plan_destroy(rafhip_lans_plan* plan);
 int rafhip_lans_plan_set_schedule(rafhip_lans_plan* plan, int32_t schedule);
 int32_t rafhip_lans_plan_schedule(const rafhip_lans_plan* plan); /* the schedule in force; -1 on NULL */
 
-/* Bytes of caller-provided scratch a step needs (partial sums, per-tensor norms, flags); 256-byte
- * alignment required.  Returns a negative value on a NULL plan. */
+/* Bytes of caller-provided scratch a step needs (partial sums, per-tensor norms, flags); 16-byte
+ * alignment required (RAF's pools hand out 64-byte aligned blocks, include/raf/memory_pool.h).
+ * Returns a negative value on a NULL plan. */
 int64_t rafhip_lans_workspace_bytes(const rafhip_lans_plan* plan);
 int32_t rafhip_lans_plan_num_tensors(const rafhip_lans_plan* plan);
 int64_t rafhip_lans_plan_num_chunks(const rafhip_lans_plan* plan);
@@ -195,8 +196,9 @@ int64_t rafhip_lans_plan_total_elements(const rafhip_lans_plan* plan);
  * Arithmetic: scalars are the fp32 schema values; everything per element and every norm is
  * evaluated in float64 and rounded once to fp32 on store.
  */
-/* A pipelined step whose bounded waits ran out (which no correct run does) leaves invalid results.
- * The failure is reported by rafhip_lans_read_norms of that step, or else by the NEXT step call on
+/* A pipelined step whose bounded waits ran out (which no correct run does) leaves the list partly
+ * updated: every element holds either its old or its correct new value (tensors whose waits ran out
+ * keep the old ones), never garbage.  The failure is reported by rafhip_lans_read_norms of that step, or else by the NEXT step call on
  * the plan, which then returns RAFHIP_ERR_HIP without launching anything; either report clears it. */
 int rafhip_lans_step(rafhip_lans_plan* plan, const void* const* g, float* const* w,
                      float* const* m, float* const* v, const float* step_dev, int32_t step_host,
@@ -219,6 +221,34 @@ int rafhip_lans_step_mixed(rafhip_lans_plan* plan, const void* const* g, float* 
                            const float* step_dev, int32_t step_host,
                            const rafhip_lans_hparams* hp, void* workspace,
                            int64_t workspace_bytes, void* stream);
+
+/*
+ * Bound form, for tensors that stay where they are (a training loop updates the same buffers every
+ * step; the reference's VM likewise hands its cached OpEnv the same storage every iteration):
+ * rafhip_lans_plan_bind checks the pointers and builds the tensor table once, and every
+ * rafhip_lans_step_bound afterwards neither walks nor compares nor uploads the pointer lists.
+ * Same arguments and same results as rafhip_lans_step_mixed (p may be NULL).  Binding again
+ * replaces the bound tensors; other step calls on the plan may be mixed in freely.
+ */
+int rafhip_lans_plan_bind(rafhip_lans_plan* plan, const void* const* g, float* const* w,
+                          float* const* m, float* const* v, void* const* p, int32_t p_dtype);
+int rafhip_lans_step_bound(rafhip_lans_plan* plan, const float* step_dev, int32_t step_host,
+                           const rafhip_lans_hparams* hp, void* workspace, int64_t workspace_bytes,
+                           void* stream);
+
+/*
+ * Dynamic loss scaling without host round trips (extension; the reference unscales with graph ops
+ * in front of the optimizer and has no skip).  From this call on, every step on the plan
+ *   - multiplies the gradients by the fp32 value at grad_unscale_dev (the reciprocal of the current
+ *     loss scale) instead of hp->grad_unscale, when grad_unscale_dev is not NULL;
+ *   - does nothing at all -- w, m, v and the 16-bit copies keep their bits, the norms of that step
+ *     are undefined -- when the fp32 value at found_inf_dev is non-zero (the flag an overflow check
+ *     of the gradients leaves), when found_inf_dev is not NULL.
+ * Both are device pointers read by the kernels when they start, so the scale may change and a step
+ * may be skipped without a new plan, a host synchronisation or a copy.  NULL switches either off.
+ */
+int rafhip_lans_plan_set_dynamic_scale(rafhip_lans_plan* plan, const float* grad_unscale_dev,
+                                       const float* found_inf_dev);
 
 /*
  * rafhip_lans_step_mixed without the workspace arguments, for callers that cannot allocate device

@@ -183,6 +183,23 @@ def lans_step(
     return ws, ms, vs, norms
 
 
+def lans_step_dynamic_scale(g_list, w_list, m_list, v_list, step, hp: LansHParams, inv_scale, found_inf,
+                            state_dtype=np.float32):
+    """The step under dynamic loss scaling (an extension of this build; the
+    reference unscales with graph ops in front of the optimizer and has no
+    skip): the gradient is multiplied by the fp32 value ``inv_scale`` instead
+    of ``hp.grad_unscale``, and a non-zero ``found_inf`` skips the step, i.e.
+    w, m, v come back as they went in (norms are then reported as NaN)."""
+    if float(np.float32(found_inf)) != 0.0:
+        n = len(w_list)
+        keep = lambda xs: [np.array(x, copy=True) for x in xs]
+        return keep(w_list), keep(m_list), keep(v_list), np.full((n, 4), np.nan)
+    import dataclasses
+
+    return lans_step(g_list, w_list, m_list, v_list, step,
+                     dataclasses.replace(hp, grad_unscale=float(np.float32(inv_scale))), state_dtype)
+
+
 def lans_mixed_step(g_list, w_list, m_list, v_list, step, hp: LansHParams = LansHParams(),
                     model_dtype: str = "float16"):
     """The mixed-precision step of the reference's wrapper: ``lans_step`` on

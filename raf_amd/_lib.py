@@ -90,6 +90,11 @@ OPTIM_SYMBOLS = {
     "rafhip_lans_step_noalloc": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
                                          POINTER(c_void_p), POINTER(c_void_p), c_int32, c_void_p, c_int32,
                                          POINTER(LansHParams), c_void_p]),
+    "rafhip_lans_plan_bind": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
+                                      POINTER(c_void_p), POINTER(c_void_p), c_int32]),
+    "rafhip_lans_step_bound": (c_int, [c_void_p, c_void_p, c_int32, POINTER(LansHParams), c_void_p, c_int64,
+                                       c_void_p]),
+    "rafhip_lans_plan_set_dynamic_scale": (c_int, [c_void_p, c_void_p, c_void_p]),
     "rafhip_sgd_plan_create": (c_int, [c_int32, POINTER(c_int64), c_int32, POINTER(c_void_p)]),
     "rafhip_sgd_plan_destroy": (c_int, [c_void_p]),
     "rafhip_sgd_multi_step": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
@@ -125,7 +130,6 @@ DIALECT_SYMBOLS = {
     "rafhip_raf_last_error": (c_char_p, []),
     "rafhip_raf_dispatch_list": (c_int, [c_char_p, c_int32, c_char_p, c_int32]),
     "rafhip_raf_set_dialect_preference": (c_int, [c_char_p]),
-    "rafhip_raf_set_lans_grad_unscale": (c_int, [c_float]),
     "rafhip_raf_sgd_make": (c_int, [POINTER(TensorDesc), POINTER(TensorDesc), POINTER(TensorDesc),
                                     c_double, c_double, POINTER(c_void_p)]),
     "rafhip_raf_sgd_execute": (c_int, [c_void_p] + [POINTER(TensorDesc)] * 5 + [c_void_p]),
@@ -177,6 +181,8 @@ DIALECT_SYMBOLS = {
     "rafhip_raf_traced_sgd_execute": (c_int, [c_void_p] + [POINTER(TensorDesc)] * 3 + [c_void_p]),
     "rafhip_raf_env_ir_text": (c_int, [c_void_p, c_int32, c_char_p, c_int32]),
     "rafhip_raf_env_set_learning_rate": (c_int, [c_void_p, c_double]),
+    "rafhip_raf_env_set_grad_unscale": (c_int, [c_void_p, c_float]),
+    "rafhip_raf_env_set_dynamic_scale": (c_int, [c_void_p, POINTER(TensorDesc), POINTER(TensorDesc)]),
     "rafhip_raf_env_name": (c_char_p, [c_void_p]),
     "rafhip_raf_env_op": (c_char_p, [c_void_p]),
     "rafhip_raf_env_destroy": (c_int, [c_void_p]),

@@ -33,6 +33,7 @@ class RecordUploader {
     hipError_t e = hipHostMalloc(reinterpret_cast<void**>(&staging_), sizeof(Rec) * count,
                                  hipHostMallocDefault);
     if (e == hipSuccess) e = hipEventCreateWithFlags(&staging_free_, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&handover_, hipEventDisableTiming);
     if (e != hipSuccess) release();
     // Its final size from the start: sync() swaps it with the caller's vector, so neither side
     // ever has to grow (a step allocates nothing, host memory included).
@@ -44,8 +45,10 @@ class RecordUploader {
     // An upload that is still reading the staging buffer must finish before the buffer goes away.
     if (staging_free_ && sent_once_) (void)hipEventSynchronize(staging_free_);
     if (staging_free_) (void)hipEventDestroy(staging_free_);
+    if (handover_) (void)hipEventDestroy(handover_);
     if (staging_) (void)hipHostFree(staging_);
     staging_free_ = nullptr;
+    handover_ = nullptr;
     staging_ = nullptr;
     sent_once_ = false;
     last_sent_.clear();
@@ -55,29 +58,49 @@ class RecordUploader {
   // vector's contents (swap) when it uploads.
   hipError_t sync(std::vector<Rec>& recs, hipStream_t s) {
     if (count_ == 0) return hipSuccess;
+    if (sent_once_ && std::memcmp(last_sent_.data(), recs.data(), sizeof(Rec) * count_) == 0)
+      return follow(s);
+    return upload(recs, s);
+  }
+
+  // The records are the ones sent last time (the caller knows, or sync() compared them) and the
+  // next reader of the table runs on `s`.  When that is another stream than the last one, `s` is
+  // ordered behind everything enqueued there so far: behind the upload, and behind the kernels
+  // that read the table, so that the table has a single line of readers and writers however the
+  // caller moves between streams.  A stream under graph capture is left alone (events of other
+  // streams cannot be recorded into it): capture after a warm-up call on that stream has completed.
+  hipError_t follow(hipStream_t s) {
+    if (count_ == 0 || !sent_once_ || s == last_stream_) return hipSuccess;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &capturing) != hipSuccess) (void)hipGetLastError();
+    if (capturing != hipStreamCaptureStatusNone) return hipSuccess;
+    hipError_t e = order_behind_last_stream(s);
+    if (e != hipSuccess) return e;
+    last_stream_ = s;
+    return hipSuccess;
+  }
+
+ private:
+  // Everything enqueued on last_stream_ so far happens before what is enqueued on `s` from now on.
+  // If the old stream no longer exists its work has completed or is completed by the fallback.
+  hipError_t order_behind_last_stream(hipStream_t s) {
+    hipError_t e = hipEventRecord(handover_, last_stream_);
+    if (e == hipSuccess) return hipStreamWaitEvent(s, handover_, 0);
+    (void)hipGetLastError();
+    return hipDeviceSynchronize();
+  }
+
+  hipError_t upload(std::vector<Rec>& recs, hipStream_t s) {
     const size_t bytes = sizeof(Rec) * count_;
-    if (sent_once_ && std::memcmp(last_sent_.data(), recs.data(), bytes) == 0) {
-      // Same records, but a different stream than the one that carried them: order this stream
-      // behind the upload unless it has landed already.  A stream under graph capture is left
-      // alone (event queries are not allowed there): capture after a warm-up call has completed.
-      if (s != last_stream_) {
-        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing(s, &capturing) != hipSuccess) (void)hipGetLastError();
-        if (capturing == hipStreamCaptureStatusNone) {
-          if (hipEventQuery(staging_free_) == hipErrorNotReady) {
-            (void)hipGetLastError();  // "not ready" is an answer, not a failure
-            hipError_t e = hipStreamWaitEvent(s, staging_free_, 0);
-            if (e != hipSuccess) return e;
-          }
-          last_stream_ = s;
-        }
-      }
-      return hipSuccess;
-    }
-    // The previous upload may still be reading the staging buffer.
     if (sent_once_) {
+      // The previous upload may still be reading the staging buffer ...
       hipError_t e = hipEventSynchronize(staging_free_);
       if (e != hipSuccess) return e;
+      // ... and kernels launched earlier on another stream may still be reading the device table.
+      if (s != last_stream_) {
+        e = order_behind_last_stream(s);
+        if (e != hipSuccess) return e;
+      }
     }
     std::memcpy(staging_, recs.data(), bytes);
     hipError_t e = hipMemcpyAsync(device_, staging_, bytes, hipMemcpyHostToDevice, s);
@@ -89,12 +112,12 @@ class RecordUploader {
     return hipSuccess;
   }
 
- private:
   Rec* device_ = nullptr;
   size_t count_ = 0;
   Rec* staging_ = nullptr;  // pinned
   hipEvent_t staging_free_ = nullptr;  // recorded after the last upload was enqueued
-  hipStream_t last_stream_ = nullptr;  // the stream that upload went to
+  hipEvent_t handover_ = nullptr;      // orders a new stream behind the previous one
+  hipStream_t last_stream_ = nullptr;  // the stream of the last upload or reader
   std::vector<Rec> last_sent_;
   bool sent_once_ = false;
 };

@@ -26,6 +26,13 @@ struct rafhip_raf_env {
   // the FuseDialect pass and the variables to bind at Execute time.
   ir::Expr traced, fused;
   std::vector<ir::Expr> vars;
+  // The tensor list of the last execute call, as descriptors and as the tuple value made from
+  // them: a training loop passes the same tensors every step, and an executor proper would hold
+  // them as values already, so the tuple is made once and handed over again while the descriptors
+  // stay the same.
+  std::vector<rafhip_tensor_desc> list_descs;
+  std::vector<int64_t> list_shapes;
+  value::Value list_tuple;
 };
 
 namespace {
@@ -58,6 +65,34 @@ value::TensorValue FromDesc(const rafhip_tensor_desc* d, const char* what) {
   t.dtype.bits = d->dtype_bits;
   t.shape.assign(d->shape, d->shape + d->ndim);
   return value::MakeTensor(t);
+}
+
+// The tuple value of a tensor list, remade only when a descriptor differs from the last call's.
+value::Value ListTuple(rafhip_raf_env* env, int32_t n, const rafhip_tensor_desc* list, const char* what) {
+  bool same = env->list_tuple != nullptr && (size_t)n == env->list_descs.size();
+  size_t dim = 0;
+  for (int32_t i = 0; same && i < n; ++i) {
+    const rafhip_tensor_desc& a = list[i];
+    const rafhip_tensor_desc& b = env->list_descs[(size_t)i];
+    same = a.data == b.data && a.ndim == b.ndim && a.dtype_code == b.dtype_code &&
+           a.dtype_bits == b.dtype_bits && a.device_type == b.device_type && a.device_id == b.device_id &&
+           (a.ndim <= 0 || a.shape != nullptr);
+    for (int32_t d = 0; same && d < a.ndim; ++d) same = a.shape[d] == env->list_shapes[dim + (size_t)d];
+    dim += (size_t)(b.ndim > 0 ? b.ndim : 0);
+  }
+  if (same) return env->list_tuple;
+  std::vector<value::Value> fields;
+  fields.reserve((size_t)n);
+  env->list_tuple = nullptr;
+  env->list_descs.assign(list, list + n);
+  env->list_shapes.clear();
+  for (int32_t i = 0; i < n; ++i) {
+    fields.push_back(FromDesc(&list[i], what));
+    env->list_shapes.insert(env->list_shapes.end(), list[i].shape, list[i].shape + list[i].ndim);
+    env->list_descs[(size_t)i].shape = nullptr;  // the caller's array may go away; the copy above is compared
+  }
+  env->list_tuple = value::MakeTuple(std::move(fields));
+  return env->list_tuple;
 }
 
 constexpr int64_t kWsAlign = 256;
@@ -150,10 +185,6 @@ int rafhip_raf_set_dialect_preference(const char* dialects_csv) {
   });
 }
 
-int rafhip_raf_set_lans_grad_unscale(float factor) {
-  return Guard([&] { hip::SetLansGradUnscale(factor); });
-}
-
 int rafhip_raf_sgd_make(const rafhip_tensor_desc* x, const rafhip_tensor_desc* dx,
                         const rafhip_tensor_desc* v, double learning_rate, double mu,
                         rafhip_raf_env** env_out) {
@@ -237,10 +268,7 @@ int rafhip_raf_lans_execute(rafhip_raf_env* env, int32_t list_len,
     if (!env) throw Error("rafhip_raf_lans_execute: env is NULL");
     if (list_len < 0 || (list_len > 0 && !tensor_list))
       throw Error("rafhip_raf_lans_execute: bad tensor list");
-    std::vector<value::Value> fields;
-    for (int32_t i = 0; i < list_len; ++i)
-      fields.push_back(FromDesc(&tensor_list[i], "tensor_list"));
-    value::Value tuple = value::MakeTuple(fields);
+    value::Value tuple = ListTuple(env, list_len, tensor_list, "tensor_list");
     std::vector<value::Value> inputs = {tuple, FromDesc(step, "step")};
     OpEnv::SetStreamForAllBackends(env->call->device, stream);
     WorkspaceBinding bind(env->env.get(), workspace, workspace_bytes);
@@ -270,10 +298,7 @@ int rafhip_raf_sgd_multi_execute(rafhip_raf_env* env, int32_t list_len,
     if (!env || !env->env) throw Error("rafhip_raf_sgd_multi_execute: env is NULL");
     if (list_len < 0 || (list_len > 0 && !tensor_list))
       throw Error("rafhip_raf_sgd_multi_execute: bad tensor list");
-    std::vector<value::Value> fields;
-    for (int32_t i = 0; i < list_len; ++i)
-      fields.push_back(FromDesc(&tensor_list[i], "tensor_list"));
-    value::Value tuple = value::MakeTuple(fields);
+    value::Value tuple = ListTuple(env, list_len, tensor_list, "tensor_list");
     std::vector<value::Value> inputs = {tuple};
     OpEnv::SetStreamForAllBackends(env->call->device, stream);
     WorkspaceBinding bind(env->env.get(), nullptr, 0);
@@ -607,6 +632,36 @@ int rafhip_raf_env_set_learning_rate(rafhip_raf_env* env, double learning_rate) 
     auto* target = dynamic_cast<hip::HasLearningRate*>(env->env.get());
     if (!target) throw Error("rafhip_raf_env_set_learning_rate: " + env->name + " has no learning rate");
     target->SetLearningRate(learning_rate);
+  });
+}
+
+int rafhip_raf_env_set_grad_unscale(rafhip_raf_env* env, float factor) {
+  return Guard([&] {
+    if (!env) throw Error("rafhip_raf_env_set_grad_unscale: env is NULL");
+    if (!env->env) return;  // declared as a no-op
+    auto* target = dynamic_cast<hip::HasGradScaling*>(env->env.get());
+    if (!target) throw Error("rafhip_raf_env_set_grad_unscale: " + env->name + " takes no gradient scale");
+    target->SetGradUnscale(factor);
+  });
+}
+
+int rafhip_raf_env_set_dynamic_scale(rafhip_raf_env* env, const rafhip_tensor_desc* grad_unscale,
+                                     const rafhip_tensor_desc* found_inf) {
+  return Guard([&] {
+    if (!env) throw Error("rafhip_raf_env_set_dynamic_scale: env is NULL");
+    if (!env->env) return;  // declared as a no-op
+    auto* target = dynamic_cast<hip::HasGradScaling*>(env->env.get());
+    if (!target) throw Error("rafhip_raf_env_set_dynamic_scale: " + env->name + " takes no gradient scale");
+    auto word = [&](const rafhip_tensor_desc* d, const char* what) -> const float* {
+      if (!d) return nullptr;
+      const TensorView t = FromDesc(d, what)->tensor;
+      if (t.dtype.code != kDLFloat || t.dtype.bits != 32 || t.numel() != 1)
+        throw Error(std::string(what) + " must be a one-element float32 tensor");
+      if (t.device.device_type() != DevType::kROCM() || t.device.device_id() != env->call->device.device_id())
+        throw Error(std::string(what) + " must live on the OpEnv's device");
+      return static_cast<const float*>(t.data);
+    };
+    target->SetDynamicScale(word(grad_unscale, "grad_unscale"), word(found_inf, "found_inf"));
   });
 }
 

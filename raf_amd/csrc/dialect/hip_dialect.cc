@@ -16,7 +16,6 @@
 // arguments are reported through error_msgs so dispatch can fall through to another dialect.
 #include "hip_dialect.h"
 
-#include <atomic>
 #include <sstream>
 
 #include "raf_iface.h"
@@ -33,8 +32,6 @@ using value::Value;
 
 namespace {
 
-std::atomic<float> g_lans_grad_unscale{1.0f};  // set by one thread, read by makers on any thread
-
 std::string KernelError(const char* what, int status) {
   std::ostringstream ss;
   ss << what << " failed with status " << status << ": " << rafhip_last_error();
@@ -49,9 +46,6 @@ int32_t KernelDType(const DType& t) {
 }
 
 }  // namespace
-
-void SetLansGradUnscale(float factor) { g_lans_grad_unscale.store(factor, std::memory_order_relaxed); }
-float GetLansGradUnscale() { return g_lans_grad_unscale.load(std::memory_order_relaxed); }
 
 // ----------------------------------------------------------------------------------------- SGD
 class SgdHipEnv : public OpEnv, public HasLearningRate {
@@ -223,7 +217,7 @@ class SgdMultiHipEnv : public OpEnv, public HasLearningRate {
 // new weights narrowed to 16 bits -- what the reference's traced optimizer does with a cast and a
 // copy after the op, python/raf/optim/lans.py:289-291, :303-305).  Half gradients are accepted by
 // both and widened in the kernel, replacing the group_cast in front of the op (lans.py:261-265).
-class LansHipEnv : public OpEnv, public HasLearningRate {
+class LansHipEnv : public OpEnv, public HasLearningRate, public HasGradScaling {
  public:
   LansHipEnv(const CallValues& cv, bool mixed)
       : blocks_(mixed ? 5 : 4),
@@ -245,7 +239,7 @@ class LansHipEnv : public OpEnv, public HasLearningRate {
     hp_.grad_averaging = args->grad_averaging;
     hp_.mode = args->mode;
     hp_.normalize_grad = args->normalize_grad ? 1 : 0;
-    hp_.grad_unscale = GetLansGradUnscale();
+    hp_.grad_unscale = 1.0f;  // see HasGradScaling
 
     const size_t total = args->tensor_list.size();
     if (total % (size_t)blocks_ != 0) {  // lans.cc:53
@@ -325,22 +319,36 @@ class LansHipEnv : public OpEnv, public HasLearningRate {
     RAF_CHECK(IsF32(step.dtype), "step must be float32");
     RAF_CHECK(workspace_ != nullptr || workspace_bytes_ == 0,
               "raf.op.hip.lans: the executor did not provide the requested workspace");
-    std::vector<void*> ptrs(tuple->fields.size());
-    for (size_t i = 0; i < ptrs.size(); ++i) ptrs[i] = AsTensor(tuple->fields[i])->tensor.data;
-    void** p = ptrs.data();
+    // An executor that hands over the very same tuple object again (a loop over fixed storage)
+    // finds the plan already bound to its tensors: no walk over the 4n or 5n fields, no table
+    // to compare or send.  Any other tuple is walked and bound afresh.  Only a weak reference is
+    // kept, so the OpEnv never prolongs the life of a caller's tensors.
+    if (bound_tuple_.expired() || bound_tuple_.lock() != tuple) {
+      ptrs_.resize(tuple->fields.size());
+      for (size_t i = 0; i < ptrs_.size(); ++i) ptrs_[i] = AsTensor(tuple->fields[i])->tensor.data;
+      void** p = ptrs_.data();
+      int st = rafhip_lans_plan_bind(plan_, reinterpret_cast<const void* const*>(p),
+                                     reinterpret_cast<float* const*>(p + n_),
+                                     reinterpret_cast<float* const*>(p + 2 * n_),
+                                     reinterpret_cast<float* const*>(p + 3 * n_),
+                                     blocks_ == 5 ? p + 4 * n_ : nullptr, copy_dtype_);
+      if (st != RAFHIP_OK) throw Error(KernelError("rafhip_lans_plan_bind", st));
+      bound_tuple_ = tuple;
+    }
     void* stream = DeviceAPI::Get(DevType::kROCM())->GetStream();
-    int st = rafhip_lans_step_mixed(plan_, reinterpret_cast<const void* const*>(p),
-                                    reinterpret_cast<float* const*>(p + n_),
-                                    reinterpret_cast<float* const*>(p + 2 * n_),
-                                    reinterpret_cast<float* const*>(p + 3 * n_),
-                                    blocks_ == 5 ? p + 4 * n_ : nullptr, copy_dtype_,
-                                    static_cast<const float*>(step.data), 0, &hp_, workspace_,
+    int st = rafhip_lans_step_bound(plan_, static_cast<const float*>(step.data), 0, &hp_, workspace_,
                                     workspace_bytes_, stream);
-    if (st != RAFHIP_OK) throw Error(KernelError("rafhip_lans_step_mixed", st));
+    if (st != RAFHIP_OK) throw Error(KernelError("rafhip_lans_step_bound", st));
   }
 
   void SetLearningRate(double learning_rate) override { hp_.learning_rate = (float)learning_rate; }
   double GetLearningRate() const override { return hp_.learning_rate; }
+
+  void SetGradUnscale(float factor) override { hp_.grad_unscale = factor; }
+  void SetDynamicScale(const float* grad_unscale_dev, const float* found_inf_dev) override {
+    int st = rafhip_lans_plan_set_dynamic_scale(plan_, grad_unscale_dev, found_inf_dev);
+    if (st != RAFHIP_OK) throw Error(KernelError("rafhip_lans_plan_set_dynamic_scale", st));
+  }
 
   static OpEnv* make(const CallValues& cv) { return new LansHipEnv(cv, false); }
   static OpEnv* make_mixed(const CallValues& cv) { return new LansHipEnv(cv, true); }
@@ -355,6 +363,8 @@ class LansHipEnv : public OpEnv, public HasLearningRate {
   rafhip_lans_plan* plan_ = nullptr;
   void* workspace_ = nullptr;  // bound by the executor around each Execute
   int64_t workspace_bytes_ = 0;
+  std::weak_ptr<value::TupleValueObj> bound_tuple_;  // the tuple whose tensors the plan is bound to
+  std::vector<void*> ptrs_;
 };
 
 // -------------------------------------------------------------------------------------- l2norm

@@ -9,11 +9,20 @@ namespace raf {
 namespace op {
 namespace hip {
 
-// Factor every LANS gradient is multiplied by before use (undoing a loss scale, e.g. 1/1024 for
-// fp16 gradients).  Captured when a LANS OpEnv is made; 1 by default.  The reference's LansArgs
-// has no such field: there, gradients are cast and unscaled by separate ops before LANS runs.
-void SetLansGradUnscale(float factor);
-float GetLansGradUnscale();
+// Loss scaling.  The reference's LansArgs has no field for it: there, gradients are cast and
+// unscaled by separate ops before LANS runs.  The hip LANS OpEnvs fold the unscaling into the
+// kernels and implement this interface, through which the executor that owns the OpEnv sets,
+// between two Execute calls,
+//   - the factor every gradient element is multiplied by first (e.g. 1/1024; 1 by default), or
+//   - for dynamic loss scaling, device pointers to that factor and to an overflow flag (fp32 words
+//     read by the kernels: a non-zero flag makes the step a no-op), either of which may be null.
+// Neither is part of what identifies the OpEnv, so a scale change keeps the OpEnv and its plan.
+class HasGradScaling {
+ public:
+  virtual ~HasGradScaling() = default;
+  virtual void SetGradUnscale(float factor) = 0;
+  virtual void SetDynamicScale(const float* grad_unscale_dev, const float* found_inf_dev) = 0;
+};
 
 // A learning-rate schedule changes one hyper-parameter every step.  The reference's schemas carry
 // the learning rate as a constant, so there every new value means a new OpEnv (the VM's cache key

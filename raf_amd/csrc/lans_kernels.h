@@ -147,7 +147,9 @@ struct LansDeviceArgs {
   const WorkItem* pipeline_items;
   uint32_t spin_limit;    // pipelined: bound of every wait, in polls
   uint32_t* host_error;   // pipelined: pinned host word raised together with sync->error, or nullptr
-  float unscale;
+  float unscale;          // every gradient element is multiplied by this first (loss-scale undo) ...
+  const float* unscale_dev;    // ... or, when not null, by the fp32 value this device pointer holds
+  const float* found_inf_dev;  // optional: a non-zero fp32 value here turns the whole step into a no-op
   int32_t p_is_bf16;      // dtype of the optional 16-bit weight copies: 0 binary16, 1 bfloat16
   StepScalars* scalars;
   TensorStats* stats;

@@ -7,6 +7,11 @@
 #include "half_types.h"
 #include "rafhip_optim.h"
 
+// No implicit contraction of a*b+c: where a fused multiply-add is wanted it is written as
+// __builtin_fma.  The same source line then gives the same bits in every kernel it is inlined
+// into, which the bit-equality of the two schedules (and of all grid sizes) relies on.
+#pragma clang fp contract(off)
+
 namespace rafhip {
 namespace {
 
@@ -45,19 +50,23 @@ __device__ __forceinline__ double wave_sum(double x) {
   return x;
 }
 
-// Block-wide sums of N values, returned to every thread.  `red` is [3][kLansWaves] doubles of
-// LDS.  The leading barrier makes the helper safe to call repeatedly on the same LDS.
-template <int N>
-__device__ __forceinline__ void block_sum(double (&x)[N], double (*red)[kLansWaves]) {
-  static_assert(N <= 3, "red holds three rows");
+// Block-wide sums of N values, returned to every thread.  `red` is [4][kLansWaves] doubles of
+// LDS.  The leading barrier makes the helper safe to call repeatedly on the same LDS.  With kFlag
+// it also tells every thread whether `flag` was set in any thread, through the same two barriers.
+template <int N, bool kFlag = false>
+__device__ __forceinline__ bool block_sum(double (&x)[N], double (*red)[kLansWaves], bool flag = false) {
+  static_assert(N <= 3, "red holds three rows of sums and one of flags");
 #pragma unroll
   for (int j = 0; j < N; ++j) x[j] = wave_sum(x[j]);
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
+  bool wave_flag = false;
+  if constexpr (kFlag) wave_flag = __any(flag ? 1 : 0) != 0;
   __syncthreads();
   if (lane == 0) {
 #pragma unroll
     for (int j = 0; j < N; ++j) red[j][wave] = x[j];
+    if constexpr (kFlag) red[3][wave] = wave_flag ? 1.0 : 0.0;
   }
   __syncthreads();
 #pragma unroll
@@ -67,6 +76,13 @@ __device__ __forceinline__ void block_sum(double (&x)[N], double (*red)[kLansWav
     for (int k = 1; k < kLansWaves; ++k) s += red[j][k];
     x[j] = s;
   }
+  if constexpr (kFlag) {
+    bool any = false;
+#pragma unroll
+    for (int k = 0; k < kLansWaves; ++k) any = any || red[3][k] != 0.0;
+    return any;
+  }
+  return false;
 }
 
 // Loads/stores that are coherent across the whole device (they go past the per-XCD L2), used for
@@ -82,6 +98,13 @@ __device__ __forceinline__ void st_dev(double* p, double v) {
 }
 
 constexpr uint64_t kNotReady = 0xFFFFFFFFFFFFFFFFull;
+// What is published in place of a value that could not be computed because a wait ran out: also a
+// NaN pattern that no computation produces.  Whoever consumes it passes it on, and pass C skips
+// the stores of an element whose parameters are lost, so that a step that ran out of a wait leaves
+// every element either at its old or at its correct new value, never at garbage.
+constexpr uint64_t kLost = 0xFFFFFFFFFFFFFFFEull;
+__device__ __forceinline__ double lost_value() { return __longlong_as_double((long long)kLost); }
+__device__ __forceinline__ bool is_lost(double v) { return (uint64_t)__double_as_longlong(v) == kLost; }
 
 __device__ __forceinline__ uint64_t ld_bits(const double* p) {
   return __hip_atomic_load(reinterpret_cast<const uint64_t*>(p), __ATOMIC_RELAXED,
@@ -93,7 +116,7 @@ __device__ __forceinline__ uint64_t ld_bits(const double* p) {
 // NaN pattern no computation produces, because published values are canonicalised), each is
 // written exactly once per step with a single 8-byte store, and a consumer re-reads a word until
 // it differs.  No ordering between words is needed.  A wait that runs out raises the error word
-// and returns whatever is there, so the grid always drains.
+// and returns the "lost" pattern, so the grid always drains.
 __device__ __forceinline__ void publish(double* p, double v) {
   st_dev(p, v != v ? __builtin_nan("") : v);
 }
@@ -104,14 +127,23 @@ struct WaitCtx {
   uint32_t* error;       // set to 1 when a wait runs out
   uint32_t limit;        // polls a wait may take
   uint32_t* host_error;  // the same flag in pinned host memory, which the host can read without a copy
+  bool gave_up = false;  // this thread has seen a wait run out: its later waits do not poll at all
 };
-__device__ __forceinline__ double wait_published(const double* word, const WaitCtx& wc) {
+__device__ __forceinline__ double wait_published(const double* word, WaitCtx& wc) {
   uint64_t bits = ld_bits(word);
   uint32_t spins = 0;
   while (bits == kNotReady) {
-    if (++spins > wc.limit) {
-      __hip_atomic_store(wc.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (wc.host_error) __hip_atomic_store(wc.host_error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    if (wc.gave_up || ++spins > wc.limit) {
+      // The step is lost.  Raise the error word and make it visible before anything this thread
+      // publishes afterwards, so that whoever consumes such a value also finds the word raised
+      // (pass C then leaves the tensors as they were).  The fence is expensive, and only here.
+      if (!wc.gave_up) {
+        __hip_atomic_store(wc.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (wc.host_error) __hip_atomic_store(wc.host_error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        wc.gave_up = true;
+      }
+      bits = kLost;
       break;
     }
     __builtin_amdgcn_s_sleep(8);
@@ -124,7 +156,7 @@ __device__ __forceinline__ double wait_published(const double* word, const WaitC
 // read again.
 template <int N>
 __device__ __forceinline__ void wait_published_n(const double* const (&words)[N], double (&out)[N],
-                                                 const WaitCtx& wc) {
+                                                 WaitCtx& wc) {
   uint64_t bits[N];
 #pragma unroll
   for (int j = 0; j < N; ++j) bits[j] = ld_bits(words[j]);
@@ -139,9 +171,10 @@ __device__ __forceinline__ void wait_published_n(const double* const (&words)[N]
 // depends on nothing but the unit count.  A unit is chunks_per_unit chunks (pass A: kChunksPerA)
 // and keeps its partial in its first chunk's slot.  With kWait the partials are awaited.
 template <int N, bool kWait>
-__device__ __forceinline__ void tensor_totals(const double* partials, int slot, int64_t n_units,
+__device__ __forceinline__ bool tensor_totals(const double* partials, int slot, int64_t n_units,
                                               int chunks_per_unit, double (&tot)[N],
-                                              double (*red)[kLansWaves], const WaitCtx& wc) {
+                                              double (*red)[kLansWaves], WaitCtx& wc) {
+  bool lost = false;  // kWait only: a partial is lost, or this thread ran out of a wait
   if (n_units == 1) {
     // One unit: the total is that partial (0 + x, as the tree below would form it), which every
     // thread can read for itself -- no trip through LDS and two barriers for the many one-chunk
@@ -152,13 +185,15 @@ __device__ __forceinline__ void tensor_totals(const double* partials, int slot, 
 #pragma unroll
       for (int j = 0; j < N; ++j) words[j] = p + j;
       wait_published_n<N>(words, tot, wc);
+#pragma unroll
+      for (int j = 0; j < N; ++j) lost = lost || is_lost(tot[j]);
     } else {
 #pragma unroll
       for (int j = 0; j < N; ++j) tot[j] = ld_dev(p + j);
     }
 #pragma unroll
     for (int j = 0; j < N; ++j) tot[j] = 0.0 + tot[j];
-    return;
+    return lost;  // each thread's own view; the publishing thread acts on its own
   }
 #pragma unroll
   for (int j = 0; j < N; ++j) tot[j] = 0.0;
@@ -171,13 +206,16 @@ __device__ __forceinline__ void tensor_totals(const double* partials, int slot, 
       for (int j = 0; j < N; ++j) words[j] = p + j;
       wait_published_n<N>(words, val, wc);
 #pragma unroll
-      for (int j = 0; j < N; ++j) tot[j] += val[j];
+      for (int j = 0; j < N; ++j) {
+        lost = lost || is_lost(val[j]);
+        tot[j] += val[j];
+      }
     } else {
 #pragma unroll
       for (int j = 0; j < N; ++j) tot[j] += ld_dev(p + j);
     }
   }
-  block_sum<N>(tot, red);
+  return block_sum<N, kWait>(tot, red, lost);
 }
 
 // ------------------------------------------------------------------ the rule, per element
@@ -274,17 +312,17 @@ __device__ __forceinline__ double chunk_sum_g(const ChunkView& cv, float unscale
 #pragma unroll
       for (int u = 0; u < kU; ++u)
 #pragma unroll
-        for (int j = 0; j < kW; ++j) acc[j & 3] += (double)x[u][j] * (double)x[u][j];
+        for (int j = 0; j < kW; ++j) acc[j & 3] = __builtin_fma((double)x[u][j], (double)x[u][j], acc[j & 3]);
     }
     const int tail = nw * kW + threadIdx.x;  // the < kW leftover elements of a last chunk
     if (tail < cv.len) {
       const double gx = GradIO<G>::load1(cv.g, tail, unscale);
-      acc[0] += gx * gx;
+      acc[0] = __builtin_fma(gx, gx, acc[0]);
     }
   } else {
     for (int i = threadIdx.x; i < cv.len; i += kLansBlock) {
       const double gx = GradIO<G>::load1(cv.g, i, unscale);
-      acc[0] += gx * gx;
+      acc[0] = __builtin_fma(gx, gx, acc[0]);
     }
   }
   return (acc[0] + acc[1]) + (acc[2] + acc[3]);
@@ -341,6 +379,11 @@ __device__ __forceinline__ void for_each_trip(const ChunkView& cv, int n4, Pre&&
   }
 }
 
+// a^2 + b^2 + c^2 + d^2 as two chains of one product and one fused multiply-add each.
+__device__ __forceinline__ double sum_sq4(double a, double b, double c, double d) {
+  return __builtin_fma(b, b, a * a) + __builtin_fma(d, d, c * c);
+}
+
 // One trip's contribution to a lane's sums of u_m^2, u_g^2 and w^2 (pass B).
 template <typename G>
 __device__ __forceinline__ void sums_of_trip(const Batch<G>& cur, int i0, int n4, float unscale,
@@ -354,10 +397,9 @@ __device__ __forceinline__ void sums_of_trip(const Batch<G>& cur, int i0, int n4
       const Directions d1 = lans_directions(g.y, cur.w[u].y, cur.m[u].y, cur.v[u].y, inv_gdiv, k);
       const Directions d2 = lans_directions(g.z, cur.w[u].z, cur.m[u].z, cur.v[u].z, inv_gdiv, k);
       const Directions d3 = lans_directions(g.w, cur.w[u].w, cur.m[u].w, cur.v[u].w, inv_gdiv, k);
-      am += (d0.um * d0.um + d1.um * d1.um) + (d2.um * d2.um + d3.um * d3.um);
-      au += (d0.ug * d0.ug + d1.ug * d1.ug) + (d2.ug * d2.ug + d3.ug * d3.ug);
-      aw += ((double)cur.w[u].x * (double)cur.w[u].x + (double)cur.w[u].y * (double)cur.w[u].y) +
-            ((double)cur.w[u].z * (double)cur.w[u].z + (double)cur.w[u].w * (double)cur.w[u].w);
+      am += sum_sq4(d0.um, d1.um, d2.um, d3.um);
+      au += sum_sq4(d0.ug, d1.ug, d2.ug, d3.ug);
+      aw += sum_sq4((double)cur.w[u].x, (double)cur.w[u].y, (double)cur.w[u].z, (double)cur.w[u].w);
     }
   }
 }
@@ -385,9 +427,9 @@ __device__ __forceinline__ void chunk_sums_u(const ChunkView& cv, float unscale,
       const Directions d = lans_directions(GradIO<G>::load1(cv.g, tail, unscale), wx,
                                            ((gc_float*)cv.m)[tail], ((gc_float*)cv.v)[tail],
                                            inv_gdiv, k);
-      am += d.um * d.um;
-      au += d.ug * d.ug;
-      aw += wx * wx;
+      am = __builtin_fma(d.um, d.um, am);
+      au = __builtin_fma(d.ug, d.ug, au);
+      aw = __builtin_fma(wx, wx, aw);
     }
   } else {
     const double inv_gdiv = get_inv_gdiv();
@@ -395,9 +437,9 @@ __device__ __forceinline__ void chunk_sums_u(const ChunkView& cv, float unscale,
       const double wx = ((gc_float*)cv.w)[i];
       const Directions d = lans_directions(GradIO<G>::load1(cv.g, i, unscale), wx,
                                            ((gc_float*)cv.m)[i], ((gc_float*)cv.v)[i], inv_gdiv, k);
-      am += d.um * d.um;
-      au += d.ug * d.ug;
-      aw += wx * wx;
+      am = __builtin_fma(d.um, d.um, am);
+      au = __builtin_fma(d.ug, d.ug, au);
+      aw = __builtin_fma(wx, wx, aw);
     }
   }
   sums[0] = am;
@@ -412,6 +454,7 @@ struct Applied {
 
 struct ApplyParams {
   double inv_gdiv, rm, rg;
+  bool valid = true;  // false: a wait ran out somewhere upstream; this thread stores nothing
 };
 
 __device__ __forceinline__ Applied apply_one(double g, double w, double m, double v,
@@ -460,10 +503,10 @@ __device__ __forceinline__ void chunk_apply(const ChunkView& cv, float unscale, 
     ApplyParams p{1.0, 0.0, 0.0};
     for_each_trip<G, kGradNT, kNT, kAhead>(cv, n4, [&] { p = get_params(); },
                                            [&](const Batch<G>& cur, int i0) {
-      apply_trip<G, kStoreNT>(cur, i0, n4, cv, unscale, p_is_bf16, p, k);
+      if (p.valid) apply_trip<G, kStoreNT>(cur, i0, n4, cv, unscale, p_is_bf16, p, k);
     });
     const int tail = (n4 << 2) + threadIdx.x;
-    if (tail < cv.len) {
+    if (tail < cv.len && p.valid) {
       const Applied o = apply_one(GradIO<G>::load1(cv.g, tail, unscale), ((gc_float*)cv.w)[tail],
                                   ((gc_float*)cv.m)[tail], ((gc_float*)cv.v)[tail], p, k);
       ((g_float*)cv.w)[tail] = o.w;
@@ -473,7 +516,7 @@ __device__ __forceinline__ void chunk_apply(const ChunkView& cv, float unscale, 
     }
   } else {
     const ApplyParams p = get_params();
-    for (int i = threadIdx.x; i < cv.len; i += kLansBlock) {
+    for (int i = threadIdx.x; p.valid && i < cv.len; i += kLansBlock) {
       const Applied o = apply_one(GradIO<G>::load1(cv.g, i, unscale), ((gc_float*)cv.w)[i],
                                   ((gc_float*)cv.m)[i], ((gc_float*)cv.v)[i], p, k);
       ((g_float*)cv.w)[i] = o.w;
@@ -525,6 +568,19 @@ __device__ __forceinline__ void stats_after_b(TensorStats* st, const double (&to
   publish(&st->ratio_g, ratio_g);
 }
 
+// In place of stats_after_a / stats_after_b when the totals could not be formed.
+__device__ __forceinline__ void stats_lost_after_a(TensorStats* st) {
+  st_dev(&st->grad_norm, lost_value());
+  st_dev(&st->inv_grad_div, lost_value());
+}
+__device__ __forceinline__ void stats_lost_after_b(TensorStats* st) {
+  st_dev(&st->param_norm, lost_value());
+  st_dev(&st->um_norm, lost_value());
+  st_dev(&st->ug_norm, lost_value());
+  st_dev(&st->ratio_m, lost_value());
+  st_dev(&st->ratio_g, lost_value());
+}
+
 __device__ __forceinline__ int64_t chunks_of(const TensorRec& tr) {
   return (tr.numel + ((int64_t)1 << tr.chunk_shift) - 1) >> tr.chunk_shift;
 }
@@ -562,6 +618,18 @@ __device__ __forceinline__ void write_step_scalars(const LansDeviceArgs& a, cons
   *a.scalars = k;
 }
 
+// Dynamic loss scaling.  The factor every gradient element is multiplied by first comes from the
+// plan's hyper-parameters or, when the caller gave one, from an fp32 word in device memory (the
+// reciprocal of the current loss scale); a non-zero `found_inf` word makes the whole step a no-op:
+// every kernel of the step returns at once and w, m, v (and the 16-bit copies) keep their bits.
+// Both words are read when a kernel starts, so the host never has to know their values.
+__device__ __forceinline__ float grad_unscale_of(const LansDeviceArgs& a) {
+  return a.unscale_dev ? *a.unscale_dev : a.unscale;
+}
+__device__ __forceinline__ bool step_is_skipped(const LansDeviceArgs& a) {
+  return a.found_inf_dev != nullptr && *a.found_inf_dev != 0.0f;
+}
+
 // ------------------------------------------------------------------ set-up launch
 // Set-up of a pipelined step: the step scalars, and every word the schedule waits on (chunk
 // partials, per-tensor statistics) marked as not ready.  The phased schedule waits on nothing and
@@ -590,7 +658,9 @@ template <typename G, int kMode>
 __global__ __launch_bounds__(kLansBlock) void lans_norm_g(LansDeviceArgs a, const float* step_dev,
                                                           int32_t step_host, HParamsPod hp) {
   constexpr CachePolicy kP = kMode == kModeStreaming ? kPhasedPolicy : kResidentPolicy;
-  __shared__ double red[3][kLansWaves];
+  __shared__ double red[4][kLansWaves];
+  if (step_is_skipped(a)) return;
+  const float unscale = grad_unscale_of(a);
   // This pass needs no scalars; the later launches find them written by the first workgroup.
   if (blockIdx.x == 0 && threadIdx.x == 0) write_step_scalars(a, step_dev, step_host, hp);
   for (int64_t i = blockIdx.x; i < a.n_items_a; i += gridDim.x) {
@@ -598,7 +668,7 @@ __global__ __launch_bounds__(kLansBlock) void lans_norm_g(LansDeviceArgs a, cons
     const TensorRec tr = a.tensors[it.tensor];
     const uint32_t unit = it.chunk_phase & kChunkMask;
     const ChunkView cv = chunk_view(tr, unit, (int)sizeof(G), kChunksPerA);
-    double s[1] = {chunk_sum_g<G, kP.a_g>(cv, a.unscale)};
+    double s[1] = {chunk_sum_g<G, kP.a_g>(cv, unscale)};
     block_sum<1>(s, red);
     if (threadIdx.x == 0)
       publish(&a.partials[kPartialSlots * ((int64_t)tr.first_chunk + (int64_t)unit * kChunksPerA)], s[0]);
@@ -607,18 +677,20 @@ __global__ __launch_bounds__(kLansBlock) void lans_norm_g(LansDeviceArgs a, cons
 
 // One workgroup per tensor.
 __global__ __launch_bounds__(kLansBlock) void lans_finish(LansDeviceArgs a, int after_b) {
-  __shared__ double red[3][kLansWaves];
+  __shared__ double red[4][kLansWaves];
+  if (step_is_skipped(a)) return;
+  WaitCtx no_wait{nullptr, 0, nullptr};
   const int t = blockIdx.x;
   const TensorRec tr = a.tensors[t];
   const double* part = a.partials + kPartialSlots * (int64_t)tr.first_chunk;
   const StepScalars k = *a.scalars;
   if (after_b) {
     double tot[3], r0, r1;
-    tensor_totals<3, false>(part, 1, chunks_of(tr), 1, tot, red, WaitCtx{nullptr, 0, nullptr});
+    tensor_totals<3, false>(part, 1, chunks_of(tr), 1, tot, red, no_wait);
     if (threadIdx.x == 0) stats_after_b(&a.stats[t], tot, k, r0, r1);
   } else {
     double tot[1];
-    tensor_totals<1, false>(part, 0, units_a_of(tr), kChunksPerA, tot, red, WaitCtx{nullptr, 0, nullptr});
+    tensor_totals<1, false>(part, 0, units_a_of(tr), kChunksPerA, tot, red, no_wait);
     if (threadIdx.x == 0) stats_after_a(&a.stats[t], tot[0], k);
   }
 }
@@ -626,7 +698,10 @@ __global__ __launch_bounds__(kLansBlock) void lans_finish(LansDeviceArgs a, int 
 template <typename G, int kMode>
 __global__ __launch_bounds__(kLansBlock) void lans_norm_u(LansDeviceArgs a) {
   constexpr CachePolicy kP = kMode == kModeStreaming ? kPhasedPolicy : kResidentPolicy;
-  __shared__ double red[3][kLansWaves];
+  __shared__ double red[4][kLansWaves];
+  if (step_is_skipped(a)) return;
+  const float unscale = grad_unscale_of(a);
+  WaitCtx no_wait{nullptr, 0, nullptr};
   const StepScalars k = *a.scalars;
   // Back to front: pass A has just streamed the gradients front to back, so the end of the list is
   // what the Infinity Cache still holds; pass C then starts at the front, where this pass ends.
@@ -640,7 +715,7 @@ __global__ __launch_bounds__(kLansBlock) void lans_norm_u(LansDeviceArgs a) {
     if constexpr (kMode == kModeResidentInline) {
       double tot[1];
       tensor_totals<1, false>(a.partials + kPartialSlots * (int64_t)tr.first_chunk, 0, units_a_of(tr),
-                              kChunksPerA, tot, red, WaitCtx{nullptr, 0, nullptr});
+                              kChunksPerA, tot, red, no_wait);
       if (chunk == 0 && threadIdx.x == 0)  // one workgroup per tensor leaves the statistics
         inv_gdiv = stats_after_a(&a.stats[it.tensor], tot[0], k);
       else
@@ -649,7 +724,7 @@ __global__ __launch_bounds__(kLansBlock) void lans_norm_u(LansDeviceArgs a) {
       inv_gdiv = a.stats[it.tensor].inv_grad_div;
     }
     double s[3];
-    chunk_sums_u<G, kP.b_g, kP.b_wmv>(cv, a.unscale, k, [&] { return inv_gdiv; }, s);
+    chunk_sums_u<G, kP.b_g, kP.b_wmv>(cv, unscale, k, [&] { return inv_gdiv; }, s);
     block_sum<3>(s, red);
     if (threadIdx.x == 0) {
       publish(&a.partials[kPartialSlots * c + 1], s[0]);
@@ -662,7 +737,10 @@ __global__ __launch_bounds__(kLansBlock) void lans_norm_u(LansDeviceArgs a) {
 template <typename G, int kMode>
 __global__ __launch_bounds__(kLansBlock) void lans_apply(LansDeviceArgs a) {
   constexpr CachePolicy kP = kMode == kModeStreaming ? kPhasedPolicy : kResidentPolicy;
-  __shared__ double red[3][kLansWaves];
+  __shared__ double red[4][kLansWaves];
+  if (step_is_skipped(a)) return;
+  const float unscale = grad_unscale_of(a);
+  WaitCtx no_wait{nullptr, 0, nullptr};
   const StepScalars k = *a.scalars;
   for (int64_t c = blockIdx.x; c < a.n_chunks; c += gridDim.x) {
     const WorkItem it = a.items[c];
@@ -673,7 +751,7 @@ __global__ __launch_bounds__(kLansBlock) void lans_apply(LansDeviceArgs a) {
     if constexpr (kMode == kModeResidentInline) {
       double tot[3];
       tensor_totals<3, false>(a.partials + kPartialSlots * (int64_t)tr.first_chunk, 1, chunks_of(tr), 1,
-                              tot, red, WaitCtx{nullptr, 0, nullptr});
+                              tot, red, no_wait);
       p.inv_gdiv = a.stats[it.tensor].inv_grad_div;  // left by pass B
       if (chunk == 0 && threadIdx.x == 0)
         stats_after_b(&a.stats[it.tensor], tot, k, p.rm, p.rg);
@@ -683,18 +761,20 @@ __global__ __launch_bounds__(kLansBlock) void lans_apply(LansDeviceArgs a) {
       const TensorStats st = a.stats[it.tensor];
       p = ApplyParams{st.inv_grad_div, st.ratio_m, st.ratio_g};
     }
-    chunk_apply<G, kP.c_g, kP.c_wmv, kP.c_stores>(cv, a.unscale, a.p_is_bf16 != 0, k, [&] { return p; });
+    chunk_apply<G, kP.c_g, kP.c_wmv, kP.c_stores>(cv, unscale, a.p_is_bf16 != 0, k, [&] { return p; });
   }
 }
 
 // ------------------------------------------------------------------ pipelined schedule
 template <typename G>
 __global__ __launch_bounds__(kLansBlock) void lans_pipelined(LansDeviceArgs a) {
-  __shared__ double red[3][kLansWaves];
+  __shared__ double red[4][kLansWaves];
   __shared__ double s_bcast[3];
   __shared__ uint32_t s_ticket;
+  if (step_is_skipped(a)) return;
+  const float unscale = grad_unscale_of(a);
   const StepScalars k = *a.scalars;
-  const WaitCtx wc{&a.sync->error, a.spin_limit, a.host_error};
+  WaitCtx wc{&a.sync->error, a.spin_limit, a.host_error};
 
   // Thread 0 draws tickets two items ahead, so an atomic's round trip is hidden behind a whole
   // item, and every thread reads the NEXT item's descriptor and tensor record while the current
@@ -740,51 +820,71 @@ __global__ __launch_bounds__(kLansBlock) void lans_pipelined(LansDeviceArgs a) {
     TensorStats* st = &a.stats[t];
 
     if (phase == kPhaseA) {
-      double s[1] = {chunk_sum_g<G, kPipelinedPolicy.a_g>(cv, a.unscale)};
+      double s[1] = {chunk_sum_g<G, kPipelinedPolicy.a_g>(cv, unscale)};
       block_sum<1>(s, red);
       if (threadIdx.x == 0) publish(part, s[0]);
     } else if (phase == kPhaseFinishA) {
       double tot[1];
-      tensor_totals<1, true>(tensor_part, 0, units_a_of(tr), kChunksPerA, tot, red, wc);
-      if (threadIdx.x == 0) stats_after_a(st, tot[0], k);
+      const bool lost = tensor_totals<1, true>(tensor_part, 0, units_a_of(tr), kChunksPerA, tot, red, wc);
+      if (threadIdx.x == 0) {
+        if (lost)
+          stats_lost_after_a(st);
+        else
+          stats_after_a(st, tot[0], k);
+      }
     } else if (phase == kPhaseB) {
       double s[3];
-      chunk_sums_u<G, kPipelinedPolicy.b_g, kPipelinedPolicy.b_wmv, kPipelinedAhead>(cv, a.unscale, k,
-                      [&] { return wait_published(&st->inv_grad_div, wc); }, s);
-      block_sum<3>(s, red);
+      bool lost = false;  // this thread's divisor never arrived
+      chunk_sums_u<G, kPipelinedPolicy.b_g, kPipelinedPolicy.b_wmv, kPipelinedAhead>(cv, unscale, k, [&] {
+        const double d = wait_published(&st->inv_grad_div, wc);
+        lost = is_lost(d);
+        return d;
+      }, s);
+      const bool any_lost = block_sum<3, true>(s, red, lost);
       if (threadIdx.x == 0) {
-        publish(part + 1, s[0]);
-        publish(part + 2, s[1]);
-        publish(part + 3, s[2]);
+        if (any_lost) {
+          st_dev(part + 1, lost_value());
+          st_dev(part + 2, lost_value());
+          st_dev(part + 3, lost_value());
+        } else {
+          publish(part + 1, s[0]);
+          publish(part + 2, s[1]);
+          publish(part + 3, s[2]);
+        }
       }
     } else if (phase == kPhaseFinishB) {
       double tot[3], r0, r1;
-      tensor_totals<3, true>(tensor_part, 1, n_chunks, 1, tot, red, wc);
-      if (threadIdx.x == 0) stats_after_b(st, tot, k, r0, r1);
+      const bool lost = tensor_totals<3, true>(tensor_part, 1, n_chunks, 1, tot, red, wc);
+      if (threadIdx.x == 0) {
+        if (lost)
+          stats_lost_after_b(st);
+        else
+          stats_after_b(st, tot, k, r0, r1);
+      }
     } else if (phase == kPhaseC) {
       chunk_apply<G, kPipelinedPolicy.c_g, kPipelinedPolicy.c_wmv, kPipelinedPolicy.c_stores, kPipelinedAhead>(
-          cv, a.unscale, a.p_is_bf16 != 0, k, [&] {
+          cv, unscale, a.p_is_bf16 != 0, k, [&] {
         const double* const words[3] = {&st->inv_grad_div, &st->ratio_m, &st->ratio_g};
         double val[3];
         wait_published_n<3>(words, val, wc);
-        return ApplyParams{val[0], val[1], val[2]};
+        return ApplyParams{val[0], val[1], val[2], !(is_lost(val[0]) || is_lost(val[1]) || is_lost(val[2]))};
       });
     } else {
       // A one-chunk tensor: all three passes here, no other workgroup involved.  The totals equal
       // the single chunk partials, exactly as the general path computes them, and travel between
       // the threads through LDS.
-      double s1[1] = {chunk_sum_g<G, false>(cv, a.unscale)};
+      double s1[1] = {chunk_sum_g<G, false>(cv, unscale)};
       block_sum<1>(s1, red);
       if (threadIdx.x == 0) s_bcast[0] = stats_after_a(st, s1[0], k);
       __syncthreads();
       const double inv_gdiv = s_bcast[0];
       double s3[3];
-      chunk_sums_u<G, false, false>(cv, a.unscale, k, [&] { return inv_gdiv; }, s3);
+      chunk_sums_u<G, false, false>(cv, unscale, k, [&] { return inv_gdiv; }, s3);
       block_sum<3>(s3, red);
       if (threadIdx.x == 0) stats_after_b(st, s3, k, s_bcast[1], s_bcast[2]);
       __syncthreads();
       const ApplyParams p{inv_gdiv, s_bcast[1], s_bcast[2]};
-      chunk_apply<G, false, false, true>(cv, a.unscale, a.p_is_bf16 != 0, k, [&] { return p; });
+      chunk_apply<G, false, false, true>(cv, unscale, a.p_is_bf16 != 0, k, [&] { return p; });
     }
     if (a.trace && threadIdx.x == 0) {  // diagnostics: when the item was started and finished
       uint64_t* rec = a.trace + 4 * (uint64_t)ticket;

@@ -221,6 +221,14 @@ struct rafhip_lans_plan {
 
   RecordUploader<TensorRec> tensors;  // a step whose pointers did not move sends nothing
   std::vector<TensorRec> recs;        // this call's records, built in place: a step allocates nothing
+  // rafhip_lans_plan_bind: records of tensors that stay where they are, built and checked once.
+  std::vector<TensorRec> bound;
+  bool bound_valid = false;
+  bool bound_on_device = false;  // the device table holds `bound` (no other step intervened)
+  int32_t bound_p_dtype = RAFHIP_F16;
+  // rafhip_lans_plan_set_dynamic_scale: optional device words read by every kernel of a step.
+  const float* unscale_dev = nullptr;
+  const float* found_inf_dev = nullptr;
 
   // This device's address of the static scratch array (rafhip_lans_step_noalloc), resolved when the
   // plan is made; nullptr with the reason in static_scratch_error if that failed.
@@ -372,6 +380,7 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
       p->n_cus = cus;
     p->static_scratch = static_scratch_of(p->device, &p->static_scratch_error);
     p->recs.resize((size_t)n_tensors);
+    p->bound.resize((size_t)n_tensors);
 
     if (n_tensors > 0) {
       std::vector<WorkItem> phased((size_t)chunks);
@@ -511,123 +520,213 @@ int rafhip_lans_step_noalloc(rafhip_lans_plan* plan, const void* const* g, float
 
 namespace {
 
+constexpr uintptr_t kWorkspaceAlign = 16;  // what the kernels' 8- and 16-byte accesses need
+
+// Checks that are the same for every kind of step; *nothing_to_do is set for an empty list.
+int check_step_args(const char* who, rafhip_lans_plan* plan, const rafhip_lans_hparams* hp,
+                    bool* nothing_to_do) {
+  *nothing_to_do = false;
+  if (!hp) return fail(RAFHIP_ERR_INVALID_ARG, "%s: hparams is NULL", who);
+  if (hp->mode != 0 && hp->mode != 1)
+    return fail(RAFHIP_ERR_INVALID_ARG, "%s: mode = %d (0 = L2, 1 = decoupled)", who, hp->mode);
+  if (plan->n_tensors == 0 || plan->n_chunks == 0) {
+    *nothing_to_do = true;
+    return RAFHIP_OK;
+  }
+  if (int st = check_plan_device(who, plan->device)) return st;
+  if (plan->host_error && __atomic_load_n(plan->host_error, __ATOMIC_RELAXED) != 0) {
+    // Raised by the persistent kernel of an earlier step; reported once, then the plan works on.
+    __atomic_store_n(plan->host_error, 0u, __ATOMIC_RELAXED);
+    return fail(RAFHIP_ERR_HIP,
+                "%s: an earlier pipelined step on this plan ran out of a bounded wait; its results are "
+                "invalid (this call did nothing)",
+                who);
+  }
+  return RAFHIP_OK;
+}
+
+// The tensor table of a call, built into `recs` (already n long: no allocation); 4-byte (fp16 g:
+// 2-byte) alignment is the hard requirement, 16-byte alignment of all four selects the vector path.
+int build_records(const char* who, const rafhip_lans_plan* plan, const void* const* g,
+                  float* const* w, float* const* m, float* const* v, void* const* p, int32_t p_dtype,
+                  std::vector<TensorRec>& recs) {
+  if (p && p_dtype != RAFHIP_F16 && p_dtype != RAFHIP_BF16)
+    return fail(RAFHIP_ERR_UNSUPPORTED, "%s: weight-copy dtype %d (binary16 or bfloat16)", who, p_dtype);
+  if (!g || !w || !m || !v) return fail(RAFHIP_ERR_INVALID_ARG, "%s: null pointer list", who);
+  const int32_t n = plan->n_tensors;
+  const uintptr_t g_elem = plan->grad_dtype == RAFHIP_F32 ? 4 : 2;
+  const uintptr_t g_vec = 16;  // pass A reads the gradient with 16-byte lane accesses
+  recs.resize((size_t)n);
+  for (int32_t t = 0; t < n; ++t) {
+    TensorRec& r = recs[t];
+    r.g = g[t];
+    r.w = w[t];
+    r.m = m[t];
+    r.v = v[t];
+    r.p = p ? p[t] : nullptr;
+    r.numel = plan->numel[t];
+    r.first_chunk = plan->first_chunk[t];
+    r.vec_ok = 0;
+    r.chunk_shift = chunk_shift_for(r.numel);
+    r.reserved = 0;
+    if (r.numel == 0) continue;
+    if (!r.g || !r.w || !r.m || !r.v)
+      return fail(RAFHIP_ERR_INVALID_ARG, "%s: tensor %d has a null data pointer", who, t);
+    if (!aligned_to(r.g, g_elem) || !aligned_to(r.w, 4) || !aligned_to(r.m, 4) ||
+        !aligned_to(r.v, 4) || !aligned_to(r.p, 2))
+      return fail(RAFHIP_ERR_INVALID_ARG, "%s: tensor %d is not element-aligned", who, t);
+    r.vec_ok = aligned_to(r.g, g_vec) && aligned_to(r.w, 16) && aligned_to(r.m, 16) &&
+               aligned_to(r.v, 16) && aligned_to(r.p, 8);
+  }
+  return RAFHIP_OK;
+}
+
+// Enqueues the kernels of one step on `s`; the device tensor table is up to date for that stream.
+int launch_step(const char* who, rafhip_lans_plan* plan, int32_t p_dtype, const float* step_dev,
+                int32_t step_host, const rafhip_lans_hparams* hp, void* workspace,
+                int64_t workspace_bytes, hipStream_t s) {
+  (void)who;
+  char* ws = static_cast<char*>(workspace);
+  LansDeviceArgs a;
+  a.tensors = plan->d_tensors;
+  a.n_tensors = plan->n_tensors;
+  a.items = plan->d_items;
+  a.n_chunks = plan->n_chunks;
+  a.items_a = plan->d_items_a;
+  a.n_items_a = plan->n_items_a;
+  a.n_items = plan->n_pipeline_items;
+  a.pipeline_items = plan->d_pipeline;
+  a.unscale = hp->grad_unscale;
+  a.unscale_dev = plan->unscale_dev;
+  a.found_inf_dev = plan->found_inf_dev;
+  a.spin_limit = plan->spin_limit;
+  a.host_error = plan->host_error_dev;
+  a.p_is_bf16 = p_dtype == RAFHIP_BF16 ? 1 : 0;
+  a.scalars = reinterpret_cast<StepScalars*>(ws + plan->ws.scalars_off);
+  a.stats = reinterpret_cast<TensorStats*>(ws + plan->ws.stats_off);
+  a.partials = reinterpret_cast<double*>(ws + plan->ws.partials_off);
+  a.sync = reinterpret_cast<SyncHeader*>(ws + plan->ws.sync_off);
+  a.trace = plan->d_trace;
+
+  HParamsPod pod;
+  pod.learning_rate = hp->learning_rate;
+  pod.beta1 = hp->beta1;
+  pod.beta2 = hp->beta2;
+  pod.eps = hp->eps;
+  pod.weight_decay = hp->weight_decay;
+  pod.bias_correction = hp->bias_correction;
+  pod.grad_averaging = hp->grad_averaging;
+  pod.mode = hp->mode;
+  pod.normalize_grad = hp->normalize_grad ? 1 : 0;
+
+  hipEvent_t* marks = nullptr;
+  if (!plan->timing.empty())
+    marks = plan->timing[plan->steps_done % (int64_t)plan->timing.size()].data();
+
+  if (plan->schedule == RAFHIP_LANS_PIPELINED) {
+    if (marks) RAFHIP_HIP_TRY(hipEventRecord(marks[0], s));
+    launch_prepare(s, a, step_dev, step_host, pod);
+    if (marks) RAFHIP_HIP_TRY(hipEventRecord(marks[1], s));
+    launch_pipelined(plan->grad_dtype, plan->pipeline_grid, s, a);
+    if (marks)
+      for (int i = 2; i < 6; ++i) RAFHIP_HIP_TRY(hipEventRecord(marks[i], s));
+  } else {
+    const int64_t bytes_per_elt = plan->grad_dtype == RAFHIP_F32 ? 16 : 14;
+    launch_phased(plan->grad_dtype, plan->total_elements * bytes_per_elt > kResidentBytes,
+                  plan->short_tensors_only, s, a, step_dev, step_host, pod, marks);
+  }
+  RAFHIP_HIP_TRY(hipGetLastError());
+  plan->steps_done++;
+  return RAFHIP_OK;
+}
+
+int check_workspace(const char* who, const rafhip_lans_plan* plan, const void* workspace,
+                    int64_t workspace_bytes) {
+  if (!workspace || workspace_bytes < plan->ws.total)
+    return fail(RAFHIP_ERR_WORKSPACE, "%s: workspace %p of %lld bytes, need %lld", who, workspace,
+                (long long)workspace_bytes, (long long)plan->ws.total);
+  if (!aligned_to(workspace, kWorkspaceAlign))
+    return fail(RAFHIP_ERR_WORKSPACE, "%s: workspace %p is not %d-byte aligned", who, workspace,
+                (int)kWorkspaceAlign);
+  return RAFHIP_OK;
+}
+
 // The step behind rafhip_lans_step, _mixed and _noalloc.  Allocates neither device nor host memory.
 int lans_step_impl(rafhip_lans_plan* plan, const void* const* g, float* const* w, float* const* m,
                    float* const* v, void* const* p, int32_t p_dtype, const float* step_dev,
                    int32_t step_host, const rafhip_lans_hparams* hp, void* workspace,
                    int64_t workspace_bytes, void* stream) {
-  if (p && p_dtype != RAFHIP_F16 && p_dtype != RAFHIP_BF16)
-    return fail(RAFHIP_ERR_UNSUPPORTED,
-                "rafhip_lans_step: weight-copy dtype %d (binary16 or bfloat16)", p_dtype);
-  if (!hp) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_step: hparams is NULL");
-  if (hp->mode != 0 && hp->mode != 1)
-    return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_step: mode = %d (0 = L2, 1 = decoupled)",
-                hp->mode);
-  const int32_t n = plan->n_tensors;
-  if (n == 0 || plan->n_chunks == 0) return RAFHIP_OK;  // nothing to update
-  if (int st = check_plan_device("rafhip_lans_step", plan->device)) return st;
-  if (plan->host_error && __atomic_load_n(plan->host_error, __ATOMIC_RELAXED) != 0) {
-    // Raised by the persistent kernel of an earlier step; reported once, then the plan works on.
-    __atomic_store_n(plan->host_error, 0u, __ATOMIC_RELAXED);
-    return fail(RAFHIP_ERR_HIP,
-                "rafhip_lans_step: an earlier pipelined step on this plan ran out of a bounded wait; "
-                "its results are invalid (this call did nothing)");
-  }
-  if (!g || !w || !m || !v)
-    return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_step: null pointer list");
-  return guarded("rafhip_lans_step", [&]() -> int {
-    if (!workspace || workspace_bytes < plan->ws.total)
-      return fail(RAFHIP_ERR_WORKSPACE, "rafhip_lans_step: workspace %p of %lld bytes, need %lld",
-                  workspace, (long long)workspace_bytes, (long long)plan->ws.total);
-    if (!aligned_to(workspace, kAlign))
-      return fail(RAFHIP_ERR_WORKSPACE, "rafhip_lans_step: workspace %p is not 256-byte aligned",
-                  workspace);
-
-    // Build this call's tensor table; 4-byte (fp16 g: 2-byte) alignment is the hard requirement,
-    // 16-byte alignment of all four selects the vector path.
-    const uintptr_t g_elem = plan->grad_dtype == RAFHIP_F32 ? 4 : 2;
-    const uintptr_t g_vec = 16;  // pass A reads the gradient with 16-byte lane accesses
-    std::vector<TensorRec>& recs = plan->recs;
-    recs.resize((size_t)n);  // its size already: no allocation
-    for (int32_t t = 0; t < n; ++t) {
-      TensorRec& r = recs[t];
-      r.g = g[t];
-      r.w = w[t];
-      r.m = m[t];
-      r.v = v[t];
-      r.p = p ? p[t] : nullptr;
-      r.numel = plan->numel[t];
-      r.first_chunk = plan->first_chunk[t];
-      r.vec_ok = 0;
-      r.chunk_shift = chunk_shift_for(r.numel);
-      r.reserved = 0;
-      if (r.numel == 0) continue;
-      if (!r.g || !r.w || !r.m || !r.v)
-        return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_step: tensor %d has a null data pointer", t);
-      if (!aligned_to(r.g, g_elem) || !aligned_to(r.w, 4) || !aligned_to(r.m, 4) ||
-          !aligned_to(r.v, 4) || !aligned_to(r.p, 2))
-        return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_step: tensor %d is not element-aligned", t);
-      r.vec_ok = aligned_to(r.g, g_vec) && aligned_to(r.w, 16) && aligned_to(r.m, 16) &&
-                 aligned_to(r.v, 16) && aligned_to(r.p, 8);
-    }
-
+  const char* who = "rafhip_lans_step";
+  bool nothing = false;
+  if (int st = check_step_args(who, plan, hp, &nothing)) return st;
+  if (nothing) return RAFHIP_OK;
+  return guarded(who, [&]() -> int {
+    if (int st = check_workspace(who, plan, workspace, workspace_bytes)) return st;
+    if (int st = build_records(who, plan, g, w, m, v, p, p_dtype, plan->recs)) return st;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    RAFHIP_HIP_TRY(plan->tensors.sync(recs, s));
-
-    char* ws = static_cast<char*>(workspace);
-    LansDeviceArgs a;
-    a.tensors = plan->d_tensors;
-    a.n_tensors = n;
-    a.items = plan->d_items;
-    a.n_chunks = plan->n_chunks;
-    a.items_a = plan->d_items_a;
-    a.n_items_a = plan->n_items_a;
-    a.n_items = plan->n_pipeline_items;
-    a.pipeline_items = plan->d_pipeline;
-    a.unscale = hp->grad_unscale;
-    a.spin_limit = plan->spin_limit;
-    a.host_error = plan->host_error_dev;
-    a.p_is_bf16 = p_dtype == RAFHIP_BF16 ? 1 : 0;
-    a.scalars = reinterpret_cast<StepScalars*>(ws + plan->ws.scalars_off);
-    a.stats = reinterpret_cast<TensorStats*>(ws + plan->ws.stats_off);
-    a.partials = reinterpret_cast<double*>(ws + plan->ws.partials_off);
-    a.sync = reinterpret_cast<SyncHeader*>(ws + plan->ws.sync_off);
-    a.trace = plan->d_trace;
-
-    HParamsPod pod;
-    pod.learning_rate = hp->learning_rate;
-    pod.beta1 = hp->beta1;
-    pod.beta2 = hp->beta2;
-    pod.eps = hp->eps;
-    pod.weight_decay = hp->weight_decay;
-    pod.bias_correction = hp->bias_correction;
-    pod.grad_averaging = hp->grad_averaging;
-    pod.mode = hp->mode;
-    pod.normalize_grad = hp->normalize_grad ? 1 : 0;
-
-    hipEvent_t* marks = nullptr;
-    if (!plan->timing.empty())
-      marks = plan->timing[plan->steps_done % (int64_t)plan->timing.size()].data();
-
-    if (plan->schedule == RAFHIP_LANS_PIPELINED) {
-      if (marks) RAFHIP_HIP_TRY(hipEventRecord(marks[0], s));
-      launch_prepare(s, a, step_dev, step_host, pod);
-      if (marks) RAFHIP_HIP_TRY(hipEventRecord(marks[1], s));
-      launch_pipelined(plan->grad_dtype, plan->pipeline_grid, s, a);
-      if (marks)
-        for (int i = 2; i < 6; ++i) RAFHIP_HIP_TRY(hipEventRecord(marks[i], s));
-    } else {
-      const int64_t bytes_per_elt = plan->grad_dtype == RAFHIP_F32 ? 16 : 14;
-      launch_phased(plan->grad_dtype, plan->total_elements * bytes_per_elt > kResidentBytes,
-                    plan->short_tensors_only, s, a, step_dev, step_host, pod, marks);
-    }
-    RAFHIP_HIP_TRY(hipGetLastError());
-    plan->steps_done++;
-    return RAFHIP_OK;
+    RAFHIP_HIP_TRY(plan->tensors.sync(plan->recs, s));
+    plan->bound_on_device = false;  // whatever was bound, the device table now follows this call
+    return launch_step(who, plan, p_dtype, step_dev, step_host, hp, workspace, workspace_bytes, s);
   });
 }
 
 }  // namespace
+
+extern "C" {
+
+int rafhip_lans_plan_bind(rafhip_lans_plan* plan, const void* const* g, float* const* w,
+                          float* const* m, float* const* v, void* const* p, int32_t p_dtype) {
+  clear_error();
+  const char* who = "rafhip_lans_plan_bind";
+  if (!plan) return fail(RAFHIP_ERR_INVALID_ARG, "%s: plan is NULL", who);
+  return guarded(who, [&]() -> int {
+    plan->bound_valid = false;
+    if (int st = build_records(who, plan, g, w, m, v, p, p_dtype, plan->bound)) return st;
+    plan->bound_p_dtype = p ? p_dtype : RAFHIP_F16;
+    plan->bound_valid = true;
+    plan->bound_on_device = false;
+    return RAFHIP_OK;
+  });
+}
+
+int rafhip_lans_step_bound(rafhip_lans_plan* plan, const float* step_dev, int32_t step_host,
+                           const rafhip_lans_hparams* hp, void* workspace, int64_t workspace_bytes,
+                           void* stream) {
+  clear_error();
+  const char* who = "rafhip_lans_step_bound";
+  if (!plan) return fail(RAFHIP_ERR_INVALID_ARG, "%s: plan is NULL", who);
+  bool nothing = false;
+  if (int st = check_step_args(who, plan, hp, &nothing)) return st;
+  if (nothing) return RAFHIP_OK;
+  if (!plan->bound_valid)
+    return fail(RAFHIP_ERR_INVALID_ARG, "%s: no tensors are bound (rafhip_lans_plan_bind first)", who);
+  return guarded(who, [&]() -> int {
+    if (int st = check_workspace(who, plan, workspace, workspace_bytes)) return st;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (plan->bound_on_device) {
+      RAFHIP_HIP_TRY(plan->tensors.follow(s));  // nothing to build, compare or send
+    } else {
+      plan->recs = plan->bound;  // same size: a copy, no allocation
+      RAFHIP_HIP_TRY(plan->tensors.sync(plan->recs, s));
+      plan->bound_on_device = true;
+    }
+    return launch_step(who, plan, plan->bound_p_dtype, step_dev, step_host, hp, workspace,
+                       workspace_bytes, s);
+  });
+}
+
+int rafhip_lans_plan_set_dynamic_scale(rafhip_lans_plan* plan, const float* grad_unscale_dev,
+                                       const float* found_inf_dev) {
+  clear_error();
+  if (!plan) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_plan_set_dynamic_scale: plan is NULL");
+  if (!aligned_to(grad_unscale_dev, 4) || !aligned_to(found_inf_dev, 4))
+    return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_plan_set_dynamic_scale: pointers must be 4-byte aligned");
+  plan->unscale_dev = grad_unscale_dev;
+  plan->found_inf_dev = found_inf_dev;
+  return RAFHIP_OK;
+}
+
+}  // extern "C"
 
 extern "C" {
 

@@ -327,20 +327,33 @@ class LansPlan:
                                                 ctypes.byref(hp), _current_stream(self.device)))
 
     def bind(self, g, w, m, v, hp: LansHParams, workspace: Optional[torch.Tensor] = None, p=None):
-        """Marshal the pointer lists once for tensors that stay where they are; ``step_bound`` then
-        costs one foreign call per step (a training loop updates the same buffers every step)."""
+        """``rafhip_lans_plan_bind``: check the pointer lists and build the tensor table once for
+        tensors that stay where they are; ``step_bound`` then costs one foreign call per step that
+        touches no list (a training loop updates the same buffers every step)."""
         ws = self.workspace if workspace is None else workspace
         pp, p_code = self._model_ptrs(p)
-        self._bound = (self._ptrs(g, self.grad_dtype, "g"), self._ptrs(w, torch.float32, "w"),
-                       self._ptrs(m, torch.float32, "m"), self._ptrs(v, torch.float32, "v"),
-                       pp, p_code, hp, ws, (list(g), list(w), list(m), list(v), p))
+        check(self.lib.rafhip_lans_plan_bind(self._h, self._ptrs(g, self.grad_dtype, "g"),
+                                             self._ptrs(w, torch.float32, "w"), self._ptrs(m, torch.float32, "m"),
+                                             self._ptrs(v, torch.float32, "v"), pp, p_code))
+        self._bound = (hp, ws, (list(g), list(w), list(m), list(v), p))
 
     def step_bound(self, step: torch.Tensor):
         """One step on the tensors given to ``bind``; ``step`` is the 0-d fp32 GPU step tensor."""
-        gp, wp, mp, vp, pp, p_code, hp, ws, _ = self._bound
-        check(self.lib.rafhip_lans_step_mixed(self._h, gp, wp, mp, vp, pp, p_code, step.data_ptr(), 0,
-                                              ctypes.byref(hp), ws.data_ptr(), ws.numel(),
-                                              _current_stream(self.device)))
+        hp, ws, _ = self._bound
+        check(self.lib.rafhip_lans_step_bound(self._h, step.data_ptr(), 0, ctypes.byref(hp), ws.data_ptr(),
+                                              ws.numel(), _current_stream(self.device)))
+
+    def set_dynamic_scale(self, grad_unscale: Optional[torch.Tensor] = None,
+                          found_inf: Optional[torch.Tensor] = None):
+        """``rafhip_lans_plan_set_dynamic_scale``: 0-d fp32 GPU tensors holding the reciprocal of the
+        loss scale and the overflow flag (non-zero: the step does nothing), read by the kernels."""
+        for t, name in ((grad_unscale, "grad_unscale"), (found_inf, "found_inf")):
+            if t is not None and (t.dtype != torch.float32 or t.numel() != 1 or not t.is_cuda):
+                raise TypeError(f"{name} must be a one-element float32 GPU tensor")
+        self._dynamic = (grad_unscale, found_inf)  # keep them alive
+        check(self.lib.rafhip_lans_plan_set_dynamic_scale(
+            self._h, grad_unscale.data_ptr() if grad_unscale is not None else None,
+            found_inf.data_ptr() if found_inf is not None else None))
 
     def read_norms(self, workspace: Optional[torch.Tensor] = None):
         """[n, 4] float64: ||g||, ||w||, ||u_m||, ||u_g|| of the last step."""

@@ -63,6 +63,8 @@ class _Env:
         self.workspace_bytes = lib.rafhip_raf_env_workspace_bytes(handle)
         self.workspaces = {}  # stream handle -> runtime.Memory
         self.learning_rate = None  # what the OpEnv was made with or last told, if it has one
+        self.grad_unscale = 1.0
+        self.dynamic_scale = (None, None)  # the tensors the OpEnv was last told to read
 
     def set_learning_rate(self, learning_rate: float) -> None:
         """A learning-rate schedule keeps its OpEnv: the hip optimizer OpEnvs take a new value between
@@ -70,6 +72,17 @@ class _Env:
         if learning_rate != self.learning_rate:
             check_raf(_lib.dialect().rafhip_raf_env_set_learning_rate(self.handle, learning_rate))
             self.learning_rate = learning_rate
+
+    def set_grad_scaling(self, factor: float, dynamic) -> None:
+        """Loss scaling is no part of what identifies an OpEnv either (hip-dialect extension)."""
+        if factor != self.grad_unscale:
+            check_raf(_lib.dialect().rafhip_raf_env_set_grad_unscale(self.handle, factor))
+            self.grad_unscale = factor
+        if dynamic[0] is not self.dynamic_scale[0] or dynamic[1] is not self.dynamic_scale[1]:
+            keep: list = []
+            descs = [ctypes.byref(_desc(t, keep)) if t is not None else None for t in dynamic]
+            check_raf(_lib.dialect().rafhip_raf_env_set_dynamic_scale(self.handle, *descs))
+            self.dynamic_scale = tuple(dynamic)
 
     def __del__(self):
         try:
@@ -119,6 +132,7 @@ _env_cache = _EnvCache()
 def clear_op_env_cache() -> None:
     _env_cache.clear()
     _marshalled.clear()
+    _slots.clear()
 
 
 class _Marshalled:
@@ -130,6 +144,7 @@ class _Marshalled:
         self.sig = tuple(_sig(t) for t in tensors)
         self.refs = [weakref.ref(t) for t in tensors]
         self.ptrs = [t.data_ptr() for t in tensors]
+        self.slot = 0
 
     def still_describes(self, tensors) -> bool:
         # the same live objects (a weak reference cannot be fooled by a recycled id) at the same
@@ -138,17 +153,26 @@ class _Marshalled:
 
 
 _marshalled: Dict[Tuple, _Marshalled] = {}
+_SLOTS_PER_SIGNATURE = 4
+_slots: Dict[Tuple, list] = {}  # signature -> identities (id tuples) of the lists seen, by slot
 
 
 def _marshal_list(tensors: list) -> _Marshalled:
     """Marshalling a list of hundreds of tensors costs milliseconds of Python; a training loop passes
-    the same tensors every step, so the last marshalling of every distinct list is kept."""
+    the same tensors every step, so the last marshalling of every distinct list is kept.  Lists of
+    equal signature get different ``slot`` numbers (up to a few; beyond that they share the last)."""
     key = tuple(map(id, tensors))
     m = _marshalled.get(key)
     if m is None or not m.still_describes(tensors):
         if len(_marshalled) >= 8:
             _marshalled.clear()
         m = _marshalled[key] = _Marshalled(tensors)
+        known = _slots.setdefault(m.sig, [])
+        if key not in known:
+            if len(known) >= _SLOTS_PER_SIGNATURE:
+                known.pop()
+            known.append(key)
+        m.slot = known.index(key)
     return m
 
 
@@ -255,7 +279,7 @@ def _sgd_multi(mixed, tensor_list, learning_rate, mu):
     n = len(tensor_list)
     m = _marshal_list(tensor_list)
     descs = m.descs
-    key = ("sgd_multi", mixed, m.sig, float(mu))
+    key = ("sgd_multi", mixed, m.sig, m.slot, float(mu))
     env = _env_cache.get(key)
     if env is None:
         h = c_void_p(None)
@@ -300,7 +324,10 @@ def _lans(op_name, tensor_list, step, learning_rate, beta1, beta2, eps, bias_cor
     dstep = _desc(step, keep)
     hp = (float(learning_rate), float(beta1), float(beta2), float(eps), int(bias_correction),
           float(weight_decay), int(grad_averaging), int(mode), int(bool(normalize_grad)))
-    key = (op_name, m.sig, _sig(step), hp[1:], get_lans_grad_unscale())  # all but the learning rate
+    # All but the learning rate and the loss scaling.  `m.slot` tells lists of equal signature
+    # apart (two models of one architecture): each keeps an OpEnv, and with it a plan whose device
+    # pointer table follows that list alone.
+    key = (op_name, m.sig, m.slot, _sig(step), hp[1:])
     env = _env_cache.get(key)
     if env is None:
         h = c_void_p(None)
@@ -310,6 +337,7 @@ def _lans(op_name, tensor_list, step, learning_rate, beta1, beta2, eps, bias_cor
         env.learning_rate = hp[0]
     if n4:
         env.set_learning_rate(hp[0])
+        env.set_grad_scaling(_lans_grad_unscale, _lans_dynamic_scale)
     stream = _stream(tensor_list[0]) if n4 else None
     ws = _workspace(env, tensor_list[0], stream) if env.workspace_bytes > 0 else None
     check_raf(lib.rafhip_raf_lans_execute(env.handle, n4, descs, dstep, ws.data if ws else None,
@@ -397,18 +425,32 @@ def defuse_tensor(data: torch.Tensor, sizes, shapes, shape_indices):
 
 
 _lans_grad_unscale = 1.0
+_lans_dynamic_scale = (None, None)
 
 
 def set_lans_grad_unscale(factor: float) -> None:
     """hip-dialect extension: LANS multiplies every gradient by ``factor`` first (e.g. 1/1024 to
-    undo a loss scale on fp16 gradients).  Applies to LANS OpEnvs made afterwards."""
+    undo a loss scale on fp16 gradients).  Applies to every LANS call from now on; OpEnvs are kept."""
     global _lans_grad_unscale
-    check_raf(_lib.dialect().rafhip_raf_set_lans_grad_unscale(float(factor)))
     _lans_grad_unscale = float(factor)
 
 
 def get_lans_grad_unscale() -> float:
     return _lans_grad_unscale
+
+
+def set_lans_dynamic_scale(grad_unscale: torch.Tensor = None, found_inf: torch.Tensor = None) -> None:
+    """hip-dialect extension for dynamic loss scaling: 0-d float32 GPU tensors holding the
+    reciprocal of the current loss scale (it replaces the static factor) and the overflow flag (a
+    non-zero value makes the LANS step a no-op).  The kernels read both on the device, so the scale
+    can change and a step can be skipped without a host synchronisation or a new OpEnv.  ``None``
+    switches either off."""
+    global _lans_dynamic_scale
+    for t, name in ((grad_unscale, "grad_unscale"), (found_inf, "found_inf")):
+        if t is not None and (not isinstance(t, torch.Tensor) or t.dtype != torch.float32 or t.numel() != 1
+                              or not t.is_cuda):
+            raise TypeError(f"{name} must be a one-element float32 GPU tensor")
+    _lans_dynamic_scale = (grad_unscale, found_inf)
 
 
 def dispatch_list(base_op: str, device_type: int = DEV_ROCM) -> List[Tuple[str, str, int]]:

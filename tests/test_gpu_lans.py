@@ -508,3 +508,162 @@ def test_two_persistent_kernels_side_by_side(native_libs):
         _assert_norms(plan.read_norms(), on)
         _assert_close([t.cpu().numpy() for t in tw], ow, TOL_1, "w")
         plan.close()
+
+
+def test_a_step_that_runs_out_of_a_wait_leaves_old_or_new_values(native_libs, monkeypatch):
+    """Whatever consumes a value that never arrived passes a 'lost' marker on instead of computing
+    with it, and the third pass skips the stores of an element whose parameters are lost: after a
+    step that reported a time-out every element of w, m and v holds either its old value or the
+    value a good step gives it -- all three of one element from the same side -- never garbage."""
+    from raf_amd import kernels
+
+    sizes = [1 << 22, 3 << 20, 70001, 5000, 1 << 21]
+    g, w, m, v = lans_inputs(sizes, cfg=93)
+    hp = LansHParams()
+    tg, tw, tm, tv = _to_dev(g), _to_dev(w), _to_dev(m), _to_dev(v)
+    plan = kernels.LansPlan(sizes, torch.float32, DEV)
+    plan.set_schedule("pipelined")
+    plan.step(tg, tw, tm, tv, 2, _khp(hp))
+    torch.cuda.synchronize()
+    plan.read_norms()  # a good step: no report
+    plan.close()
+    new = [[t.cpu().numpy() for t in ts] for ts in (tw, tm, tv)]
+
+    monkeypatch.setenv("RAFHIP_LANS_SPIN_LIMIT", "0")
+    tg, tw, tm, tv = _to_dev(g), _to_dev(w), _to_dev(m), _to_dev(v)
+    plan = kernels.LansPlan(sizes, torch.float32, DEV)
+    plan.set_schedule("pipelined")
+    plan.step(tg, tw, tm, tv, 2, _khp(hp))
+    torch.cuda.synchronize()
+    monkeypatch.delenv("RAFHIP_LANS_SPIN_LIMIT")
+    with pytest.raises(native_libs.RafHipError, match="bounded wait"):
+        plan.read_norms()
+    plan.close()
+    got = [[t.cpu().numpy() for t in ts] for ts in (tw, tm, tv)]
+    old = [w, m, v]
+    for t in range(len(sizes)):
+        is_new = [got[q][t].view(np.uint32) == new[q][t].view(np.uint32) for q in range(3)]
+        is_old = [got[q][t].view(np.uint32) == old[q][t].view(np.uint32) for q in range(3)]
+        for q in range(3):
+            assert np.all(is_new[q] | is_old[q]), f"tensor {t}, array {'wmv'[q]}: a value that is neither old nor new"
+        # an element is updated as a whole or not at all (where old and new differ, which they do
+        # for m and v of every element with a non-zero gradient)
+        updated = is_new[1] & ~is_old[1]
+        kept = is_old[1] & ~is_new[1]
+        assert not np.any(updated & ~is_new[0]) and not np.any(updated & ~is_new[2])
+        assert not np.any(kept & ~is_old[0]) and not np.any(kept & ~is_old[2])
+
+
+def test_workspace_needs_only_16_byte_alignment(native_libs):
+    """RAF's memory pools hand out blocks aligned to 64 bytes (include/raf/memory_pool.h), not 256:
+    a workspace at such an address must be accepted and give the same bits."""
+    from raf_amd import kernels
+
+    sizes = [70001, 300000, 9]
+    g, w, m, v = lans_inputs(sizes, cfg=94)
+    outs = []
+    for offset in (0, 64, 16):
+        tg, tw, tm, tv = _to_dev(g), _to_dev(w), _to_dev(m), _to_dev(v)
+        plan = kernels.LansPlan(sizes, torch.float32, DEV)
+        for schedule in ("phased", "pipelined"):
+            plan.set_schedule(schedule)
+            block = torch.empty(plan.workspace_bytes + 256, dtype=torch.uint8, device=DEV)
+            ws = block[offset:offset + plan.workspace_bytes]
+            assert ws.data_ptr() % 256 == offset
+            plan.step(tg, tw, tm, tv, 1 if schedule == "phased" else 2, _khp(LansHParams()), workspace=ws)
+        torch.cuda.synchronize()
+        outs.append([t.cpu().numpy() for t in tw + tm + tv])
+        plan.close()
+    for other in outs[1:]:
+        assert all(np.array_equal(a, b) for a, b in zip(outs[0], other))
+    tg, tw, tm, tv = _to_dev(g), _to_dev(w), _to_dev(m), _to_dev(v)
+    plan = kernels.LansPlan(sizes, torch.float32, DEV)
+    block = torch.empty(plan.workspace_bytes + 256, dtype=torch.uint8, device=DEV)
+    with pytest.raises(native_libs.RafHipError, match="16-byte aligned"):
+        plan.step(tg, tw, tm, tv, 1, _khp(LansHParams()), workspace=block[8:8 + plan.workspace_bytes])
+    plan.close()
+
+
+@pytest.mark.parametrize("schedule", ["phased", "pipelined"])
+def test_bound_form_equals_the_unbound_step(native_libs, schedule):
+    """rafhip_lans_plan_bind + rafhip_lans_step_bound: same bits as rafhip_lans_step_mixed, over
+    several steps, after binding other tensors, and with unbound steps on the same plan in between."""
+    from raf_amd import kernels
+
+    sizes = [70001, 5, 8192, 300000, 1, 0]
+    hp = _khp(LansHParams())
+    ga, wa, ma, va = lans_inputs(sizes, cfg=95)
+    gb, wb, mb, vb = lans_inputs(sizes, cfg=96)
+
+    def run(bound):
+        A = [_to_dev(x) for x in (ga, wa, ma, va)]
+        B = [_to_dev(x) for x in (gb, wb, mb, vb)]
+        plan = kernels.LansPlan(sizes, torch.float32, DEV)
+        plan.set_schedule(schedule)
+        step = torch.zeros((), device=DEV)
+
+        def do(lst, rebind):
+            step.add_(1.0)
+            if bound:
+                if rebind:
+                    plan.bind(*lst, hp)
+                plan.step_bound(step)
+            else:
+                plan.step(*lst, step, hp)
+
+        do(A, True)
+        do(A, False)
+        do(B, True)
+        do(B, False)
+        step.add_(1.0)
+        plan.step(*A, step, hp)  # an unbound step takes the device table away from the bound tensors ...
+        do(B, False)             # ... and the next bound step brings it back
+        torch.cuda.synchronize()
+        plan.close()
+        return [t.cpu().numpy() for lst in (A, B) for ts in lst[1:] for t in ts]
+
+    for a, b in zip(run(False), run(True)):
+        assert np.array_equal(a, b)
+
+
+def test_bound_step_without_binding_is_an_error(native_libs):
+    from raf_amd import _lib, kernels
+    import ctypes
+
+    plan = kernels.LansPlan([100], torch.float32, DEV)
+    hp = _khp(LansHParams())
+    st = plan.lib.rafhip_lans_step_bound(plan._h, None, 1, ctypes.byref(hp), plan.workspace.data_ptr(),
+                                         plan.workspace.numel(), None)
+    assert st == _lib.RAFHIP_ERR_INVALID_ARG and "rafhip_lans_plan_bind" in _lib.last_error()
+    plan.close()
+
+
+def test_two_lists_alternating_on_two_streams_through_one_plan(native_libs):
+    """The device pointer table is rewritten when the pointers change.  A kernel launched earlier on
+    another stream may still be reading it: the library orders the new stream behind the previous
+    one before it overwrites the table, so steps on one plan are serialised whatever stream they
+    are issued on, and each gets its own list's pointers."""
+    from raf_amd import kernels
+
+    sizes = [3 << 20, 1 << 22, 70001, 2 << 20]
+    hp = LansHParams()
+    lists = []
+    for cfg in (97, 98):
+        g, w, m, v = lans_inputs(sizes, cfg=cfg)
+        lists.append((g, w, m, v, _to_dev(g), _to_dev(w), _to_dev(m), _to_dev(v)))
+    plan = kernels.LansPlan(sizes, torch.float32, DEV)
+    plan.set_schedule("pipelined")
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    torch.cuda.synchronize()
+    for step in (1, 2, 3):
+        for (g, w, m, v, tg, tw, tm, tv), s in zip(lists, streams):
+            with torch.cuda.stream(s):
+                plan.step(tg, tw, tm, tv, step, _khp(hp))
+    torch.cuda.synchronize()
+    for g, w, m, v, tg, tw, tm, tv in lists:
+        ow, om, ov = w, m, v
+        for step in (1, 2, 3):
+            ow, om, ov, _ = lans_f64.lans_step(g, ow, om, ov, step, hp)
+        _assert_close([t.cpu().numpy() for t in tw], ow, TOL_1, "w")
+        _assert_close([t.cpu().numpy() for t in tv], ov, TOL_1, "v")
+    plan.close()
