@@ -1,24 +1,40 @@
 #!/usr/bin/env python3
 """Benchmark of the fused optimizer step on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME|all]
 
-A step is one pass of the hot path over one resident parameter set: for the default workload one
-`raf.op.lans` step over a BERT-large-shaped list (391 tensors, 335,141,888 elements; fp32 weights and
-state, fp16 gradients scaled by 1024 and unscaled in the kernel), called through the C ABI.  Inputs
-are synthetic (seeded, generated on the GPU) and resident in HBM before the timed region.  Prints
-ONE JSON line; `value` is algorithmic bytes per step divided by the wall time per step.
+A step is one pass of the hot path over one resident parameter set.  The headline workload is one
+`raf.op.lans` step over a BERT-large-shaped list (391 tensors, 335,141,888 elements; fp32 weights
+and state, fp16 gradients scaled by 1024 and unscaled in the kernel), called through the C ABI.
+Inputs are synthetic (seeded, generated on the GPU) and resident in HBM before the timed region.
+
+Prints ONE JSON line.  Its top-level fields are the headline workload's; `value` is algorithmic
+bytes per step (the three-pass model: 46 B per element with fp16 gradients, 52 B with fp32) divided
+by the wall time per step.  With the default `--workload all` the line also carries
+  "configs"  every benchmark configuration (SGD on one tensor; LANS on the BERT-base, BERT-large,
+             2000-small-tensor and GPT-2-1.5B lists): step time, the dominant kernel's time from
+             HIP events, and its fraction of the 8 TB/s peak by the algorithmic and by the
+             compulsory bytes; for BERT-large and the small-tensor list also the step time through
+             the operator front end (`raf_amd.op.lans`: dialect dispatch -> OpEnv -> Execute);
+  "parity"   a check of the very buffers that were timed, after the timed region, against the CPU
+             oracle: SGD bit for bit, LANS w, m, v of whole tensors of the timed list by the strict
+             per-element relative error, the count of elements over the tolerance, and the error
+             relative to max(|reference|, |old weight|).
 """
 from __future__ import annotations
 
 import argparse
+import hashlib
 import json
 import os
+import re
 import sys
 import time
+from pathlib import Path
 
 import numpy as np
 
+ROOT = Path(__file__).resolve().parent
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 
 # Algorithmic bytes per element of a three-pass LANS step, the figure the bandwidth is quoted on:
@@ -39,19 +55,54 @@ def lans_kernel_bytes_per_elt(g_bytes: int):
 
 SGD_BYTES_PER_ELT = 20  # read x, dx, v; write v1, x1
 
-# Memory traffic per launch of the dominant kernel (bytes), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs scaled by a plain 1 GiB copy (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); figures and commands are in
-# profiles/.  Workloads not listed were not measured (null).
-MEASURED_TRAFFIC = {
-    ("lans_bert_large_fp16grad", "lans_pipelined"): 14_088_700_000,
-    ("lans_bert_large_fp16grad", "lans_apply"): 8_716_600_000,
-    ("sgd_4m_fp32", "sgd_vec4_kernel"): 83_925_600,
-    ("lans_bert_large_mixed_fp16", "lans_pipelined"): 14_759_300_000,
-    ("sgd_multi_bert_large_fp32", "sgd_multi_kernel"): 6_708_200_000,
-    ("l2norm_bert_large_flat_fp32", "l2norm_partials"): 1_340_800_000,
-    ("fuse_bert_large_fp32", "fuse_copy"): 2_683_900_000,
-    ("defuse_bert_large_fp32", "fuse_copy"): 2_683_900_000,
-}
+
+def kernel_sources_digest() -> str:
+    """Digest of the HIP sources the kernel library is built from: a traffic figure measured with
+    rocprofv3 belongs to the kernels it was measured on."""
+    from raf_amd import build
+
+    h = hashlib.sha256()
+    files = sorted([build.CSRC / s for s in build.OPTIM_SOURCES] + list(build.CSRC.glob("*.h")))
+    for f in files:
+        h.update(f.name.encode())
+        h.update(f.read_bytes())
+    return h.hexdigest()[:16]
+
+
+_TRAFFIC_LINE = re.compile(r"^traffic: workload=(\S+) kernel=(\S+) bytes_per_launch=(\d+) kernel_sources=(\w+)\s*$")
+
+
+def measured_traffic(workload: str, kernel: str):
+    """(bytes per launch or None, where that comes from).  The figures live in the rocprofv3
+    summaries under profiles/ as lines `traffic: workload=... kernel=... bytes_per_launch=...
+    kernel_sources=<digest>`; one measured on other kernel sources than the ones in the tree is not
+    quoted."""
+    try:
+        now = kernel_sources_digest()
+    except Exception as e:  # sources not shipped with the library
+        return None, f"kernel sources not readable ({e})"
+    stale = None
+    for md in sorted((ROOT / "profiles").glob("*.md")):
+        for line in md.read_text().splitlines():
+            m = _TRAFFIC_LINE.match(line.strip())
+            if m and m.group(1) == workload and m.group(2) == kernel:
+                if m.group(4) == now:
+                    return int(m.group(3)), f"profiles/{md.name} (rocprofv3 FETCH_SIZE + WRITE_SIZE, kernel sources {now})"
+                stale = f"profiles/{md.name} holds a figure for other kernel sources ({m.group(4)}, tree is {now}): not quoted"
+    return None, stale or "not measured"
+
+
+def roofline_obj(workload, kernel, bytes_per_launch, launch_ms, **extra):
+    achieved = bytes_per_launch / (launch_ms * 1e-3) / 1e9
+    traffic, source = measured_traffic(workload, kernel)
+    obj = {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+           "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+           "traffic_source": source, "bytes_per_launch": bytes_per_launch,
+           "avg_launch_ms": round(launch_ms, 5)}
+    if traffic:
+        obj["frac_by_measured_traffic"] = round(traffic / (launch_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)
+    obj.update(extra)
+    return obj
 
 
 def workloads():
@@ -156,54 +207,185 @@ def cpu_baseline_sgd(n, budget_s=10.0):
                                       f"(-ffp-contract=off), OpenMP {threads} threads"}
 
 
-def bench_lans(name, wl, args):
+# ------------------------------------------------------------------ parity after the timed region
+TOL_ONE_STEP = 1e-5     # max relative error per element after one step
+TOL_100_STEPS = 1e-4    # ... and after up to 100 consecutive steps
+PARITY_ELEMENT_BUDGET = 48_000_000  # elements followed on the CPU per LANS workload
+
+
+def pick_parity_tensors(sizes):
+    """Whole tensors of the timed list to follow on the CPU: the first, the last, the smallest, the
+    median and the largest that fit the budget, then more from the front while the budget lasts
+    (lists of small tensors are checked completely)."""
+    order = sorted(range(len(sizes)), key=lambda t: sizes[t])
+    wanted = [0, len(sizes) - 1, order[0], order[len(order) // 2]]
+    big = [t for t in order if sizes[t] <= PARITY_ELEMENT_BUDGET // 2]
+    if big:
+        wanted.append(big[-1])
+    picks, used = [], 0
+    for t in wanted + list(range(len(sizes))):
+        if t in picks or sizes[t] == 0 or used + sizes[t] > PARITY_ELEMENT_BUDGET:
+            continue
+        picks.append(t)
+        used += sizes[t]
+    return sorted(picks)
+
+
+def error_metrics(got, ref, old_w=None, tol=TOL_ONE_STEP):
+    """Strict max relative error, count of elements over the tolerance, and (for weights) the error
+    relative to max(|reference|, |old weight|), which does not blow up where a weight lands next to
+    zero."""
+    got = got.astype(np.float64).ravel()
+    ref = ref.astype(np.float64).ravel()
+    d = np.abs(got - ref)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        rel = np.where(d == 0.0, 0.0, d / np.abs(ref))
+    out = {"max_rel": float(rel.max()) if rel.size else 0.0, "over_tol": int((rel > tol).sum()),
+           "not_bit_equal": int((d != 0.0).sum())}
+    if old_w is not None:
+        floor = np.maximum(np.abs(ref), np.abs(old_w.astype(np.float64).ravel()))
+        with np.errstate(divide="ignore", invalid="ignore"):
+            out["max_floored"] = float(np.where(d == 0.0, 0.0, d / floor).max()) if d.size else 0.0
+    return out
+
+
+class LansParity:
+    """Follows picked tensors of a LANS workload on the CPU.  Up to 100 steps the whole trajectory
+    is recomputed from the initial state (the GPU's state after warm-up + timed steps is a
+    deterministic function of it); beyond that, ONE more step is run on the GPU from the state the
+    timed region left and compared with one oracle step from that same state."""
+
+    def __init__(self, sizes, g, w, m, v, g16, step0, hp):
+        self.picks = pick_parity_tensors(sizes)
+        self.g16, self.step0, self.hp = g16, step0, hp
+        self.host = lambda ts: [ts[t].cpu().numpy() for t in self.picks]
+        self.g0, self.w0, self.m0, self.v0 = (self.host(x) for x in (g, w, m, v))
+        self.elements = sum(sizes[t] for t in self.picks)
+
+    def check(self, steps_done, g, w, m, v, one_more_step):
+        import torch
+
+        from oracle import c_oracle
+        from oracle.lans_f64 import LansHParams
+
+        threads = min(16, os.cpu_count() or 1, c_oracle.max_threads())
+        ohp = LansHParams(learning_rate=self.hp.learning_rate, beta1=self.hp.beta1, beta2=self.hp.beta2,
+                          eps=self.hp.eps, bias_correction=self.hp.bias_correction,
+                          weight_decay=self.hp.weight_decay, grad_averaging=self.hp.grad_averaging,
+                          mode=self.hp.mode, normalize_grad=bool(self.hp.normalize_grad),
+                          grad_unscale=self.hp.grad_unscale)
+        t0 = time.perf_counter()
+        if steps_done <= 100:
+            mode, tol = f"trajectory of {steps_done} steps from the initial state", (
+                TOL_ONE_STEP if steps_done == 1 else TOL_100_STEPS)
+            rw, rm, rv = [a.copy() for a in self.w0], [a.copy() for a in self.m0], [a.copy() for a in self.v0]
+            old_w = [a.copy() for a in self.w0]
+            for s in range(steps_done):
+                if s == steps_done - 1:
+                    old_w = [a.copy() for a in rw]
+                c_oracle.lans_step_inplace(self.g0, rw, rm, rv, self.step0 + s, ohp, threads=threads)
+        else:
+            mode, tol = f"one more step from the state after {steps_done} steps", TOL_ONE_STEP
+            torch.cuda.synchronize()
+            rw, rm, rv = self.host(w), self.host(m), self.host(v)
+            old_w = [a.copy() for a in rw]
+            one_more_step()
+            torch.cuda.synchronize()
+            c_oracle.lans_step_inplace(self.g0, rw, rm, rv, self.step0 + steps_done, ohp, threads=threads)
+        worst = {}
+        for name, dev, ref, old in (("w", w, rw, old_w), ("m", m, rm, None), ("v", v, rv, None)):
+            agg = {"max_rel": 0.0, "over_tol": 0, "not_bit_equal": 0}
+            for i, t in enumerate(self.picks):
+                e = error_metrics(dev[t].cpu().numpy(), ref[i], old[i] if old else None, tol)
+                agg["max_rel"] = max(agg["max_rel"], e["max_rel"])
+                agg["over_tol"] += e["over_tol"]
+                agg["not_bit_equal"] += e["not_bit_equal"]
+                if "max_floored" in e:
+                    agg["max_floored"] = max(agg.get("max_floored", 0.0), e["max_floored"])
+            worst[name] = {k: (float(f"{x:.3e}") if isinstance(x, float) else x) for k, x in agg.items()}
+        g_intact = all(np.array_equal(g[t].cpu().numpy(), self.g0[i]) for i, t in enumerate(self.picks))
+        ok = g_intact and all(worst[q]["over_tol"] == 0 and np.isfinite(worst[q]["max_rel"]) for q in "wmv")
+        return {"ok": bool(ok), "against": "float64 C restatement of the rule (oracle/optim_oracle.c)",
+                "mode": mode, "tolerance": tol, "tensors_checked": len(self.picks),
+                "elements_checked": self.elements, "w": worst["w"], "m": worst["m"], "v": worst["v"],
+                "gradient_untouched": bool(g_intact), "cpu_seconds": round(time.perf_counter() - t0, 2)}
+
+
+def bench_lans(name, wl, args, entry="c_abi", parity=True, cpu_baseline=True):
     import torch
 
-    from raf_amd import kernels
+    from raf_amd import kernels, op
 
     dev = torch.device("cuda:0")
     sizes, g16 = wl["sizes"], wl["g16"]
     total = sum(sizes)
     g, w, m, v = gen_lans(sizes, g16, wl["zero_state"], dev)
-    plan = kernels.LansPlan(sizes, torch.float16 if g16 else torch.float32, dev)
-    if args.schedule != "auto":
-        plan.set_schedule(args.schedule)
-    schedule = plan.schedule
     hp = kernels.make_hparams(grad_unscale=(1.0 / 1024 if g16 else 1.0))
     copy16 = bool(wl.get("copy16"))
     p16 = [torch.empty(n, dtype=torch.float16, device=dev) for n in sizes] if copy16 else None
-    plan.bind(g, w, m, v, hp, p=p16)
     step_t = torch.full((), float(wl["step0"]), dtype=torch.float32, device=dev)
+    checker = LansParity(sizes, g, w, m, v, g16, wl["step0"], hp) if parity and not args.hip_graph else None
 
-    def one_step():
-        plan.step_bound(step_t)
-        step_t.add_(1.0)  # the step counter lives on the device, as in the reference's traced optimizer
+    plan = None
+    if entry == "c_abi":
+        # rafhip_lans_plan_bind once, then one rafhip_lans_step_bound per step
+        plan = kernels.LansPlan(sizes, torch.float16 if g16 else torch.float32, dev)
+        if args.schedule != "auto":
+            plan.set_schedule(args.schedule)
+        schedule = plan.schedule
+        plan.bind(g, w, m, v, hp, p=p16)
 
+        def one_step():
+            plan.step_bound(step_t)
+            step_t.add_(1.0)  # the step counter lives on the device, as in the reference's traced optimizer
+    else:
+        # raf.op.lans(tensor_list, step, ...) as the reference's LANS.step calls it
+        # (python/raf/optim/lans.py:74-103): schema -> declare -> dialect dispatch -> OpEnv -> Execute
+        if args.schedule != "auto":
+            os.environ["RAFHIP_LANS_SCHEDULE"] = args.schedule
+        op.clear_op_env_cache()
+        op.set_lans_grad_unscale(hp.grad_unscale)
+        tensor_list = g + w + m + v + (p16 or [])
+        call = op.lans_mixed if copy16 else op.lans
+        schedule = args.schedule
+
+        def one_step():
+            call(tensor_list, step_t, hp.learning_rate, hp.beta1, hp.beta2, hp.eps, True, hp.weight_decay,
+                 True, True, True)
+            step_t.add_(1.0)
+
+    steps_done = 0
     for _ in range(args.warmup):
         one_step()
+    steps_done += args.warmup
     graph = None
+    kernel_events = entry == "c_abi" and not args.no_kernel_events and not args.hip_graph
     if args.hip_graph:
         # The launches of one step (and the counter's increment) recorded once and replayed: what a
         # training loop captured in a HIP graph pays per step.  Per-kernel events stay outside.
-        args.no_kernel_events = True
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             one_step()
         for _ in range(3):
             graph.replay()
-    if not args.no_kernel_events:
+    if kernel_events:
         plan.timing_enable(args.steps)
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    start.record()
     for _ in range(args.steps):
         if graph is not None:
             graph.replay()
         else:
             one_step()
+    stop.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    steps_done += args.steps
     ms_per_step = wall * 1e3 / args.steps
+    dev_ms_per_step = start.elapsed_time(stop) / args.steps  # events on the stream the steps run on
 
     a, b, c = lans_bytes_per_elt(2 if g16 else 4)
     ka, kb, kc = lans_kernel_bytes_per_elt(2 if g16 else 4)
@@ -212,38 +394,39 @@ def bench_lans(name, wl, args):
     lib = _libs()
     short = all(-(-n // lib.rafhip_lans_chunk_elements(n)) <= 32 for n in sizes if n)
     cached = total * (14 if g16 else 16) <= (192 << 20)
+    if schedule == "auto":
+        schedule = "pipelined" if total >= (64 << 20) else "phased"
     launches = 2 if schedule == "pipelined" else (3 if short and cached else 5)
     if copy16:  # the third pass also writes the 2-byte copy of the new weight
         c, kc = c + 2, kc + 2
     bytes_step = total * (a + b + c)
     out = {
-        "metric": "LANS optimizer-step achieved HBM bandwidth (algorithmic bytes / step time); "
-                  "ms_per_step is the step time",
+        "metric": "LANS optimizer step: algorithmic bandwidth = three-pass model bytes "
+                  f"({a + b + c} B per element) / step time, not bytes moved; ms_per_step is the step time",
         "value": round(bytes_step / (ms_per_step * 1e-3) / 1e9, 1),
         "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f64", "data": "synthetic",
-        "config": {"workload": name, "tensors": len(sizes), "elements": total,
+        "config": {"workload": name, "entry": entry, "tensors": len(sizes), "elements": total,
                    "storage": "fp32 w/m/v, " + ("fp16 g (x1024, unscaled in kernel)" if g16 else "fp32 g") +
                               (", fp16 copy of the new weights written" if copy16 else ""),
                    "bytes_per_element": a + b + c, "bytes_per_step": bytes_step,
-                   "kernel_bytes_per_element": ka + kb + kc,
-                   "pct_of_hbm_peak": round(100 * bytes_step / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
+                   "kernel_bytes_per_element": ka + kb + kc, "compulsory_bytes_per_element": c,
+                   "pct_of_peak_by_algorithmic_bytes": round(100 * bytes_step / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
+                   "pct_of_peak_by_requested_bytes": round(100 * total * (ka + kb + kc) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
+                   "pct_of_peak_by_compulsory_bytes": round(100 * total * c / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
+                   "device_ms_per_step": round(dev_ms_per_step, 4),
                    "schedule": schedule, "launches_per_step": launches, "hip_graph": bool(args.hip_graph)},
     }
-    if not args.no_kernel_events:
+    if kernel_events:
         ts = np.array([plan.timing_read(i) for i in range(args.steps)], dtype=np.float64)
         avg = ts.mean(axis=0)
         if schedule == "phased":
             # dominant kernel: lans_apply (reads g,w,m,v, writes w,m,v)
             apply_ms = float(avg[4])
-            achieved = total * c / (apply_ms * 1e-3) / 1e9
-            out["roofline"] = {"bound": "hbm", "kernel": "lans_apply", "achieved": round(achieved, 1),
-                               "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                               "traffic": MEASURED_TRAFFIC.get((name, "lans_apply")),
-                               "bytes_per_launch": total * c, "avg_launch_ms": round(apply_ms, 4)}
+            out["roofline"] = roofline_obj(name, "lans_apply", total * c, apply_ms)
             out["kernels_ms"] = {"lans_norm_g": round(float(avg[0]), 4), "lans_finish(a)": round(float(avg[1]), 4),
                                  "lans_norm_u": round(float(avg[2]), 4), "lans_finish(b)": round(float(avg[3]), 4),
                                  "lans_apply": round(apply_ms, 4)}
@@ -251,24 +434,35 @@ def bench_lans(name, wl, args):
                                    "lans_norm_u": round(total * kb / avg[2] / 1e6, 1),
                                    "lans_apply": round(total * kc / avg[4] / 1e6, 1)}
         else:
-            # one persistent kernel does all three passes
+            # one persistent kernel does all three passes; the same launch is also priced by the bytes
+            # the kernel requests (the norm of w rides on pass B) and by the compulsory
+            # read-once/write-once bytes
             k_ms = float(avg[1])
-            achieved = bytes_step / (k_ms * 1e-3) / 1e9
-            out["roofline"] = {"bound": "hbm", "kernel": "lans_pipelined", "achieved": round(achieved, 1),
-                               "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                               "traffic": MEASURED_TRAFFIC.get((name, "lans_pipelined")),
-                               "bytes_per_launch": bytes_step, "avg_launch_ms": round(k_ms, 4),
-                               # the same launch priced by the bytes the kernel requests (the norm of w
-                               # rides on pass B) and by the compulsory read-once/write-once bytes
-                               "achieved_by_requested_bytes": round(total * (ka + kb + kc) / (k_ms * 1e-3) / 1e9, 1),
-                               "achieved_by_compulsory_bytes": round(total * c / (k_ms * 1e-3) / 1e9, 1)}
+            out["roofline"] = roofline_obj(
+                name, "lans_pipelined", bytes_step, k_ms,
+                achieved_by_requested_bytes=round(total * (ka + kb + kc) / (k_ms * 1e-3) / 1e9, 1),
+                achieved_by_compulsory_bytes=round(total * c / (k_ms * 1e-3) / 1e9, 1),
+                frac_by_requested_bytes=round(total * (ka + kb + kc) / (k_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                frac_by_compulsory_bytes=round(total * c / (k_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4))
             out["kernels_ms"] = {"lans_prepare": round(float(avg[0]), 4), "lans_pipelined": round(k_ms, 4)}
-    if not args.no_cpu_baseline:
+    else:
+        # no per-kernel events through this entry: the whole step on the device stands in for the launch
+        out["roofline"] = roofline_obj(name, "lans step (all launches)", bytes_step, dev_ms_per_step,
+                                       note="device time of the whole step between events on the step's stream")
+    if checker is not None:
+        out["parity"] = checker.check(steps_done, g, w, m, v, one_step)
+    if entry != "c_abi":
+        op.set_lans_grad_unscale(1.0)
+        op.clear_op_env_cache()
+        os.environ.pop("RAFHIP_LANS_SCHEDULE", None)
+    if plan is not None:
+        plan.close()
+    if cpu_baseline and not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline_lans(sizes, g16)
     return out
 
 
-def bench_sgd(name, wl, args):
+def bench_sgd(name, wl, args, parity=True, cpu_baseline=True):
     import torch
 
     from raf_amd import kernels
@@ -302,20 +496,30 @@ def bench_sgd(name, wl, args):
     ms_per_step = wall * 1e3 / args.steps
     dev_ms = start.elapsed_time(stop) / args.steps  # kernels run on torch's current stream
     bytes_step = n * SGD_BYTES_PER_ELT
-    achieved = bytes_step / (dev_ms * 1e-3) / 1e9
     out = {
-        "metric": "SGD momentum step achieved HBM bandwidth (algorithmic bytes / step time)",
+        "metric": "SGD momentum step: algorithmic bandwidth (20 B per element / step time)",
         "value": round(bytes_step / (ms_per_step * 1e-3) / 1e9, 1), "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": name, "elements": n, "bytes_per_element": SGD_BYTES_PER_ELT,
-                   "buffer_sets_rotated": sets},
-        "roofline": {"bound": "hbm", "kernel": "sgd_vec4_kernel", "achieved": round(achieved, 1),
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC.get((name, "sgd_vec4_kernel")), "bytes_per_launch": bytes_step,
-                     "avg_launch_ms": round(dev_ms, 5)},
+        "config": {"workload": name, "entry": "c_abi", "elements": n, "bytes_per_element": SGD_BYTES_PER_ELT,
+                   "compulsory_bytes_per_element": SGD_BYTES_PER_ELT, "buffer_sets_rotated": sets},
+        "roofline": roofline_obj(name, "sgd_vec4_kernel", bytes_step, dev_ms),
     }
-    if not args.no_cpu_baseline:
+    if parity:
+        # every element of the outputs of the timed calls, bit for bit: the op is out of place, so
+        # each buffer set still holds the inputs its outputs were computed from
+        from oracle import c_oracle
+
+        bad, checked = 0, 0
+        for x, dx, v, v1, x1 in bufs[:min(sets, args.warmup + args.steps)]:
+            ov, ox = c_oracle.sgd_step(x.cpu().numpy(), dx.cpu().numpy(), v.cpu().numpy(), 0.01, 0.9, threads=8)
+            bad += int((v1.cpu().numpy().view(np.uint32) != ov.view(np.uint32)).sum())
+            bad += int((x1.cpu().numpy().view(np.uint32) != ox.view(np.uint32)).sum())
+            checked += 2 * n
+        out["parity"] = {"ok": bad == 0, "against": "fp32 C restatement, four roundings, no contraction (oracle/optim_oracle.c)",
+                         "mode": "bit-exact comparison of v1 and x1 of every buffer set used", "elements_checked": checked,
+                         "not_bit_equal": bad}
+    if cpu_baseline and not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline_sgd(n)
     return out
 
@@ -340,23 +544,18 @@ def _timed(fn, args):
 
 
 def _line(metric, name, dtype, bytes_step, wall_ms, dev_ms, kernel, args, config):
-    achieved = bytes_step / (dev_ms * 1e-3) / 1e9
     return {
         "metric": metric, "value": round(bytes_step / (wall_ms * 1e-3) / 1e9, 1), "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
         "config": dict(workload=name, **config),
-        "roofline": {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC.get((name, kernel)), "bytes_per_launch": bytes_step,
-                     "avg_launch_ms": round(dev_ms, 5)},
+        "roofline": roofline_obj(name, kernel, bytes_step, dev_ms),
     }
 
 
 def bench_sgd_multi(name, wl, args):
     import torch
 
-    from oracle import c_oracle
     from raf_amd import kernels
 
     dev = torch.device("cuda:0")
@@ -381,7 +580,6 @@ def bench_sgd_multi(name, wl, args):
 def bench_l2norm(name, wl, args):
     import torch
 
-    from oracle import tensor_ops
     from raf_amd import kernels
 
     dev = torch.device("cuda:0")
@@ -393,6 +591,8 @@ def bench_l2norm(name, wl, args):
     res = _line("L2 norm achieved HBM bandwidth (algorithmic bytes / time)", name, "f64", 4 * n, wall_ms, dev_ms,
                 "l2norm_partials", args, {"elements": n, "bytes_per_element": 4, "storage": "fp32"})
     if not args.no_cpu_baseline:
+        from oracle import tensor_ops
+
         sample = x[:1 << 26].cpu().numpy()
         best = None
         for _ in range(5):
@@ -408,7 +608,6 @@ def bench_l2norm(name, wl, args):
 def bench_fuse(name, wl, args):
     import torch
 
-    from oracle import tensor_ops
     from raf_amd import kernels
 
     dev = torch.device("cuda:0")
@@ -427,6 +626,8 @@ def bench_fuse(name, wl, args):
                 kernel, args, {"tensors": len(sizes), "bytes_read_per_step": plan.total_bytes,
                                "bytes_written_per_step": plan.total_bytes, "launches_per_step": 1})
     if not args.no_cpu_baseline:
+        from oracle import tensor_ops
+
         host = [p.cpu().numpy() for p in parts[:48]]
         best = None
         for _ in range(5):
@@ -471,9 +672,7 @@ def bench_copy(name, wl, args):
             "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
             "config": {"workload": name, "bytes_read_per_step": wl["nbytes"], "bytes_written_per_step": wl["nbytes"]},
-            "roofline": {"bound": "hbm", "kernel": "torch copy", "achieved": round(moved / (dev_ms * 1e-3) / 1e9, 1),
-                         "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(moved / (dev_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-                         "traffic": None, "bytes_per_launch": moved, "avg_launch_ms": round(dev_ms, 4)}}
+            "roofline": roofline_obj(name, "torch copy", moved, dev_ms)}
 
 
 def bench_traced_sgd(name, wl, args):
@@ -510,15 +709,97 @@ def bench_traced_sgd(name, wl, args):
     return res
 
 
+def _config_entry(line):
+    """What the "configs" block keeps of a workload's full line."""
+    cfg, roof = line["config"], line["roofline"]
+    comp = cfg.get("compulsory_bytes_per_element")
+    launch_s = roof["avg_launch_ms"] * 1e-3
+    entry = {
+        "entry": cfg.get("entry", "c_abi"), "elements": cfg["elements"], "tensors": cfg.get("tensors", 1),
+        "schedule": cfg.get("schedule"), "ms_per_step": line["ms_per_step"], "steps": line["steps"],
+        "algorithmic_GBps": line["value"], "bytes_per_element": cfg["bytes_per_element"],
+        "kernel": roof["kernel"], "kernel_ms": roof["avg_launch_ms"],
+        "frac_by_algorithmic_bytes": roof["frac"],
+        "frac_by_compulsory_bytes": roof.get("frac_by_compulsory_bytes"),
+        "traffic": roof["traffic"], "traffic_source": roof["traffic_source"],
+    }
+    if entry["frac_by_compulsory_bytes"] is None and comp and roof["kernel"] not in ("lans_apply",):
+        entry["frac_by_compulsory_bytes"] = round(cfg["elements"] * comp / launch_s / 1e9 / HBM_PEAK_GBPS, 4)
+    if "kernels_ms" in line:
+        entry["kernels_ms"] = line["kernels_ms"]
+    return entry
+
+
+def run_suite(table, args):
+    """Every benchmark configuration in one process, one after the other, each with its parity
+    check; the headline workload first, and its line is the one whose fields go to the top level."""
+    import copy
+    import gc
+
+    import torch
+
+    def release():
+        gc.collect()
+        torch.cuda.empty_cache()
+
+    headline = "lans_bert_large_fp16grad"
+    out = bench_lans(headline, table[headline], args, entry="c_abi", parity=True, cpu_baseline=True)
+    configs = {headline: _config_entry(out)}
+    parity = {headline: out.pop("parity", None)}
+    release()
+
+    def more_steps(k):
+        a = copy.copy(args)
+        a.steps, a.warmup = max(1, int(args.steps * k)), args.warmup
+        return a
+
+    def add(name, line):
+        configs[name] = _config_entry(line)
+        if "parity" in line:
+            parity[name] = line["parity"]
+        release()
+
+    # the operator front end on the headline list: raf.op.lans -> dialect dispatch -> OpEnv -> Execute
+    line = bench_lans(headline, table[headline], args, entry="dialect", parity=True, cpu_baseline=False)
+    add(headline + "@dialect", line)
+    add("sgd_4m_fp32", bench_sgd("sgd_4m_fp32", table["sgd_4m_fp32"], more_steps(4), parity=True, cpu_baseline=False))
+    add("lans_bert_base_fp32", bench_lans("lans_bert_base_fp32", table["lans_bert_base_fp32"], args, cpu_baseline=False))
+    small = "lans_2000_small_tensors"
+    quiet = copy.copy(args)
+    quiet.no_kernel_events = True  # per-kernel events cost a fifth of this 0.1 ms step
+    line = bench_lans(small, table[small], more_steps(4), cpu_baseline=False)
+    add(small, line)
+    quiet.steps = line["steps"]
+    add(small + "@c_abi_no_events", bench_lans(small, table[small], quiet, parity=False, cpu_baseline=False))
+    add(small + "@dialect", bench_lans(small, table[small], quiet, entry="dialect", cpu_baseline=False))
+    big = copy.copy(args)
+    big.steps, big.warmup = min(args.steps, 20), min(args.warmup, 5)  # 11.5 ms per step, 25 GB resident
+    add("lans_gpt2_1p5b_fp32", bench_lans("lans_gpt2_1p5b_fp32", table["lans_gpt2_1p5b_fp32"], big, cpu_baseline=False))
+
+    for base in (headline, small):
+        direct = configs[base + "@c_abi_no_events"] if base == small else configs[base]
+        via = configs[base + "@dialect"]
+        via["overhead_vs_c_abi_us"] = round((via["ms_per_step"] - direct["ms_per_step"]) * 1e3, 1)
+        via["overhead_vs_c_abi_pct"] = round(100 * (via["ms_per_step"] / direct["ms_per_step"] - 1), 2)
+    out["configs"] = configs
+    parity["ok"] = all(p is None or p.get("ok", False) for p in parity.values())
+    out["parity"] = parity
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="lans_bert_large_fp16grad")
+    ap.add_argument("--workload", default="all",
+                    help="a workload name, or 'all' (default): the headline line plus every configuration and parity")
+    ap.add_argument("--entry", default="c_abi", choices=["c_abi", "dialect"],
+                    help="LANS workloads: call the C ABI (bound plan) or the operator front end raf_amd.op.lans")
     ap.add_argument("--schedule", default="auto", choices=["auto", "phased", "pipelined"],
                     help="LANS launch schedule (bit-identical results); auto = the library's choice")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline leg")
+    ap.add_argument("--no-parity", action="store_true", help="skip the parity check after the timed region")
     ap.add_argument("--no-kernel-events", action="store_true", help="do not record per-kernel HIP events")
     ap.add_argument("--hip-graph", action="store_true",
                     help="LANS workloads: capture one step in a HIP graph and time its replays")
@@ -529,8 +810,8 @@ def main():
     if args.steps < 1 or args.warmup < 0:
         sys.exit("bench.py: --steps must be >= 1 and --warmup >= 0")
     table = workloads()
-    if args.workload not in table:
-        sys.exit(f"bench.py: unknown workload {args.workload!r}; choose from {sorted(table)}")
+    if args.workload != "all" and args.workload not in table:
+        sys.exit(f"bench.py: unknown workload {args.workload!r}; choose from {sorted(table)} or 'all'")
     import torch
 
     if not torch.cuda.is_available():
@@ -538,11 +819,22 @@ def main():
     from raf_amd import _lib
 
     _lib.optim()  # fails loudly if the HIP library is not built
-    wl = table[args.workload]
-    fn = {"lans": bench_lans, "sgd": bench_sgd, "copy": bench_copy, "l2norm": bench_l2norm,
-          "fuse": bench_fuse, "sgd_multi": bench_sgd_multi, "traced_sgd": bench_traced_sgd}[wl["kind"]]
-    out = fn(args.workload, wl, args)
+    if args.workload == "all":
+        out = run_suite(table, args)
+    else:
+        wl = table[args.workload]
+        if wl["kind"] == "lans":
+            out = bench_lans(args.workload, wl, args, entry=args.entry, parity=not args.no_parity)
+        elif wl["kind"] == "sgd":
+            out = bench_sgd(args.workload, wl, args, parity=not args.no_parity)
+        else:
+            fn = {"copy": bench_copy, "l2norm": bench_l2norm, "fuse": bench_fuse, "sgd_multi": bench_sgd_multi,
+                  "traced_sgd": bench_traced_sgd}[wl["kind"]]
+            out = fn(args.workload, wl, args)
     print(json.dumps(out), flush=True)
+    parity = out.get("parity")
+    if parity is not None and not parity.get("ok", True):
+        sys.exit("bench.py: the parity check after the timed region FAILED; the figures above are invalid")
 
 
 if __name__ == "__main__":

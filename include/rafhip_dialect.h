@@ -174,6 +174,35 @@ int rafhip_raf_traced_sgd_execute(rafhip_raf_env* env, const rafhip_tensor_desc*
                                   void* stream);
 int rafhip_raf_env_ir_text(const rafhip_raf_env* env, int32_t fused, char* buf, int32_t buflen);
 
+/* Whole traced optimizers.  Builds the optimizer part of the function that the reference's traced
+ * optimizer makes for a model with n parameters -- kind 0: SGD (python/raf/optim/sgd.py:187-215;
+ * g = the gradients, m unused), kind 1: LANS for a half-precision model
+ * (python/raf/optim/lans.py:244-312: group_cast, raf.op.lans, cast, add(out=p)) -- runs FuseDialect
+ * with the hip dialect's graph rewrites and patterns, and makes one OpEnv per call of the result.
+ * Every list holds n descriptors; p (the model's 16-bit parameters) may be NULL for SGD on a
+ * float32 model.  zero_is_constant tells whether the optimizer's zero tensor is already bound into
+ * the graph as a constant (then cast and copy are folded into the multi-tensor op) or is a free
+ * variable as traced (then they stay, and have no backend in this library: the make call fails
+ * unless allow_partial, which skips the result fields that need them).  hyper: SGD
+ * {learning_rate, momentum}; LANS the nine schema values in order (ints and bools as numbers).
+ * _execute runs the OpEnvs in order, in place on the caller's tensors; workspace as reported by
+ * rafhip_raf_env_workspace_bytes.  rafhip_raf_env_graph_ops lists what the fused graph calls, in
+ * order, joined by ';': dialect ops, "<dialect>._fused_op(<pattern>)", and with a leading '!' ops
+ * that were left without a backend.  On failure *env_out still holds the graphs for
+ * rafhip_raf_env_ir_text. */
+int rafhip_raf_traced_optimizer_make(int32_t kind, int32_t n, const rafhip_tensor_desc* g,
+                                     const rafhip_tensor_desc* w, const rafhip_tensor_desc* m,
+                                     const rafhip_tensor_desc* v, const rafhip_tensor_desc* p,
+                                     const rafhip_tensor_desc* step, int32_t zero_is_constant,
+                                     const double* hyper, int32_t n_hyper, int32_t allow_partial,
+                                     rafhip_raf_env** env_out);
+int rafhip_raf_traced_optimizer_execute(rafhip_raf_env* env, int32_t n, const rafhip_tensor_desc* g,
+                                        const rafhip_tensor_desc* w, const rafhip_tensor_desc* m,
+                                        const rafhip_tensor_desc* v, const rafhip_tensor_desc* p,
+                                        const rafhip_tensor_desc* step, int32_t allow_partial,
+                                        void* workspace, int64_t workspace_bytes, void* stream);
+int rafhip_raf_env_graph_ops(const rafhip_raf_env* env, char* buf, int32_t buflen);
+
 /* hip-dialect extension for learning-rate schedules: moves the learning rate of an OpEnv made by
  * the sgd, sgd_multi, lans or lans_mixed makers, so that a new value every step does not mean a
  * new OpEnv (in the reference the learning rate is a schema constant and part of the OpEnv cache

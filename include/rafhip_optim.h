@@ -155,13 +155,15 @@ typedef enum rafhip_lans_schedule {
 } rafhip_lans_schedule;
 
 /*
- * Pure host arithmetic: the work list of the pipelined schedule as int32 triples
- * (kind, tensor, index), kind being 0 = pass A unit, 1 = pass B chunk, 2 = pass C chunk,
- * 3 = a one-chunk tensor taken through all three passes by one workgroup, 4 = finish pass A
+ * Pure host arithmetic: the work list of the pipelined schedule (as made for a device of 256 CUs)
+ * as int32 triples (kind, tensor, index), kind being 0 = pass A unit, 1 = pass B chunk, 2 = pass C
+ * chunk, 3 = a one-chunk tensor taken through all three passes by one workgroup, 4 = finish pass A
  * (add the tensor's partials, publish ||g||), 5 = finish pass B (publish ||w|| and the trust
- * ratios).  group_elements <= 0 selects the default group size.  triples_out may be NULL to query
- * the count.  The kernel's bounded waits rely on this order, per tensor: every pass-A unit, then
- * finish A, then every pass-B chunk, then finish B, then every pass-C chunk.
+ * ratios); + 8 for an item of a tensor too large for the Infinity Cache, whose accesses bypass it
+ * and whose items are spread over the whole list.
+ * group_elements <= 0 selects the default group size.  triples_out may be NULL to query the count.
+ * The kernel's bounded waits rely on this order, per tensor: every pass-A unit, then finish A,
+ * then every pass-B chunk, then finish B, then every pass-C chunk.
  */
 int rafhip_lans_pipeline_order(int32_t n_tensors, const int64_t* numel, int64_t group_elements,
                                int32_t* triples_out, int64_t capacity, int64_t* n_items_out);

@@ -180,6 +180,11 @@ DIALECT_SYMBOLS = {
                                            c_double, c_double, POINTER(c_void_p)]),
     "rafhip_raf_traced_sgd_execute": (c_int, [c_void_p] + [POINTER(TensorDesc)] * 3 + [c_void_p]),
     "rafhip_raf_env_ir_text": (c_int, [c_void_p, c_int32, c_char_p, c_int32]),
+    "rafhip_raf_traced_optimizer_make": (c_int, [c_int32, c_int32] + [POINTER(TensorDesc)] * 6 +
+                                         [c_int32, POINTER(c_double), c_int32, c_int32, POINTER(c_void_p)]),
+    "rafhip_raf_traced_optimizer_execute": (c_int, [c_void_p, c_int32] + [POINTER(TensorDesc)] * 6 +
+                                            [c_int32, c_void_p, c_int64, c_void_p]),
+    "rafhip_raf_env_graph_ops": (c_int, [c_void_p, c_char_p, c_int32]),
     "rafhip_raf_env_set_learning_rate": (c_int, [c_void_p, c_double]),
     "rafhip_raf_env_set_grad_unscale": (c_int, [c_void_p, c_float]),
     "rafhip_raf_env_set_dynamic_scale": (c_int, [c_void_p, POINTER(TensorDesc), POINTER(TensorDesc)]),

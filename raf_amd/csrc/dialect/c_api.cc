@@ -33,6 +33,17 @@ struct rafhip_raf_env {
   std::vector<rafhip_tensor_desc> list_descs;
   std::vector<int64_t> list_shapes;
   value::Value list_tuple;
+  // Only for an env made from a whole optimizer graph (rafhip_raf_traced_optimizer_make): one
+  // OpEnv per call of the fused graph, in execution order.
+  struct GraphCall {
+    const ir::ExprNode* node = nullptr;
+    std::string what;       // the dialect op, or "<dialect>._fused_op(<pattern>)"; "!" + op if it has no backend
+    OpEnvPtr env;           // empty if unsupported
+    int out_arg = -1;       // fused function: the argument whose memory the result shares
+  };
+  std::vector<GraphCall> graph_calls;
+  std::vector<size_t> var_counts;  // how many variables each descriptor list of the make call bound
+  int kind = -1;                   // 0 SGD, 1 LANS
 };
 
 namespace {
@@ -148,6 +159,201 @@ std::vector<value::TensorValue> Outputs(const rafhip_raf_env* env) {
     for (const auto& f : value::AsTuple(env->call->out)->fields) outs.push_back(value::AsTensor(f));
   }
   return outs;
+}
+
+// ------------------------------------------------------------------ running a fused graph
+// A small evaluator for graphs that FuseDialect has worked on: variables take the caller's
+// tensors, tuples and projections are formed, and every call is either a `hip` dialect op of the
+// optimizer family or a fused function, each with an OpEnv of its own that is made once and then
+// executed in order.  Anything else (an element-wise base op that nothing fused) has no backend in
+// this library; a result field that needs one is skipped when the caller allows that, and the
+// make call reports the op with a leading '!'.
+struct Unsupported : Error {
+  using Error::Error;
+};
+
+class GraphRunner {
+ public:
+  GraphRunner(rafhip_raf_env* env, const std::map<const ir::ExprNode*, value::Value>& bindings, bool make,
+              char* workspace, int64_t workspace_bytes)
+      : env_(env), bindings_(bindings), make_(make), ws_(workspace), ws_left_(workspace_bytes) {}
+
+  value::Value Eval(const ir::Expr& e) {
+    auto it = memo_.find(e.get());
+    if (it != memo_.end()) return it->second;
+    value::Value v = Compute(e);
+    memo_[e.get()] = v;
+    return v;
+  }
+
+ private:
+  static double Number(const value::Value& v, const char* what) {
+    if (auto f = std::dynamic_pointer_cast<FloatValueObj>(v)) return f->value;
+    if (auto i = std::dynamic_pointer_cast<IntValueObj>(v)) return (double)i->value;
+    throw Error(std::string(what) + " must be a scalar constant");
+  }
+
+  rafhip_raf_env::GraphCall& Slot(const ir::ExprNode* node) {
+    for (auto& gc : env_->graph_calls)
+      if (gc.node == node) return gc;
+    RAF_CHECK(make_, "the graph was not prepared for this call");
+    env_->graph_calls.emplace_back();
+    env_->graph_calls.back().node = node;
+    return env_->graph_calls.back();
+  }
+
+  void Run(OpEnv* op_env, const std::vector<value::Value>& inputs, const value::Value& out) {
+    int64_t need = 0;
+    for (const auto& r : op_env->workspace_requests()) need += RoundUp(r.nbytes);
+    if (need > ws_left_) throw Error("the workspace is too small for the graph's operators");
+    WorkspaceBinding bind(op_env, ws_, need);
+    ws_ += need;
+    ws_left_ -= need;
+    op_env->Execute(inputs, out);
+  }
+
+  value::Value Compute(const ir::Expr& e) {
+    if (ir::AsVar(e)) {
+      auto it = bindings_.find(e.get());
+      RAF_CHECK(it != bindings_.end(), "a variable of the graph has no value");
+      return it->second;
+    }
+    if (const auto* k = ir::AsConstant(e)) {
+      switch (k->value_kind) {
+        case ir::ConstantNode::kNull:
+          return nullptr;
+        case ir::ConstantNode::kFloat: {
+          auto v = std::make_shared<FloatValueObj>();
+          v->value = k->f;
+          return v;
+        }
+        case ir::ConstantNode::kInt: {
+          auto v = std::make_shared<IntValueObj>();
+          v->value = k->i;
+          return v;
+        }
+        case ir::ConstantNode::kString: {
+          auto v = std::make_shared<StringValueObj>();
+          v->value = k->s;
+          return v;
+        }
+        default:
+          throw Unsupported("a tensor constant that nothing folded away has no storage here");
+      }
+    }
+    if (const auto* t = ir::AsTupleNode(e)) {
+      std::vector<value::Value> fields;
+      for (const auto& f : t->fields) fields.push_back(Eval(f));
+      return value::MakeTuple(std::move(fields));
+    }
+    if (const auto* g = ir::AsTupleGetItem(e)) {
+      auto tuple = value::AsTuple(Eval(g->tuple));
+      RAF_CHECK((size_t)g->index < tuple->fields.size(), "tuple index out of range");
+      return tuple->fields[(size_t)g->index];
+    }
+    const auto* c = ir::AsCall(e);
+    RAF_CHECK(c != nullptr, "unexpected expression in a graph to run");
+    std::vector<value::Value> args;
+    for (const auto& a : c->args) args.push_back(Eval(a));
+    const Device device = env_->call->device;
+    if (const auto* func = ir::AsFunction(c->op)) {
+      auto& slot = Slot(e.get());
+      if (make_) {
+        auto list = std::make_shared<schema::ListArgs>();
+        list->args = args;
+        auto cv = std::make_shared<CallValuesNode>();
+        cv->closure = c->op;
+        cv->args = list;
+        cv->device = device;
+        slot.env = DispatchFusedOp(cv);
+        auto name = func->attrs.find(ir::kPatternName);
+        slot.what = func->attrs.at(ir::kDialect) + "._fused_op(" + (name == func->attrs.end() ? "" : name->second) + ")";
+        // an element-wise root with out=: the result shares that argument's memory
+        const auto* root = ir::AsCall(func->body);
+        if (root && root->args.size() == 4)
+          for (size_t i = 0; i < func->params.size(); ++i)
+            if (func->params[i].get() == root->args[2].get()) slot.out_arg = (int)i;
+        RAF_CHECK(slot.out_arg >= 0, "cannot tell where the fused function's result lives");
+      } else {
+        Run(slot.env.get(), args, args[(size_t)slot.out_arg]);
+      }
+      return args[(size_t)slot.out_arg];
+    }
+    const std::string& name = ir::AsOp(c->op)->name;
+    const bool lans = name == "raf.op.hip.lans" || name == "raf.op.hip.lans_mixed";
+    const bool sgd = name == "raf.op.hip.sgd_multi" || name == "raf.op.hip.sgd_multi_mixed";
+    if (!lans && !sgd) {
+      if (make_) {
+        auto& slot = Slot(e.get());
+        slot.what = "!" + name;
+      }
+      throw Unsupported("Cannot find a valid dispatch for op " + name +
+                        ": outside a fused function the hip dialect has no backend for it");
+    }
+    auto& slot = Slot(e.get());
+    auto tuple = value::AsTuple(args.at(0));
+    if (make_) {
+      std::shared_ptr<schema::ArgsBase> sargs;
+      std::vector<value::TensorValue> tensors;
+      for (const auto& f : tuple->fields) tensors.push_back(value::AsTensor(f));
+      if (lans) {
+        RAF_CHECK(args.size() == 11, name + " takes 11 arguments");
+        auto a = std::make_shared<schema::LansArgs>();
+        a->tensor_list = tensors;
+        a->step = value::AsTensor(args[1]);
+        a->learning_rate = (float)Number(args[2], "learning_rate");
+        a->beta1 = (float)Number(args[3], "beta1");
+        a->beta2 = (float)Number(args[4], "beta2");
+        a->eps = (float)Number(args[5], "eps");
+        a->bias_correction = (int)Number(args[6], "bias_correction");
+        a->weight_decay = (float)Number(args[7], "weight_decay");
+        a->grad_averaging = (int)Number(args[8], "grad_averaging");
+        a->mode = (int)Number(args[9], "mode");
+        a->normalize_grad = Number(args[10], "normalize_grad") != 0;
+        sargs = a;
+      } else {
+        RAF_CHECK(args.size() == 3, name + " takes 3 arguments");
+        auto a = std::make_shared<schema::SgdMultiArgs>();
+        a->tensor_list = tensors;
+        a->learning_rate = Number(args[1], "learning_rate");
+        a->mu = Number(args[2], "mu");
+        sargs = a;
+      }
+      CallValues cv = MakeCall(name, sargs);
+      cv->device = device;
+      cv->out = tuple;
+      slot.env = DispatchSingleOp(cv);
+      slot.what = name;
+    } else {
+      std::vector<value::Value> inputs = {tuple};
+      if (lans) inputs.push_back(args[1]);
+      Run(slot.env.get(), inputs, tuple);
+    }
+    return tuple;  // these ops return their list: the update is in place
+  }
+
+  rafhip_raf_env* env_;
+  const std::map<const ir::ExprNode*, value::Value>& bindings_;
+  bool make_;
+  char* ws_;
+  int64_t ws_left_;
+  std::map<const ir::ExprNode*, value::Value> memo_;
+};
+
+// Evaluates the fields of the graph's result tuple one by one; a field that needs an operator
+// without a backend is skipped if `allow_partial`, else the error goes up.
+void RunGraph(rafhip_raf_env* env, const std::map<const ir::ExprNode*, value::Value>& bindings, bool make,
+              bool allow_partial, void* workspace, int64_t workspace_bytes) {
+  GraphRunner runner(env, bindings, make, static_cast<char*>(workspace), workspace_bytes);
+  const auto* result = ir::AsTupleNode(env->fused);
+  RAF_CHECK(result != nullptr, "the optimizer graph must end in a tuple");
+  for (const auto& field : result->fields) {
+    try {
+      runner.Eval(field);
+    } catch (const Unsupported&) {
+      if (!allow_partial) throw;
+    }
+  }
 }
 
 }  // namespace
@@ -551,6 +757,13 @@ int64_t rafhip_raf_pool_alloc_bytes(int32_t device_type, int32_t device_id, int6
 
 int64_t rafhip_raf_env_workspace_bytes(const rafhip_raf_env* env) {
   if (!env) return -1;
+  if (!env->graph_calls.empty()) {
+    int64_t total = 0;
+    for (const auto& gc : env->graph_calls)
+      if (gc.env)
+        for (const auto& r : gc.env->workspace_requests()) total += RoundUp(r.nbytes);
+    return total;
+  }
   if (!env->env) return 0;
   int64_t need = 0;
   for (const auto& r : env->env->workspace_requests()) need += RoundUp(r.nbytes);
@@ -611,6 +824,129 @@ int rafhip_raf_traced_sgd_execute(rafhip_raf_env* env, const rafhip_tensor_desc*
     WorkspaceBinding bind(env->env.get(), nullptr, 0);
     // the executors hand a fused function all of its arguments (arg_indices covers them all)
     env->env->Execute(call->args_as<schema::ListArgs>()->args, call->out);
+  });
+}
+
+namespace {
+// Binds the descriptor lists of a traced-optimizer call to the graph's variables (same order as at
+// make time) and returns the bindings.
+std::map<const ir::ExprNode*, value::Value> BindLists(const rafhip_raf_env* env, int32_t n,
+                                                      const rafhip_tensor_desc* const* lists, int n_lists,
+                                                      const rafhip_tensor_desc* step) {
+  std::map<const ir::ExprNode*, value::Value> bindings;
+  size_t next = 0;
+  for (int l = 0; l < n_lists; ++l) {
+    const size_t count = env->var_counts.at((size_t)l);
+    if (count == 0) continue;
+    RAF_CHECK(lists[l] != nullptr && (size_t)n == count, "a tensor list is missing or has another length than at make time");
+    for (size_t i = 0; i < count; ++i) bindings[env->vars.at(next++).get()] = FromDesc(&lists[l][i], "tensor list");
+  }
+  if (env->var_counts.size() > (size_t)n_lists && env->var_counts[(size_t)n_lists] == 1) {
+    RAF_CHECK(step != nullptr, "the step tensor is missing");
+    bindings[env->vars.at(next++).get()] = FromDesc(step, "step");
+  }
+  return bindings;
+}
+}  // namespace
+
+int rafhip_raf_traced_optimizer_make(int32_t kind, int32_t n, const rafhip_tensor_desc* g,
+                                     const rafhip_tensor_desc* w, const rafhip_tensor_desc* m,
+                                     const rafhip_tensor_desc* v, const rafhip_tensor_desc* p,
+                                     const rafhip_tensor_desc* step, int32_t zero_is_constant,
+                                     const double* hyper, int32_t n_hyper, int32_t allow_partial,
+                                     rafhip_raf_env** env_out) {
+  return Guard([&] {
+    if (!env_out) throw Error("rafhip_raf_traced_optimizer_make: env_out is NULL");
+    *env_out = nullptr;
+    if (kind != 0 && kind != 1) throw Error("rafhip_raf_traced_optimizer_make: kind must be 0 (SGD) or 1 (LANS)");
+    if (n <= 0 || !g || !w || !v) throw Error("rafhip_raf_traced_optimizer_make: bad tensor lists");
+    if (kind == 1 && (!m || !p || !step)) throw Error("rafhip_raf_traced_optimizer_make: LANS needs m, p and step");
+    if (!hyper || n_hyper != (kind == 0 ? 2 : 9))
+      throw Error("rafhip_raf_traced_optimizer_make: SGD takes 2 hyper-parameters, LANS 9");
+    std::unique_ptr<rafhip_raf_env> h(new rafhip_raf_env());
+    h->kind = kind;
+    const rafhip_tensor_desc* lists[5] = {g, w, kind == 1 ? m : nullptr, v, p};
+    const char* names[5] = {"g", "w", "m", "v", "p"};
+    std::vector<ir::Expr> vars[5];
+    for (int l = 0; l < 5; ++l) {
+      h->var_counts.push_back(lists[l] ? (size_t)n : 0);
+      for (int32_t i = 0; lists[l] && i < n; ++i) {
+        value::TensorValue t = FromDesc(&lists[l][i], names[l]);
+        ir::TensorType ty;
+        ty.defined = true;
+        ty.shape = t->tensor.shape;
+        ty.dtype = t->tensor.dtype;
+        vars[l].push_back(ir::MakeVar(std::string(names[l]) + std::to_string(i), ty));
+        h->vars.push_back(vars[l].back());
+      }
+    }
+    const Device device = FromDesc(&w[0], "w")->tensor.device;
+    ir::Expr zero;
+    if (p) {
+      ir::TensorType zt;
+      zt.defined = true;
+      zt.dtype = ir::TypeOf(vars[4][0]).dtype;
+      // as traced the optimizer's zero tensor is one more input of the function; bound as a
+      // constant it is a zeros constant (it then needs no storage: nothing is left to read it)
+      zero = zero_is_constant ? ir::MakeZeros(zt) : ir::MakeVar("zero", zt);
+    }
+    if (kind == 0) {
+      h->var_counts.push_back(0);
+      h->traced = hip::TracedSgdOptimizer(vars[1], vars[0], vars[3], vars[4], zero, hyper[0], hyper[1]);
+    } else {
+      value::TensorValue st = FromDesc(step, "step");
+      ir::TensorType sty;
+      sty.defined = true;
+      sty.shape = st->tensor.shape;
+      sty.dtype = st->tensor.dtype;
+      ir::Expr step_var = ir::MakeVar("step", sty);
+      h->vars.push_back(step_var);
+      h->var_counts.push_back(1);
+      hip::LansHyper hy;
+      hy.learning_rate = hyper[0];
+      hy.beta1 = hyper[1];
+      hy.beta2 = hyper[2];
+      hy.eps = hyper[3];
+      hy.bias_correction = (int)hyper[4];
+      hy.weight_decay = hyper[5];
+      hy.grad_averaging = (int)hyper[6];
+      hy.mode = (int)hyper[7];
+      hy.normalize_grad = (int)hyper[8];
+      h->traced = hip::TracedLansOptimizer(vars[0], vars[1], vars[2], vars[3], vars[4], zero, step_var, hy);
+    }
+    h->fused = pass::FuseDialect(h->traced, device.device_type());
+    h->call = std::make_shared<CallValuesNode>();
+    h->call->device = device;
+    h->op = kind == 0 ? "traced SGD optimizer" : "traced LANS optimizer";
+    h->name = h->op;
+    const rafhip_tensor_desc* all[5] = {g, w, kind == 1 ? m : nullptr, v, p};
+    *env_out = h.get();  // kept on failure too: it still holds the graphs for rafhip_raf_env_ir_text
+    rafhip_raf_env* raw = h.release();
+    RunGraph(raw, BindLists(raw, n, all, 5, step), /*make=*/true, allow_partial != 0, nullptr, 0);
+  });
+}
+
+int rafhip_raf_traced_optimizer_execute(rafhip_raf_env* env, int32_t n, const rafhip_tensor_desc* g,
+                                        const rafhip_tensor_desc* w, const rafhip_tensor_desc* m,
+                                        const rafhip_tensor_desc* v, const rafhip_tensor_desc* p,
+                                        const rafhip_tensor_desc* step, int32_t allow_partial,
+                                        void* workspace, int64_t workspace_bytes, void* stream) {
+  return Guard([&] {
+    if (!env || env->kind < 0) throw Error("rafhip_raf_traced_optimizer_execute: env was not made by rafhip_raf_traced_optimizer_make");
+    const rafhip_tensor_desc* all[5] = {g, w, env->kind == 1 ? m : nullptr, v, p};
+    auto bindings = BindLists(env, n, all, 5, step);
+    OpEnv::SetStreamForAllBackends(env->call->device, stream);
+    RunGraph(env, bindings, /*make=*/false, allow_partial != 0, workspace, workspace_bytes);
+  });
+}
+
+int rafhip_raf_env_graph_ops(const rafhip_raf_env* env, char* buf, int32_t buflen) {
+  return Guard([&] {
+    if (!env || !buf || buflen <= 0) throw Error("rafhip_raf_env_graph_ops: bad arguments");
+    std::string s;
+    for (const auto& gc : env->graph_calls) s += (s.empty() ? "" : ";") + gc.what;
+    if ((int64_t)s.size() >= (int64_t)buflen) throw Error("rafhip_raf_env_graph_ops: buffer too small");
+    std::memcpy(buf, s.c_str(), s.size() + 1);
   });
 }
 

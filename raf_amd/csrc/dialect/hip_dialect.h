@@ -56,6 +56,34 @@ constexpr int kSgdUpdatePatternPlevel = 60;  // above every pattern of the refer
 ir::Expr TracedSgdUpdate(const ir::Expr& w, const ir::Expr& dx, const ir::Expr& v,
                          double learning_rate, double momentum);
 
+// The optimizer part of the function that the reference's traced SGD optimizer builds for a model
+// with n parameters (python/raf/optim/sgd.py:187-215): TracedSgdUpdate for every parameter and,
+// when `p` is not empty (a half-precision model with fp32 master weights), the cast to the model's
+// dtype and the copy `add(new_w, zero, out=p)` behind it.  The result is the tuple of the n new
+// model weights.  `zero` is the optimizer's zero tensor: a variable as traced, or a zeros constant
+// once the model's constant attributes are bound into the graph.
+ir::Expr TracedSgdOptimizer(const std::vector<ir::Expr>& w, const std::vector<ir::Expr>& dx,
+                            const std::vector<ir::Expr>& v, const std::vector<ir::Expr>& p,
+                            const ir::Expr& zero, double learning_rate, double momentum);
+
+// Hyper-parameters of raf.op.lans in schema order (scripts/src_codegen/def_schema.py:685-693).
+struct LansHyper {
+  double learning_rate = 1e-3, beta1 = 0.9, beta2 = 0.999, eps = 1e-6;
+  int bias_correction = 1;
+  double weight_decay = 0.01;
+  int grad_averaging = 1, mode = 1, normalize_grad = 1;
+};
+
+// The optimizer part of what the reference's traced LANS optimizer builds for a half-precision
+// model (python/raf/optim/lans.py:244-312): group_cast of the n gradients to float32, raf.op.lans
+// over [g32..., w..., m..., v...], and per parameter cast(new_w, dtype) and add(_, zero, out=p).
+// The result is the tuple (new model weights..., new m..., new v...).  The increment of the step
+// counter in front of it (lans.py:240, a scalar add) is left out: `step` is passed as it is.
+ir::Expr TracedLansOptimizer(const std::vector<ir::Expr>& g, const std::vector<ir::Expr>& w,
+                             const std::vector<ir::Expr>& m, const std::vector<ir::Expr>& v,
+                             const std::vector<ir::Expr>& p, const ir::Expr& zero, const ir::Expr& step,
+                             const LansHyper& hyper);
+
 }  // namespace hip
 }  // namespace op
 }  // namespace raf

@@ -42,6 +42,40 @@ Expr MakeString(const std::string& v) {
   return n;
 }
 
+Expr MakeZeros(const TensorType& type) {
+  RAF_CHECK(type.defined, "a zeros constant needs a type");
+  auto n = std::make_shared<ConstantNode>();
+  n->value_kind = ConstantNode::kZeros;
+  n->type = type;
+  return n;
+}
+
+Expr MakeTuple(std::vector<Expr> fields) {
+  for (const auto& f : fields) RAF_CHECK(f != nullptr, "undefined tuple field");
+  auto n = std::make_shared<TupleNode>();
+  n->fields = std::move(fields);
+  return n;
+}
+
+Expr MakeTupleGetItem(const Expr& tuple, int index) {
+  RAF_CHECK(tuple != nullptr && index >= 0, "TupleGetItem needs a tuple and a non-negative index");
+  if (const auto* t = AsTupleNode(tuple))
+    RAF_CHECK((size_t)index < t->fields.size(), "TupleGetItem: index out of range");
+  auto n = std::make_shared<TupleGetItemNode>();
+  n->tuple = tuple;
+  n->index = index;
+  return n;
+}
+
+Expr MakeTupleCall(const Expr& op, std::vector<Expr> args, std::vector<TensorType> field_types) {
+  RAF_CHECK(AsOp(op) || AsFunction(op), "the callee must be an operator or a function");
+  auto n = std::make_shared<CallNode>();
+  n->op = op;
+  n->args = std::move(args);
+  n->field_types = std::move(field_types);
+  return n;
+}
+
 Expr GetOp(const std::string& name) {
   static std::mutex mu;
   static std::map<std::string, Expr> ops;
@@ -76,7 +110,93 @@ Expr MakeFunction(std::vector<Expr> params, const Expr& body,
 TensorType TypeOf(const Expr& e) {
   if (const auto* v = AsVar(e)) return v->type;
   if (const auto* c = AsCall(e)) return c->type;
+  if (const auto* k = AsConstant(e)) return k->value_kind == ConstantNode::kZeros ? k->type : TensorType();
+  if (const auto* g = AsTupleGetItem(e)) {
+    if (const auto* t = AsTupleNode(g->tuple))
+      return (size_t)g->index < t->fields.size() ? TypeOf(t->fields[(size_t)g->index]) : TensorType();
+    if (const auto* c = AsCall(g->tuple))
+      return (size_t)g->index < c->field_types.size() ? c->field_types[(size_t)g->index] : TensorType();
+  }
   return TensorType();
+}
+
+namespace {
+void PostOrderVisit(const Expr& e, std::set<const ExprNode*>* seen, std::vector<Expr>* out) {
+  if (!e || !seen->insert(e.get()).second) return;
+  if (const auto* c = AsCall(e)) {
+    PostOrderVisit(c->op, seen, out);
+    for (const auto& a : c->args) PostOrderVisit(a, seen, out);
+  } else if (const auto* f = AsFunction(e)) {
+    for (const auto& p : f->params) PostOrderVisit(p, seen, out);
+    PostOrderVisit(f->body, seen, out);
+  } else if (const auto* t = AsTupleNode(e)) {
+    for (const auto& x : t->fields) PostOrderVisit(x, seen, out);
+  } else if (const auto* g = AsTupleGetItem(e)) {
+    PostOrderVisit(g->tuple, seen, out);
+  }
+  out->push_back(e);
+}
+
+class Substituter {
+ public:
+  explicit Substituter(const std::map<const ExprNode*, Expr>& replace) : replace_(replace) {}
+  Expr Mutate(const Expr& e) {
+    if (!e) return e;
+    auto r = replace_.find(e.get());
+    if (r != replace_.end()) return r->second;
+    auto it = memo_.find(e.get());
+    if (it != memo_.end()) return it->second;
+    Expr post = e;
+    if (const auto* c = AsCall(e)) {
+      Expr op = Mutate(c->op);
+      bool changed = op.get() != c->op.get();
+      std::vector<Expr> args;
+      for (const auto& a : c->args) {
+        args.push_back(Mutate(a));
+        changed = changed || args.back().get() != a.get();
+      }
+      if (changed) {
+        auto n = std::make_shared<CallNode>();
+        n->op = op;
+        n->args = std::move(args);
+        n->type = c->type;
+        n->field_types = c->field_types;
+        post = n;
+      }
+    } else if (const auto* t = AsTupleNode(e)) {
+      bool changed = false;
+      std::vector<Expr> fields;
+      for (const auto& x : t->fields) {
+        fields.push_back(Mutate(x));
+        changed = changed || fields.back().get() != x.get();
+      }
+      if (changed) post = MakeTuple(std::move(fields));
+    } else if (const auto* g = AsTupleGetItem(e)) {
+      Expr tuple = Mutate(g->tuple);
+      if (tuple.get() != g->tuple.get()) post = MakeTupleGetItem(tuple, g->index);
+    } else if (const auto* f = AsFunction(e)) {
+      Expr body = Mutate(f->body);
+      if (body.get() != f->body.get()) post = MakeFunction(f->params, body, f->attrs);
+    }
+    memo_[e.get()] = post;
+    return post;
+  }
+
+ private:
+  const std::map<const ExprNode*, Expr>& replace_;
+  std::map<const ExprNode*, Expr> memo_;
+};
+}  // namespace
+
+std::vector<Expr> PostOrder(const Expr& root) {
+  std::set<const ExprNode*> seen;
+  std::vector<Expr> out;
+  PostOrderVisit(root, &seen, &out);
+  return out;
+}
+
+Expr Substitute(const Expr& root, const std::map<const ExprNode*, Expr>& replace) {
+  return Substituter(replace).Mutate(root);
 }
 
 // --------------------------------------------------------------------------------------- text
@@ -107,6 +227,8 @@ std::string ConstantText(const ConstantNode* c) {
     }
     case ConstantNode::kInt:
       return std::to_string(c->i) + "i64";
+    case ConstantNode::kZeros:
+      return "zeros(" + TypeText(c->type) + ")";
     default:
       return "\"" + c->s + "\"";
   }
@@ -145,6 +267,15 @@ class Printer {
       os_ << ")";
       if (call->type.defined) os_ << " /* ty=" << TypeText(call->type) << " */";
       os_ << ";\n";
+    } else if (const auto* t = AsTupleNode(e)) {
+      std::vector<std::string> fields;
+      for (const auto& x : t->fields) fields.push_back(Ref(x, depth));
+      name = "%" + std::to_string(n_values_++);
+      os_ << Indent(depth) << name << " = (";
+      for (size_t i = 0; i < fields.size(); ++i) os_ << (i ? ", " : "") << fields[i];
+      os_ << (fields.size() == 1 ? ",)" : ")") << ";\n";
+    } else if (const auto* g = AsTupleGetItem(e)) {
+      return Ref(g->tuple, depth) + "." + std::to_string(g->index);  // printed in place
     } else {
       const auto* f = AsFunction(e);
       name = "%fn" + std::to_string(n_funcs_++);
@@ -183,6 +314,8 @@ bool SameConstant(const ConstantNode* a, const ConstantNode* b) {
       return a->f == b->f;
     case ConstantNode::kInt:
       return a->i == b->i;
+    case ConstantNode::kZeros:
+      return SameType(a->type, b->type);
     default:
       return a->s == b->s;
   }
@@ -217,6 +350,17 @@ class Equal {
         ok = fa->params.size() == fb->params.size() && fa->attrs == fb->attrs;
         for (size_t i = 0; ok && i < fa->params.size(); ++i) ok = Check(fa->params[i], fb->params[i]);
         ok = ok && Check(fa->body, fb->body);
+        break;
+      }
+      case ExprNode::kTuple: {
+        const auto *ta = AsTupleNode(a), *tb = AsTupleNode(b);
+        ok = ta->fields.size() == tb->fields.size();
+        for (size_t i = 0; ok && i < ta->fields.size(); ++i) ok = Check(ta->fields[i], tb->fields[i]);
+        break;
+      }
+      case ExprNode::kTupleGetItem: {
+        const auto *ga = AsTupleGetItem(a), *gb = AsTupleGetItem(b);
+        ok = ga->index == gb->index && Check(ga->tuple, gb->tuple);
         break;
       }
     }
@@ -383,7 +527,14 @@ class Rewriter {
         args.push_back(Mutate(a));
         changed = changed || args.back().get() != a.get();
       }
-      if (changed) post = MakeCall(op, args, c->type);
+      if (changed) {
+        auto n = std::make_shared<CallNode>();
+        n->op = op;
+        n->args = args;
+        n->type = c->type;
+        n->field_types = c->field_types;
+        post = n;
+      }
       origin_[post.get()] = e.get();
       NodeMap node_map;
       if (MatchPattern(pattern_, post, &node_map) && InteriorIsPrivate(post, node_map))
@@ -393,6 +544,17 @@ class Rewriter {
         Expr body = Mutate(f->body);
         if (body.get() != f->body.get()) post = MakeFunction(f->params, body, f->attrs);
       }
+    } else if (const auto* t = AsTupleNode(e)) {
+      bool changed = false;
+      std::vector<Expr> fields;
+      for (const auto& x : t->fields) {
+        fields.push_back(Mutate(x));
+        changed = changed || fields.back().get() != x.get();
+      }
+      if (changed) post = MakeTuple(std::move(fields));
+    } else if (const auto* g = AsTupleGetItem(e)) {
+      Expr tuple = Mutate(g->tuple);
+      if (tuple.get() != g->tuple.get()) post = MakeTupleGetItem(tuple, g->index);
     }
     memo_[e.get()] = post;
     keep_alive_.push_back(e);
@@ -412,6 +574,14 @@ class Rewriter {
     } else if (const auto* f = AsFunction(e)) {
       ++uses_[f->body.get()];
       CountUses(f->body);
+    } else if (const auto* t = AsTupleNode(e)) {
+      for (const auto& x : t->fields) {
+        ++uses_[x.get()];
+        CountUses(x);
+      }
+    } else if (const auto* g = AsTupleGetItem(e)) {
+      ++uses_[g->tuple.get()];
+      CountUses(g->tuple);
     }
   }
 
@@ -490,6 +660,30 @@ void DialectFusePattern::AddPattern(const ir::DFPattern& pattern, const std::str
   for (; it != list->end(); ++it) {
     RAF_CHECK(plevel != it->plevel, "InternalError: dialect pattern with plevel " +
                                         std::to_string(plevel) + " is already registered");
+    if (plevel > it->plevel) break;
+  }
+  list->insert(it, entry);
+}
+
+std::list<DialectGraphRewrite>* DialectGraphRewrite::Get() {
+  static std::list<DialectGraphRewrite> rewrites;
+  return &rewrites;
+}
+
+void DialectGraphRewrite::Add(const std::string& dialect, int plevel, const std::string& name, Fn fn) {
+  static std::mutex mu;
+  std::lock_guard<std::mutex> lock(mu);
+  auto* list = Get();
+  DialectGraphRewrite entry;
+  entry.dialect = dialect;
+  entry.plevel = plevel;
+  entry.name = name;
+  entry.fn = std::move(fn);
+  auto it = list->begin();
+  for (; it != list->end(); ++it) {
+    RAF_CHECK(!(plevel == it->plevel && dialect == it->dialect),
+              "InternalError: dialect " + dialect + " already has a graph rewrite with plevel " +
+                  std::to_string(plevel));
     if (plevel > it->plevel) break;
   }
   list->insert(it, entry);
@@ -645,6 +839,9 @@ class FuseMutator {
 ir::Expr FuseDialect(const ir::Expr& expr, DevType device_type) {
   if (device_type == DevType::kUnknown()) return expr;  // the reference warns and skips the pass
   Expr ret = expr;
+  const std::list<op::DialectGraphRewrite> rewrites = *op::DialectGraphRewrite::Get();
+  for (const auto& rw : rewrites)
+    if (op::Dialect::IsEnabled(rw.dialect, device_type)) ret = rw.fn(ret);
   // A snapshot: makers may not register patterns while the pass runs.
   const op::DialectFusePattern::PatternList patterns = *op::DialectFusePattern::Get();
   for (const auto& pat : patterns) {

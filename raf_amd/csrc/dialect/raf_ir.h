@@ -41,7 +41,7 @@ struct TensorType {
 };
 
 struct ExprNode {
-  enum Kind { kVar, kConstant, kOp, kCall, kFunction };
+  enum Kind { kVar, kConstant, kOp, kCall, kFunction, kTuple, kTupleGetItem };
   explicit ExprNode(Kind k) : kind(k) {}
   virtual ~ExprNode() = default;
   const Kind kind;
@@ -53,14 +53,17 @@ struct VarNode : ExprNode {
   TensorType type;
 };
 
-// A constant holds a value: null (the reference's `const(None)`), a float, an integer or a string.
+// A constant holds a value: null (the reference's `const(None)`), a float, an integer, a string,
+// or a tensor all of whose elements are zero (what binding a model's constant attribute such as
+// `self.zero` and folding constants leaves in the graph; only its type matters to a pass).
 struct ConstantNode : ExprNode {
-  enum ValueKind { kNull, kFloat, kInt, kString };
+  enum ValueKind { kNull, kFloat, kInt, kString, kZeros };
   ConstantNode() : ExprNode(kConstant) {}
   ValueKind value_kind = kNull;
   double f = 0.0;
   int64_t i = 0;
   std::string s;
+  TensorType type;  // kZeros
 };
 
 struct OpNode : ExprNode {
@@ -73,6 +76,20 @@ struct CallNode : ExprNode {
   Expr op;  // an OpNode or a FunctionNode
   std::vector<Expr> args;
   TensorType type;  // result type, when known
+  std::vector<TensorType> field_types;  // for a call that returns a tuple: its fields' types, when known
+};
+
+// Tuples: the tensor lists of the multi-tensor ops and the results of ops that return several
+// tensors (relay Tuple / TupleGetItem).
+struct TupleNode : ExprNode {
+  TupleNode() : ExprNode(kTuple) {}
+  std::vector<Expr> fields;
+};
+
+struct TupleGetItemNode : ExprNode {
+  TupleGetItemNode() : ExprNode(kTupleGetItem) {}
+  Expr tuple;
+  int index = 0;
 };
 
 struct FunctionNode : ExprNode {
@@ -91,6 +108,11 @@ Expr MakeNull();
 Expr MakeFloat(double v);
 Expr MakeInt(int64_t v);
 Expr MakeString(const std::string& v);
+Expr MakeZeros(const TensorType& type);
+Expr MakeTuple(std::vector<Expr> fields);
+Expr MakeTupleGetItem(const Expr& tuple, int index);
+// A call whose result is a tuple of tensors of the given types.
+Expr MakeTupleCall(const Expr& op, std::vector<Expr> args, std::vector<TensorType> field_types);
 Expr GetOp(const std::string& name);  // one node per operator name
 Expr MakeCall(const Expr& op, std::vector<Expr> args, const TensorType& type = TensorType());
 Expr MakeFunction(std::vector<Expr> params, const Expr& body,
@@ -105,9 +127,22 @@ inline const ConstantNode* AsConstant(const Expr& e) { return As<ConstantNode>(e
 inline const OpNode* AsOp(const Expr& e) { return As<OpNode>(e, ExprNode::kOp); }
 inline const CallNode* AsCall(const Expr& e) { return As<CallNode>(e, ExprNode::kCall); }
 inline const FunctionNode* AsFunction(const Expr& e) { return As<FunctionNode>(e, ExprNode::kFunction); }
+inline const TupleNode* AsTupleNode(const Expr& e) { return As<TupleNode>(e, ExprNode::kTuple); }
+inline const TupleGetItemNode* AsTupleGetItem(const Expr& e) {
+  return As<TupleGetItemNode>(e, ExprNode::kTupleGetItem);
+}
 
-// The type of a variable or call, undefined for everything else.
+// The type of a variable, a call that returns a tensor, a zeros constant, or a field taken from a
+// tuple or from a call that returns a tuple; undefined for everything else.
 TensorType TypeOf(const Expr& e);
+
+// Every expression reachable from `root` (function bodies included), each once, arguments before
+// the expressions that use them.
+std::vector<Expr> PostOrder(const Expr& root);
+
+// `root` rebuilt with every expression that is a key of `replace` swapped for its value (the
+// values are taken as they are, not rewritten again); untouched sub-graphs are shared.
+Expr Substitute(const Expr& root, const std::map<const ExprNode*, Expr>& replace);
 
 // Text form for messages and for the cache of fused functions; shared sub-expressions are bound
 // to %n names, so the text is linear in the size of the graph.
@@ -173,6 +208,24 @@ class DialectFusePattern {
                          const std::string& name = "");
 };
 
+// A rewrite of a whole graph on behalf of a dialect.  DialectFusePattern covers what a dataflow
+// pattern can say: a fixed number of calls under ONE root.  A multi-tensor optimizer step gathers a
+// variable number of per-parameter roots (every parameter's update, or every parameter's cast and
+// copy behind raf.op.lans) into one call that returns a tuple, which no such pattern expresses;
+// dialects register those as functions over the graph.  FuseDialect runs them, for the dialects
+// enabled on the device, in descending plevel order ahead of the patterns.  (Inside RAF proper
+// each is one more pass in front of FuseDialect in the pass sequence.)
+class DialectGraphRewrite {
+ public:
+  using Fn = std::function<ir::Expr(const ir::Expr&)>;
+  std::string dialect;
+  int plevel = 0;
+  std::string name;
+  Fn fn;
+  static std::list<DialectGraphRewrite>* Get();
+  static void Add(const std::string& dialect, int plevel, const std::string& name, Fn fn);
+};
+
 // The dialect op registered for `base_op` by `dialect` (an OpNode), or an empty Expr.
 ir::Expr LowerOp(const std::string& base_op, const std::string& dialect);
 
@@ -194,9 +247,9 @@ struct StringValueObj : value::ValueObj {
   std::string value;
 };
 
-// CallValues for `call`, whose callee is an operator or a primitive function: variables take
-// their values from `bindings`, constants become scalar values (null: an empty Value).  For a
-// function callee the arguments go into ListArgs and the function into call->closure.
+// CallValues for `call`, whose callee is a primitive function: variables take their values from
+// `bindings`, constants become scalar values (null: an empty Value).  The arguments go into
+// ListArgs and the function into call->closure.
 CallValues BindCall(const ir::Expr& call, const std::map<const ir::ExprNode*, value::Value>& bindings,
                     const Device& device);
 

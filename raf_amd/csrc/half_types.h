@@ -74,6 +74,16 @@ struct GradIO<float> {
 #pragma unroll
     for (int j = 0; j < kWide; ++j) out[j] = r[j] * us;
   }
+  // The wide access in two steps, so that many loads can be in flight before any is widened.
+  typedef f32x4 RawWide;
+  template <bool kNT>
+  static __device__ __forceinline__ RawWide load_raw_wide(const void* g, int iw) {
+    return ldg<kNT>((const RAFHIP_GLOBAL f32x4*)g + iw);
+  }
+  static __device__ __forceinline__ void widen_wide(const RawWide& r, float us, float (&out)[kWide]) {
+#pragma unroll
+    for (int j = 0; j < kWide; ++j) out[j] = r[j] * us;
+  }
   template <bool kNT>
   static __device__ __forceinline__ f32x4 load4(const void* g, int64_t i4, float us) {
     const f32x4 r = ldg<kNT>((const RAFHIP_GLOBAL f32x4*)g + i4);
@@ -103,6 +113,15 @@ struct GradIO<_Float16> {
 #pragma unroll
     for (int j = 0; j < kWide; ++j) out[j] = (float)r[j] * us;
   }
+  typedef f16x8 RawWide;
+  template <bool kNT>
+  static __device__ __forceinline__ RawWide load_raw_wide(const void* g, int iw) {
+    return ldg<kNT>((const RAFHIP_GLOBAL f16x8*)g + iw);
+  }
+  static __device__ __forceinline__ void widen_wide(const RawWide& r, float us, float (&out)[kWide]) {
+#pragma unroll
+    for (int j = 0; j < kWide; ++j) out[j] = (float)r[j] * us;
+  }
   template <bool kNT>
   static __device__ __forceinline__ f32x4 load4(const void* g, int64_t i4, float us) {
     const f16x4 r = ldg<kNT>((const RAFHIP_GLOBAL f16x4*)g + i4);
@@ -128,6 +147,15 @@ struct GradIO<Bf16> {
   static __device__ __forceinline__ void load_wide(const void* g, int iw, float us,
                                                    float (&out)[kWide]) {
     const u16x8 r = ldg<kNT>((const RAFHIP_GLOBAL u16x8*)g + iw);
+#pragma unroll
+    for (int j = 0; j < kWide; ++j) out[j] = bf16_widen(r[j]) * us;
+  }
+  typedef u16x8 RawWide;
+  template <bool kNT>
+  static __device__ __forceinline__ RawWide load_raw_wide(const void* g, int iw) {
+    return ldg<kNT>((const RAFHIP_GLOBAL u16x8*)g + iw);
+  }
+  static __device__ __forceinline__ void widen_wide(const RawWide& r, float us, float (&out)[kWide]) {
 #pragma unroll
     for (int j = 0; j < kWide; ++j) out[j] = bf16_widen(r[j]) * us;
   }

@@ -103,8 +103,13 @@ struct WorkItem {
   int32_t tensor;
   uint32_t chunk_phase;
 };
+// chunk_phase: [31..29] kind | [28] streaming | [27..0] chunk.
+//   streaming  the item belongs to a tensor too large for the Infinity Cache: all of its accesses
+//              carry the non-temporal hint, so that it flows past the cache without evicting the
+//              groups that live there between their passes.
 constexpr uint32_t kPhaseShift = 29;
-constexpr uint32_t kChunkMask = (1u << kPhaseShift) - 1;
+constexpr uint32_t kStreamBit = 1u << 28;
+constexpr uint32_t kChunkMask = kStreamBit - 1;
 
 // Global scalars of a step, produced on the device from the step tensor (256 bytes reserved).
 struct StepScalars {

@@ -39,6 +39,10 @@ constexpr CachePolicy kPhasedPolicy = {true, false, true, false, true, true};
 // kept) and writes non-temporally.  Measured best of nine combinations.
 constexpr CachePolicy kPipelinedPolicy = {false, true, false, true, true, true};
 constexpr bool kPipelinedAhead = true;  // issue the next trip's loads before evaluating this one
+#ifndef RAFHIP_PIPELINED_A_UNROLL
+#define RAFHIP_PIPELINED_A_UNROLL 8
+#endif
+constexpr int kPipelinedAUnroll = RAFHIP_PIPELINED_A_UNROLL;
 // Lists whose whole working set fits in the cache (a few million elements) are better off cached.
 constexpr CachePolicy kResidentPolicy = {false, false, false, false, false, false};
 
@@ -290,29 +294,30 @@ __device__ __forceinline__ ChunkView chunk_view(const TensorRec& tr, uint32_t ch
 // ------------------------------------------------------------------ pass A on one chunk
 // Per-thread contribution to sum g^2 (block reduction is the caller's).  Only the gradient is read:
 // ||w|| is not needed before the trust ratios, so its sum rides along with pass B.
-template <typename G, bool kNT>
+// kU: 16-byte accesses in flight per lane per trip.  A lane adds its elements in ascending order
+// whatever kU is, so the sum does not depend on it.
+template <typename G, bool kNT, int kU = 4>
 __device__ __forceinline__ double chunk_sum_g(const ChunkView& cv, float unscale) {
   constexpr int kW = GradIO<G>::kWide;  // elements per 16-byte lane access
-  constexpr int kU = 4;                 // accesses in flight per lane per trip
   double acc[4] = {0.0, 0.0, 0.0, 0.0};
   if (cv.vec_ok) {
     const int nw = cv.len / kW;
     for (int i0 = threadIdx.x; i0 < nw; i0 += kLansBlock * kU) {
-      float x[kU][kW];
+      typename GradIO<G>::RawWide raw[kU];
 #pragma unroll
       for (int u = 0; u < kU; ++u) {
         const int i = i0 + u * kLansBlock;
-        if (i < nw) {
-          GradIO<G>::template load_wide<kNT>(cv.g, i, unscale, x[u]);
-        } else {
-#pragma unroll
-          for (int j = 0; j < kW; ++j) x[u][j] = 0.f;
-        }
+        if (i < nw) raw[u] = GradIO<G>::template load_raw_wide<kNT>(cv.g, i);
       }
 #pragma unroll
-      for (int u = 0; u < kU; ++u)
+      for (int u = 0; u < kU; ++u) {
+        if (i0 + u * kLansBlock < nw) {
+          float x[kW];
+          GradIO<G>::widen_wide(raw[u], unscale, x);
 #pragma unroll
-        for (int j = 0; j < kW; ++j) acc[j & 3] = __builtin_fma((double)x[u][j], (double)x[u][j], acc[j & 3]);
+          for (int j = 0; j < kW; ++j) acc[j & 3] = __builtin_fma((double)x[j], (double)x[j], acc[j & 3]);
+        }
+      }
     }
     const int tail = nw * kW + threadIdx.x;  // the < kW leftover elements of a last chunk
     if (tail < cv.len) {
@@ -811,6 +816,7 @@ __global__ __launch_bounds__(kLansBlock) void lans_pipelined(LansDeviceArgs a) {
     const int t = it.tensor;
     const uint32_t phase = it.chunk_phase >> kPhaseShift;
     const uint32_t chunk = it.chunk_phase & kChunkMask;
+    const bool streaming = (it.chunk_phase & kStreamBit) != 0;  // uniform, like everything read off the item
     const bool unit_a = phase == kPhaseA;  // pass-A items count in units of kChunksPerA chunks
     const ChunkView cv = chunk_view(tr, chunk, (int)sizeof(G), unit_a ? kChunksPerA : 1);
     const int64_t n_chunks = chunks_of(tr);
@@ -820,7 +826,13 @@ __global__ __launch_bounds__(kLansBlock) void lans_pipelined(LansDeviceArgs a) {
     TensorStats* st = &a.stats[t];
 
     if (phase == kPhaseA) {
-      double s[1] = {chunk_sum_g<G, kPipelinedPolicy.a_g>(cv, unscale)};
+      double s[1];
+      // Three workgroups per CU have to keep the gradient stream busy on their own here: twice
+      // the accesses in flight of the one-launch-per-pass kernel, which runs five.
+      if (streaming)
+        s[0] = chunk_sum_g<G, true, kPipelinedAUnroll>(cv, unscale);
+      else
+        s[0] = chunk_sum_g<G, kPipelinedPolicy.a_g, kPipelinedAUnroll>(cv, unscale);
       block_sum<1>(s, red);
       if (threadIdx.x == 0) publish(part, s[0]);
     } else if (phase == kPhaseFinishA) {
@@ -835,11 +847,15 @@ __global__ __launch_bounds__(kLansBlock) void lans_pipelined(LansDeviceArgs a) {
     } else if (phase == kPhaseB) {
       double s[3];
       bool lost = false;  // this thread's divisor never arrived
-      chunk_sums_u<G, kPipelinedPolicy.b_g, kPipelinedPolicy.b_wmv, kPipelinedAhead>(cv, unscale, k, [&] {
+      auto divisor = [&] {
         const double d = wait_published(&st->inv_grad_div, wc);
         lost = is_lost(d);
         return d;
-      }, s);
+      };
+      if (streaming)
+        chunk_sums_u<G, true, true, kPipelinedAhead>(cv, unscale, k, divisor, s);
+      else
+        chunk_sums_u<G, kPipelinedPolicy.b_g, kPipelinedPolicy.b_wmv, kPipelinedAhead>(cv, unscale, k, divisor, s);
       const bool any_lost = block_sum<3, true>(s, red, lost);
       if (threadIdx.x == 0) {
         if (any_lost) {
@@ -862,13 +878,17 @@ __global__ __launch_bounds__(kLansBlock) void lans_pipelined(LansDeviceArgs a) {
           stats_after_b(st, tot, k, r0, r1);
       }
     } else if (phase == kPhaseC) {
-      chunk_apply<G, kPipelinedPolicy.c_g, kPipelinedPolicy.c_wmv, kPipelinedPolicy.c_stores, kPipelinedAhead>(
-          cv, unscale, a.p_is_bf16 != 0, k, [&] {
+      auto params = [&] {
         const double* const words[3] = {&st->inv_grad_div, &st->ratio_m, &st->ratio_g};
         double val[3];
         wait_published_n<3>(words, val, wc);
         return ApplyParams{val[0], val[1], val[2], !(is_lost(val[0]) || is_lost(val[1]) || is_lost(val[2]))};
-      });
+      };
+      if (streaming)
+        chunk_apply<G, true, true, true, kPipelinedAhead>(cv, unscale, a.p_is_bf16 != 0, k, params);
+      else
+        chunk_apply<G, kPipelinedPolicy.c_g, kPipelinedPolicy.c_wmv, kPipelinedPolicy.c_stores, kPipelinedAhead>(
+            cv, unscale, a.p_is_bf16 != 0, k, params);
     } else {
       // A one-chunk tensor: all three passes here, no other workgroup involved.  The totals equal
       // the single chunk partials, exactly as the general path computes them, and travel between

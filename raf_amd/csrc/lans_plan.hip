@@ -77,32 +77,98 @@ int round_slices_setting() {
   return kDefaultRoundSlices;
 }
 
-inline WorkItem make_item(int32_t tensor, uint32_t phase, int64_t chunk) {
-  return WorkItem{tensor, (phase << kPhaseShift) | (uint32_t)chunk};
+int env_count(const char* name, int fallback) {
+  if (const char* e = std::getenv(name)) {
+    const int v = std::atoi(e);
+    if (v >= 0) return v;
+  }
+  return fallback;
 }
 
-// The pipelined work list.  Tensors are packed, in list order, into groups of at most group_elems
-// elements (a larger tensor is a group of its own).  "Round" r holds pass A of group r, then pass
-// B of group r-1 and pass C of group r-2 in alternating slices.  (Merging all three so that they
-// advance together was measured too: items then sit right behind the ones they depend on and the
-// kernel waits more.)
-// Invariant the kernel's waits rely on, per tensor: pass-A chunks, then its finish-A item, then
+inline WorkItem make_item(int32_t tensor, uint32_t phase, int64_t chunk, uint32_t flags = 0) {
+  return WorkItem{tensor, (phase << kPhaseShift) | flags | (uint32_t)chunk};
+}
+
+// A tensor whose w, m, v alone exceed the 256 MB Infinity Cache cannot keep anything there between
+// its passes; handled like the others it would only flush the groups that can.
+constexpr int64_t kStreamedTensorFromElems = (256LL << 20) / 12;
+int64_t streamed_from_setting() {
+  if (const char* e = std::getenv("RAFHIP_LANS_STREAM_FROM_ELEMS")) {
+    const long long v = std::atoll(e);
+    if (v > 0) return v;
+  }
+  return kStreamedTensorFromElems;
+}
+
+// Resident workgroups of the persistent kernel on a 256-CU device, for the host-only queries.
+constexpr int kDefaultPipelineGrid = 256 * 3;
+
+// The pipelined work list.
+//
+// Cached groups.  Tensors are packed, in list order, into groups of at most group_elems elements.
+// "Round" r holds pass A of group r, then pass B of group r-1 and pass C of group r-2 in
+// alternating slices, so that a group's gradient survives in the cache from pass A to pass B and
+// its w, m, v from pass B to pass C.  (Merging all three so that they advance together was
+// measured too: items then sit right behind the ones they depend on and the kernel waits more.)
+//
+// Streamed tensors.  A tensor too large for the cache forms no group.  Its three passes depend on
+// each other as a whole, so on its own it would run them one after the other, each bound by HBM
+// alone while the cache and the rest of the fabric idle -- at the head of a BERT list (the word
+// embedding comes first) that was a tenth of the step.  Its items are marked streaming and spread
+// over the whole list of rounds in proportion to the bytes they move: the tensor then trickles
+// through HBM underneath the cached groups' traffic.
+//
+// Invariant the kernel's waits rely on, per tensor: pass-A units, then its finish-A item, then
 // pass-B chunks, then its finish-B item, then pass-C chunks.
-std::vector<WorkItem> build_pipeline(int32_t n, const int64_t* numel, int64_t group_elems) {
+std::vector<WorkItem> build_pipeline(int32_t n, const int64_t* numel, int64_t group_elems,
+                                     int grid = kDefaultPipelineGrid) {
   struct Group {
     std::vector<WorkItem> a, b, c;
   };
   std::vector<Group> groups;
-  int64_t in_group = 0;
+  std::vector<WorkItem> streamed;  // every streamed tensor: A units, finish A, B chunks, finish B, C chunks
+  std::vector<int64_t> streamed_bytes;  // what each of those items moves (for the proportional merge)
+  const bool stream_large = std::getenv("RAFHIP_LANS_NO_STREAMED_TENSORS") == nullptr;
+  const int64_t stream_from = streamed_from_setting();
+  std::vector<int32_t> cached_tensors;
   for (int32_t t = 0; t < n; ++t) {
     if (numel[t] == 0) continue;
+    const int64_t nc = chunks_of(numel[t]);
+    const int64_t ce = chunk_elems_for(numel[t]);
+    if (stream_large && numel[t] >= stream_from) {
+      auto len_of = [&](int64_t idx, int64_t unit) { return std::min(unit, numel[t] - idx * unit); };
+      for (int64_t u = 0; u < units_a_of(numel[t]); ++u) {
+        streamed.push_back(make_item(t, kPhaseA, u, kStreamBit));
+        streamed_bytes.push_back(4 * len_of(u, ce * kChunksPerA));
+      }
+      streamed.push_back(make_item(t, kPhaseFinishA, 0));
+      streamed_bytes.push_back(0);
+      for (int64_t c = 0; c < nc; ++c) {
+        streamed.push_back(make_item(t, kPhaseB, c, kStreamBit));
+        streamed_bytes.push_back(16 * len_of(c, ce));
+      }
+      streamed.push_back(make_item(t, kPhaseFinishB, 0));
+      streamed_bytes.push_back(0);
+      for (int64_t c = 0; c < nc; ++c) {
+        streamed.push_back(make_item(t, kPhaseC, c, kStreamBit));
+        streamed_bytes.push_back(28 * len_of(c, ce));
+      }
+      continue;
+    }
+    cached_tensors.push_back(t);
+  }
+
+  // (Small groups at either end, to fill and drain the pipeline faster, were measured and are
+  // slower: a short round puts pass-B items right behind the finish items they wait for.)
+  int64_t in_group = 0;
+  for (const int32_t t : cached_tensors) {
+    const int64_t nc = chunks_of(numel[t]);
     if (groups.empty() || (in_group > 0 && in_group + numel[t] > group_elems)) {
       groups.emplace_back();
       in_group = 0;
     }
     in_group += numel[t];
     Group& g = groups.back();
-    const int64_t nc = chunks_of(numel[t]);
     if (nc == 1) {
       g.a.push_back(make_item(t, kPhaseWhole, 0));  // one workgroup does all three passes
       continue;
@@ -115,7 +181,7 @@ std::vector<WorkItem> build_pipeline(int32_t n, const int64_t* numel, int64_t gr
     g.a.push_back(make_item(t, kPhaseFinishA, 0));  // after the tensor's chunks of the pass
     g.b.push_back(make_item(t, kPhaseFinishB, 0));
   }
-  std::vector<WorkItem> out;
+  std::vector<WorkItem> cached;
   const int64_t ng = (int64_t)groups.size();
   // Within a round, passes B and C alternate in slices: pass C then follows more closely behind
   // the pass B that loaded its group one round earlier, which shortens the time a group has to
@@ -126,10 +192,67 @@ std::vector<WorkItem> build_pipeline(int32_t n, const int64_t* numel, int64_t gr
   for (int64_t r = 0; r < ng + 2; ++r) {
     const std::vector<WorkItem>& b = (r >= 1 && r - 1 < ng) ? groups[r - 1].b : none;
     const std::vector<WorkItem>& c = (r >= 2 && r - 2 < ng) ? groups[r - 2].c : none;
-    if (r < ng) out.insert(out.end(), groups[r].a.begin(), groups[r].a.end());
+    if (r < ng) cached.insert(cached.end(), groups[r].a.begin(), groups[r].a.end());
     for (size_t k = 0; k < slices; ++k) {
-      out.insert(out.end(), b.begin() + b.size() * k / slices, b.begin() + b.size() * (k + 1) / slices);
-      out.insert(out.end(), c.begin() + c.size() * k / slices, c.begin() + c.size() * (k + 1) / slices);
+      cached.insert(cached.end(), b.begin() + b.size() * k / slices, b.begin() + b.size() * (k + 1) / slices);
+      cached.insert(cached.end(), c.begin() + c.size() * k / slices, c.begin() + c.size() * (k + 1) / slices);
+    }
+  }
+
+  // Merge the two streams so that each has moved the same share of its bytes at every point.
+  std::vector<WorkItem> out;
+  if (streamed.empty()) {
+    out.swap(cached);
+  } else if (cached.empty()) {
+    out.swap(streamed);
+  } else {
+    auto bytes_of = [&](const WorkItem& it) -> int64_t {
+      const int64_t ne = numel[it.tensor];
+      const int64_t ce = chunk_elems_for(ne);
+      const int64_t c = it.chunk_phase & kChunkMask;
+      switch (it.chunk_phase >> kPhaseShift) {
+        case kPhaseA: return 4 * std::min(ce * kChunksPerA, ne - c * ce * kChunksPerA);
+        case kPhaseB: return 16 * std::min(ce, ne - c * ce);
+        case kPhaseC: return 28 * std::min(ce, ne - c * ce);
+        case kPhaseWhole: return 48 * ne;
+        default: return 0;
+      }
+    };
+    const int hold_items = env_count("RAFHIP_LANS_STREAM_HOLD_ITEMS", 4 * grid);
+    double total_c = 0, total_s = 0;
+    for (const WorkItem& it : cached) total_c += (double)bytes_of(it);
+    for (int64_t b : streamed_bytes) total_s += (double)b;
+    if (total_c <= 0) total_c = 1;
+    if (total_s <= 0) total_s = 1;
+    out.reserve(cached.size() + streamed.size());
+    size_t i = 0, j = 0;
+    double left_c = total_c, left_s = total_s;  // bytes still to be placed
+    double base_c = total_c, base_s = total_s;  // ... when the pacing was last set
+    // What follows a finish item of the streamed tensor waits for it, and it waits for the last
+    // items of the pass before it, which have only just been drawn: the streamed stream pauses for
+    // a few items per workgroup of cached work, or most workgroups would sit in that wait.  After
+    // the pause the two streams are paced by what each has left, so that the streamed one does
+    // not catch up in one burst (which would be a stretch of pure HBM traffic again).
+    int64_t hold = 0;
+    while (i < cached.size() || j < streamed.size()) {
+      if (hold == 0) {
+        base_c = left_c > 0 ? left_c : 1;
+        base_s = left_s > 0 ? left_s : 1;
+        hold = -1;
+      }
+      const bool take_streamed =
+          j < streamed.size() &&
+          (i >= cached.size() || (hold < 0 && (base_s - left_s) / base_s <= (base_c - left_c) / base_c));
+      if (take_streamed) {
+        left_s -= (double)streamed_bytes[j];
+        const uint32_t kind = streamed[j].chunk_phase >> kPhaseShift;
+        if (kind == kPhaseFinishA || kind == kPhaseFinishB) hold = hold_items > 0 ? (int64_t)hold_items : 0;
+        out.push_back(streamed[j++]);
+      } else {
+        left_c -= (double)bytes_of(cached[i]);
+        if (hold > 0) --hold;
+        out.push_back(cached[i++]);
+      }
     }
   }
   return out;
@@ -271,7 +394,7 @@ int validate_list(const char* who, int32_t n_tensors, const int64_t* numel) {
     if (numel[t] < 0)
       return fail(RAFHIP_ERR_INVALID_ARG, "%s: numel[%d] = %lld < 0", who, t, (long long)numel[t]);
     chunks += chunks_of(numel[t]);
-    if (chunks >= (int64_t)kChunkMask / 4)
+    if (chunks >= (int64_t)kChunkMask)
       return fail(RAFHIP_ERR_UNSUPPORTED, "%s: too many chunks (more than 2^28)", who);
   }
   return RAFHIP_OK;
@@ -329,9 +452,10 @@ int rafhip_lans_pipeline_order(int32_t n_tensors, const int64_t* numel, int64_t 
         return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_pipeline_order: capacity %lld < %zu items",
                     (long long)capacity, items.size());
       for (size_t i = 0; i < items.size(); ++i) {
-        triples_out[3 * i + 0] = (int32_t)(items[i].chunk_phase >> kPhaseShift);
+        const uint32_t cp = items[i].chunk_phase;
+        triples_out[3 * i + 0] = (int32_t)(cp >> kPhaseShift) + ((cp & kStreamBit) ? 8 : 0);
         triples_out[3 * i + 1] = items[i].tensor;
-        triples_out[3 * i + 2] = (int32_t)(items[i].chunk_phase & kChunkMask);
+        triples_out[3 * i + 2] = (int32_t)(cp & kChunkMask);
       }
     }
     return RAFHIP_OK;
@@ -391,8 +515,6 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
       for (int32_t t = 0; t < n_tensors; ++t)
         for (int64_t u = 0; u < units_a_of(numel[t]); ++u) phased_a.push_back(make_item(t, kPhaseA, u));
       p->n_items_a = (int64_t)phased_a.size();
-      const std::vector<WorkItem> pipeline = build_pipeline(n_tensors, numel, group_elems_setting());
-      p->n_pipeline_items = (uint32_t)pipeline.size();
       // Resident workgroups per CU: never more than fit (every workgroup must be running), and by
       // default three: a larger window of in-flight items measured slower on MI355X (it crowds the
       // Infinity Cache).  RAFHIP_LANS_BLOCKS_PER_CU overrides the default downwards or up to the fit.
@@ -403,6 +525,9 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
         if (want > 0) per_cu = (fit > 0 && want > fit) ? fit : want;
       }
       p->pipeline_grid = (unsigned)(p->n_cus * per_cu);
+      const std::vector<WorkItem> pipeline =
+          build_pipeline(n_tensors, numel, group_elems_setting(), (int)p->pipeline_grid);
+      p->n_pipeline_items = (uint32_t)pipeline.size();
       if (p->pipeline_grid > p->n_pipeline_items) p->pipeline_grid = p->n_pipeline_items;
 
       const size_t tensors_bytes = (size_t)align_up((int64_t)sizeof(TensorRec) * n_tensors);

@@ -20,6 +20,7 @@
 // (python/raf/optim/sgd.py:187-215) -- and for the one-op-call-per-parameter loop of its imperative
 // optimizer (sgd.py:51-58).
 #include <cstdint>
+#include <cstdlib>
 #include <memory>
 #include <new>
 #include <vector>
@@ -34,7 +35,15 @@ namespace rafhip {
 namespace {
 
 constexpr int kSgdBlock = 256;
-constexpr int kSgdUnroll = 2;  // float4 groups in flight per lane per trip
+constexpr int kSgdUnroll = 2;  // float4 groups in flight per lane per trip (multi-tensor default)
+
+int env_int(const char* name, int fallback) {
+  if (const char* e = std::getenv(name)) {
+    const int v = std::atoi(e);
+    if (v > 0) return v;
+  }
+  return fallback;
+}
 
 __device__ __forceinline__ void sgd_elem(float x0, float dx, float v0, float lr, float mu,
                                          float& v1, float& x1) {
@@ -45,6 +54,7 @@ __device__ __forceinline__ void sgd_elem(float x0, float dx, float v0, float lr,
 }
 
 // Vector path: all five pointers 16-byte aligned.  n4 = number of whole float4 groups.
+template <int kSgdUnroll>
 __global__ __launch_bounds__(kSgdBlock) void sgd_vec4_kernel(
     const f32x4* x, const f32x4* dx, const f32x4* v, f32x4* v_out, f32x4* x_out, int64_t n4,
     float lr, float mu) {
@@ -94,7 +104,7 @@ __global__ __launch_bounds__(kSgdBlock) void sgd_scalar_kernel(
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // ------------------------------------------------------------------ multi-tensor, in place
-constexpr int kSgdChunk = 4096;  // elements per work item
+constexpr int kSgdChunkShiftDefault = 12;  // 4096 elements per work item
 
 struct SgdRec {  // 48 bytes, one per parameter
   float* x;      // fp32 (master) weight, updated in place
@@ -111,15 +121,16 @@ struct SgdItem {
   int32_t chunk;
 };
 
-template <typename G, bool kNT>
+template <typename G, bool kNT, int kSgdUnroll>
 __global__ __launch_bounds__(kSgdBlock) void sgd_multi_kernel(const SgdRec* recs,
                                                               const SgdItem* items,
                                                               int64_t n_items, float lr, float mu,
-                                                              int p_is_bf16) {
+                                                              int p_is_bf16, int chunk_shift) {
+  const int kSgdChunk = 1 << chunk_shift;
   for (int64_t it = blockIdx.x; it < n_items; it += gridDim.x) {
     const SgdItem item = items[it];
     const SgdRec r = recs[item.tensor];
-    const int64_t begin = (int64_t)item.chunk * kSgdChunk;
+    const int64_t begin = (int64_t)item.chunk << chunk_shift;
     const int64_t rest = r.numel - begin;
     const int len = rest < kSgdChunk ? (int)rest : kSgdChunk;
     float* x = r.x + begin;
@@ -175,14 +186,23 @@ __global__ __launch_bounds__(kSgdBlock) void sgd_multi_kernel(const SgdRec* recs
 constexpr int64_t kSgdStreamFromBytes = 160LL << 20;
 
 template <typename G>
-void launch_sgd_multi(bool stream_nt, unsigned grid, hipStream_t s, const SgdRec* recs,
-                      const SgdItem* items, int64_t n_items, float lr, float mu, int p_is_bf16) {
-  if (stream_nt)
-    hipLaunchKernelGGL((sgd_multi_kernel<G, true>), dim3(grid), dim3(kSgdBlock), 0, s, recs, items,
-                       n_items, lr, mu, p_is_bf16);
-  else
-    hipLaunchKernelGGL((sgd_multi_kernel<G, false>), dim3(grid), dim3(kSgdBlock), 0, s, recs, items,
-                       n_items, lr, mu, p_is_bf16);
+void launch_sgd_multi(bool stream_nt, int unroll, unsigned grid, hipStream_t s, const SgdRec* recs,
+                      const SgdItem* items, int64_t n_items, float lr, float mu, int p_is_bf16,
+                      int chunk_shift) {
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kSgdBlock), 0, s, recs, items, n_items, lr, mu,
+                       p_is_bf16, chunk_shift);
+  };
+  if (stream_nt) {
+    if (unroll >= 4)
+      go(sgd_multi_kernel<G, true, 4>);
+    else if (unroll == 1)
+      go(sgd_multi_kernel<G, true, 1>);
+    else
+      go(sgd_multi_kernel<G, true, 2>);
+  } else {
+    go(sgd_multi_kernel<G, false, kSgdUnroll>);
+  }
 }
 
 }  // namespace
@@ -208,13 +228,26 @@ extern "C" int rafhip_sgd_f32(const float* x, const float* dx, const float* v, f
   int64_t done = 0;
   if (vec && n >= 4) {
     const int64_t n4 = n / 4;
-    const int64_t per_block = (int64_t)kSgdBlock * kSgdUnroll;
+    static const int unroll = env_int("RAFHIP_SGD_UNROLL", 8);
+    static const int per_cu = env_int("RAFHIP_SGD_BLOCKS_PER_CU", 8);
+    const int64_t per_block = (int64_t)kSgdBlock * unroll;
     int64_t blocks = (n4 + per_block - 1) / per_block;
-    if (blocks > cap) blocks = cap;
-    hipLaunchKernelGGL(sgd_vec4_kernel, dim3((unsigned)blocks), dim3(kSgdBlock), 0, s,
-                       reinterpret_cast<const f32x4*>(x), reinterpret_cast<const f32x4*>(dx),
-                       reinterpret_cast<const f32x4*>(v), reinterpret_cast<f32x4*>(v_out),
-                       reinterpret_cast<f32x4*>(x_out), n4, lr32, mu32);
+    const int64_t gcap = (int64_t)cap / 8 * per_cu;
+    if (blocks > gcap) blocks = gcap;
+    auto go = [&](auto kernel) {
+      hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kSgdBlock), 0, s,
+                         reinterpret_cast<const f32x4*>(x), reinterpret_cast<const f32x4*>(dx),
+                         reinterpret_cast<const f32x4*>(v), reinterpret_cast<f32x4*>(v_out),
+                         reinterpret_cast<f32x4*>(x_out), n4, lr32, mu32);
+    };
+    if (unroll == 1)
+      go(sgd_vec4_kernel<1>);
+    else if (unroll == 4)
+      go(sgd_vec4_kernel<4>);
+    else if (unroll == 8)
+      go(sgd_vec4_kernel<8>);
+    else
+      go(sgd_vec4_kernel<2>);
     RAFHIP_HIP_TRY(hipGetLastError());
     done = n4 * 4;
   }
@@ -237,6 +270,9 @@ struct rafhip_sgd_plan {
   std::vector<int64_t> numel;
   int64_t total_elements = 0;
   int64_t n_items = 0;
+  int chunk_shift = 12;
+  int unroll = 2;
+  int blocks_per_cu = 8;  // grid cap per CU; 0 = one workgroup per item
   void* d_tables = nullptr;
   rafhip::SgdRec* d_recs = nullptr;
   rafhip::SgdItem* d_items = nullptr;
@@ -270,6 +306,11 @@ extern "C" int rafhip_sgd_plan_create(int32_t n_tensors, const int64_t* numel, i
     std::unique_ptr<rafhip_sgd_plan, void (*)(rafhip_sgd_plan*)> p(new rafhip_sgd_plan(), free_sgd_plan);
     p->n = n_tensors;
     p->grad_dtype = grad_dtype;
+    p->chunk_shift = env_int("RAFHIP_SGD_CHUNK_SHIFT", kSgdChunkShiftDefault);
+    if (p->chunk_shift < 10 || p->chunk_shift > 20) p->chunk_shift = kSgdChunkShiftDefault;
+    p->unroll = env_int("RAFHIP_SGD_MULTI_UNROLL", 4);
+    p->blocks_per_cu = std::getenv("RAFHIP_SGD_MULTI_BLOCKS_PER_CU") ? std::atoi(std::getenv("RAFHIP_SGD_MULTI_BLOCKS_PER_CU")) : 0;
+    const int64_t kSgdChunk = (int64_t)1 << p->chunk_shift;
     std::vector<SgdItem> items;
     for (int32_t t = 0; t < n_tensors; ++t) {
       if (numel[t] < 0)
@@ -343,16 +384,17 @@ extern "C" int rafhip_sgd_multi_step(rafhip_sgd_plan* plan, float* const* x, con
     // One rounding double -> fp32, as for the single-tensor op.
     const float lr32 = static_cast<float>(learning_rate);
     const float mu32 = static_cast<float>(mu);
-    const int64_t cap = streaming_grid_cap();
+    const int64_t cap = plan->blocks_per_cu > 0 ? (int64_t)streaming_grid_cap() / 8 * plan->blocks_per_cu
+                                                : (int64_t)1 << 20;
     const unsigned grid = (unsigned)(plan->n_items < cap ? plan->n_items : cap);
     const bool nt = plan->total_elements * (int64_t)(8 + g_elem) > kSgdStreamFromBytes;
     const int bf = p_dtype == RAFHIP_BF16 ? 1 : 0;
     if (plan->grad_dtype == RAFHIP_F16)
-      launch_sgd_multi<_Float16>(nt, grid, s, plan->d_recs, plan->d_items, plan->n_items, lr32, mu32, bf);
+      launch_sgd_multi<_Float16>(nt, plan->unroll, grid, s, plan->d_recs, plan->d_items, plan->n_items, lr32, mu32, bf, plan->chunk_shift);
     else if (plan->grad_dtype == RAFHIP_BF16)
-      launch_sgd_multi<Bf16>(nt, grid, s, plan->d_recs, plan->d_items, plan->n_items, lr32, mu32, bf);
+      launch_sgd_multi<Bf16>(nt, plan->unroll, grid, s, plan->d_recs, plan->d_items, plan->n_items, lr32, mu32, bf, plan->chunk_shift);
     else
-      launch_sgd_multi<float>(nt, grid, s, plan->d_recs, plan->d_items, plan->n_items, lr32, mu32, bf);
+      launch_sgd_multi<float>(nt, plan->unroll, grid, s, plan->d_recs, plan->d_items, plan->n_items, lr32, mu32, bf, plan->chunk_shift);
     RAFHIP_HIP_TRY(hipGetLastError());
     return RAFHIP_OK;
   });

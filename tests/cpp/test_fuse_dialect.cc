@@ -231,10 +231,12 @@ int main() {
   {
     Expr w2 = MakeVar("w2", Ty({1024, 1024})), dx2 = MakeVar("dx2", Ty({1024, 1024})), v2 = MakeVar("v2", Ty({1024, 1024}));
     Expr w3 = MakeVar("w3", Ty({1024})), dx3 = MakeVar("dx3", Ty({1024})), v3 = MakeVar("v3", Ty({1024}));
-    // the three updates hang under one root, as outputs of the traced function would
+    // the three updates hang under one root, as outputs of the traced function would; their
+    // learning rates differ, so they are not gathered into one multi-tensor call (the constants
+    // are lifted into parameters, so the functions are still identical)
     Expr root = MakeCall(GetOp("raf.op.tuple3"),
-                         {hip::TracedSgdUpdate(w, dx, v, 0.01, 0.9), hip::TracedSgdUpdate(w2, dx2, v2, 0.01, 0.9),
-                          hip::TracedSgdUpdate(w3, dx3, v3, 0.01, 0.9)});
+                         {hip::TracedSgdUpdate(w, dx, v, 0.01, 0.9), hip::TracedSgdUpdate(w2, dx2, v2, 0.02, 0.9),
+                          hip::TracedSgdUpdate(w3, dx3, v3, 0.03, 0.9)});
     Expr fused = pass::FuseDialect(root, DevType::kROCM());
     const auto* c = AsCall(fused);
     EXPECT(c && c->args.size() == 3);
@@ -243,13 +245,13 @@ int main() {
     Expr fn;
     Expr e0 = ExpectedFusedUpdate(w, dx, v, 0.01, 0.9, &fn);
     Expr expected = MakeCall(GetOp("raf.op.tuple3"),
-                             {e0, ExpectedFusedUpdate(w2, dx2, v2, 0.01, 0.9, nullptr, fn),
-                              ExpectedFusedUpdate(w3, dx3, v3, 0.01, 0.9)});
+                             {e0, ExpectedFusedUpdate(w2, dx2, v2, 0.02, 0.9, nullptr, fn),
+                              ExpectedFusedUpdate(w3, dx3, v3, 0.03, 0.9)});
     EXPECT(StructuralEqual(fused, expected));
     // sharing is part of the structure: three separate functions are a different graph
     Expr separate = MakeCall(GetOp("raf.op.tuple3"),
-                             {ExpectedFusedUpdate(w, dx, v, 0.01, 0.9), ExpectedFusedUpdate(w2, dx2, v2, 0.01, 0.9),
-                              ExpectedFusedUpdate(w3, dx3, v3, 0.01, 0.9)});
+                             {ExpectedFusedUpdate(w, dx, v, 0.01, 0.9), ExpectedFusedUpdate(w2, dx2, v2, 0.02, 0.9),
+                              ExpectedFusedUpdate(w3, dx3, v3, 0.03, 0.9)});
     EXPECT(!StructuralEqual(fused, separate));
   }
 

@@ -40,6 +40,22 @@ def test_cpp_ir_patterns_fuse_dialect_pass(native_libs, tmp_path):
     assert "ALL OK" in r.stdout
 
 
+def test_cpp_graph_rewrites_multi_tensor_sgd_and_mixed_lans(native_libs, tmp_path):
+    """The hip dialect's whole-graph rewrites on the traced SGD and LANS optimizers: expected graphs,
+    variants that must stay as they are (tests/cpp/test_graph_rewrites.cc)."""
+    exe = tmp_path / "test_graph_rewrites"
+    d = ROOT / "raf_amd" / "csrc" / "dialect"
+    subprocess.run(["g++", "-O1", "-std=c++17", "-Wall", f"-I{d}", f"-I{ROOT / 'include'}",
+                    str(ROOT / "tests" / "cpp" / "test_graph_rewrites.cc"),
+                    str(d / "registry.cc"), str(d / "raf_ir.cc"), str(d / "hip_fusion.cc"),
+                    str(d / "hip_dialect.cc"), str(d / "device_api.cc"), str(d / "memory_pool.cc"),
+                    f"-L{native_libs.LIB_DIR}", "-lraf_hip_optim", f"-Wl,-rpath,{native_libs.LIB_DIR}",
+                    "-o", str(exe)], check=True)
+    r = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "ALL OK" in r.stdout
+
+
 def test_traced_update_needs_a_rocm_device(native_libs):
     import torch
     from raf_amd import op

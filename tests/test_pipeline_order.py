@@ -5,15 +5,35 @@ import pytest
 KIND_A, KIND_B, KIND_C, KIND_WHOLE, KIND_FIN_A, KIND_FIN_B = range(6)
 
 
+STREAMED = 8  # flag added to the kind
+
+
+def _normalise(order):
+    """Strips the flag: returns the list of (base kind, tensor, chunk) and the set of tensors whose
+    items are marked streamed."""
+    out, streamed = [], set()
+    for kind, t, c in order:
+        base = kind & 7
+        assert kind in (base, base | STREAMED)
+        if kind & STREAMED:
+            streamed.add(t)
+            assert base in (KIND_A, KIND_B, KIND_C), "only data-moving items carry the streaming mark"
+        out.append((base, t, c))
+    return out, streamed
+
+
 def _check(order, sizes, lib):
     # a tensor's chunk size (and first-pass unit) depends on its own element count
     n_chunks = [-(-n // lib.rafhip_lans_chunk_elements(n)) for n in sizes]
     n_units = [-(-n // lib.rafhip_lans_pass_a_unit_elements(n)) for n in sizes]
+    order, streamed = _normalise(order)
     seen = {}
     for pos, (kind, t, c) in enumerate(order):
         assert 0 <= t < len(sizes) and sizes[t] > 0, "empty tensors contribute no work"
         assert (kind, t, c) not in seen, "duplicate work item"
         seen[(kind, t, c)] = pos
+    for t in streamed:
+        assert sizes[t] * 12 >= 256 << 20, "only tensors beyond the cache are streamed"
     for t, nc in enumerate(n_chunks):
         if nc == 0:
             continue
@@ -48,6 +68,9 @@ def test_order_invariants(native_libs, group):
         shapes.numels(shapes.bert_base_shapes()),
         [],
         [0, 0],
+        [23_000_000, 5000, 70_000],            # a streamed tensor with hardly anything beside it
+        [40_000_000],                          # ... and alone
+        [1 << 20] * 30 + [30_000_000] + [1 << 20] * 30 + [25_000_000],  # two streamed tensors among cached groups
     ]
     for sizes in lists:
         _check(kernels.pipeline_order(sizes, group), sizes, lib)
@@ -60,14 +83,14 @@ def test_groups_bound_the_reuse_distance(native_libs):
 
     chunk = native_libs.optim().rafhip_lans_chunk_elements(1)
     sizes = [8 * chunk] * 40  # 40 equal tensors, group = 2 tensors
-    order = kernels.pipeline_order(sizes, 16 * chunk)
+    order, _ = _normalise(kernels.pipeline_order(sizes, 16 * chunk))
     first_a = {t: min(i for i, (k, tt, _) in enumerate(order) if k == KIND_A and tt == t) for t in range(40)}
     last_c = {t: max(i for i, (k, tt, _) in enumerate(order) if k == KIND_C and tt == t) for t in range(40)}
     per_group = 2 * (2 * 8 + 1 + 2)
     for t in range(40):
         assert last_c[t] - first_a[t] <= 3 * per_group
     # one giant group degenerates into pass-major order: all of A, then all of B, then all of C
-    order = kernels.pipeline_order(sizes, 10**12)
+    order, _ = _normalise(kernels.pipeline_order(sizes, 10**12))
     kinds = [k for k, _, _ in order]
     assert max(i for i, k in enumerate(kinds) if k in (KIND_A, KIND_FIN_A)) < min(
         i for i, k in enumerate(kinds) if k == KIND_B)
@@ -82,3 +105,21 @@ def test_bert_large_group_structure(native_libs):
     _check(order, sizes, lib)
     assert sum(1 for k, _, _ in order if k == KIND_WHOLE) == sum(
         1 for n in sizes if 0 < n <= lib.rafhip_lans_chunk_elements(n))
+    # the word embedding (31 M elements: 375 MB of w, m, v) is streamed, and its items are spread
+    # over the list instead of standing at its head
+    emb = [i for i, (k, t, _) in enumerate(order) if t == 0]
+    assert all(k & STREAMED for k, t, _ in order if t == 0 and (k & 7) in (KIND_A, KIND_B, KIND_C))
+    assert not any(k & STREAMED for k, t, _ in order if t != 0)
+    assert emb[-1] > 0.9 * len(order) and emb[len(emb) // 2] > 0.3 * len(order)
+
+
+def test_streamed_items_keep_clear_of_their_finish_items(native_libs):
+    """What follows a finish item of a streamed tensor waits for it: the next streamed item comes
+    only after a few items per workgroup of other work."""
+    from raf_amd import kernels, shapes
+
+    order = kernels.pipeline_order(shapes.numels(shapes.bert_large_shapes()))
+    pos = {(k & 7): i for i, (k, t, _) in enumerate(order) if t == 0 and (k & 7) in (KIND_FIN_A, KIND_FIN_B)}
+    for fin in pos.values():
+        nxt = next(i for i in range(fin + 1, len(order)) if order[i][1] == 0)
+        assert nxt - fin > 2 * 768
