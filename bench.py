@@ -124,7 +124,7 @@ def workloads():
                                     zero_state=True, step0=1),
         "sgd_4m_fp32": dict(kind="sgd", n=4_194_304),
         "sgd_multi_bert_large_fp32": dict(kind="sgd_multi", sizes=shapes.numels(shapes.bert_large_shapes())),
-        # the traced optimizer's per-parameter op sequence after dialect fusion: one fused call per parameter
+        # the traced optimizer's per-parameter op sequence after dialect fusion: one multi-tensor call
         "traced_sgd_fused_bert_large_fp32": dict(kind="traced_sgd", sizes=shapes.numels(shapes.bert_large_shapes())),
         # neighbours of the optimizer step that reuse its machinery
         "l2norm_bert_large_flat_fp32": dict(kind="l2norm", n=sum(shapes.numels(shapes.bert_large_shapes()))),
@@ -676,8 +676,10 @@ def bench_copy(name, wl, args):
 
 
 def bench_traced_sgd(name, wl, args):
-    """One step = the traced SGD update of every parameter, each parameter's add/multiply/subtract
-    sequence fused by the dialect pass into one primitive function and run as one launch."""
+    """One step = the optimizer part of the reference's traced SGD optimizer over the whole model
+    (per parameter: add(multiply(momentum, v), dx, out=v), subtract(w, multiply(lr, new_v), out=w)),
+    taken through the FuseDialect pass: the hip dialect gathers every parameter's update into one
+    raf.op.hip.sgd_multi call, i.e. one launch for the model."""
     import torch
 
     from raf_amd import op
@@ -689,21 +691,14 @@ def bench_traced_sgd(name, wl, args):
     x = [torch.randn(n, device=dev, generator=gen) * 0.02 for n in sizes]
     dx = [torch.randn(n, device=dev, generator=gen) * 1e-3 for n in sizes]
     v = [torch.zeros(n, device=dev) for n in sizes]
-
-    updates = [op.TracedSgdUpdate(w_, d_, v_, 0.01, 0.9) for w_, d_, v_ in zip(x, dx, v)]
-
-    def step(_):
-        for upd in updates:
-            upd()
-
-    wall_ms, dev_ms = _timed(step, args)
-    res = _line("traced SGD update after dialect fusion, achieved HBM bandwidth (algorithmic bytes / step time)",
-                name, "f32", total * SGD_BYTES_PER_ELT, wall_ms, dev_ms, "sgd_vec4_kernel", args,
+    opt = op.TracedSgdOptimizer(x, dx, v, 0.01, 0.9)
+    calls = opt.ops
+    wall_ms, dev_ms = _timed(lambda i: opt(), args)
+    res = _line("traced SGD optimizer after dialect fusion: algorithmic bandwidth (20 B per element / step time)",
+                name, "f32", total * SGD_BYTES_PER_ELT, wall_ms, dev_ms, "sgd_multi_kernel", args,
                 {"tensors": len(sizes), "elements": total, "bytes_per_element": SGD_BYTES_PER_ELT,
-                 "launches_per_step": len(sizes), "unfused_kernels_per_step": 4 * len(sizes)})
-    # the roofline object is about one launch of the dominant kernel; here a step is many launches of
-    # different sizes, so the step as a whole stands in for it
-    res["roofline"]["note"] = "whole step (one launch per parameter), not a single launch"
+                 "calls_in_fused_graph": calls, "launches_per_step": len(calls),
+                 "unfused_kernels_per_step": 4 * len(sizes)})
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline_sgd(1 << 24)
     return res

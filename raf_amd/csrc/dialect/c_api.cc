@@ -203,6 +203,7 @@ class GraphRunner {
   }
 
   void Run(OpEnv* op_env, const std::vector<value::Value>& inputs, const value::Value& out) {
+    if (!op_env) throw Error("a call of the graph has no OpEnv: making the graph did not succeed");
     int64_t need = 0;
     for (const auto& r : op_env->workspace_requests()) need += RoundUp(r.nbytes);
     if (need > ws_left_) throw Error("the workspace is too small for the graph's operators");

@@ -63,7 +63,10 @@ constexpr int64_t kSmallTensorBelow = 1 << 19;  // finer work for lists of small
 constexpr int kChunksPerAShift = 3;
 constexpr int kChunksPerA = 1 << kChunksPerAShift;   // pass A reads 2-4 bytes per element, so its unit of work (and of
                                  // partial sums) is 8 chunks; its partial lives in the first one's slot
-constexpr int kUnroll = 2;       // 4-element groups in flight per lane per trip
+#ifndef RAFHIP_LANS_UNROLL
+#define RAFHIP_LANS_UNROLL 2
+#endif
+constexpr int kUnroll = RAFHIP_LANS_UNROLL;  // 4-element groups in flight per lane per trip
 constexpr int kPartialSlots = 4; // doubles per chunk: [0] sum g^2 | [1] sum u_m^2 [2] sum u_g^2 [3] sum w^2
 
 // A tensor's chunk size depends on its own element count alone, so its result does not depend on

@@ -66,6 +66,9 @@ constexpr int64_t kPipelinedFromElems = 64 * 1024 * 1024;
 // Lists whose g, w, m, v together stay under this many bytes fit in the cache: temporal accesses.
 constexpr int64_t kResidentBytes = 192LL << 20;
 
+// From this many elements on a tensor counts as long when the persistent kernel's occupancy is chosen.
+constexpr int64_t kLongTensorElems = 6 * 1000 * 1000;
+
 // Slices per round in which passes B and C alternate (measured on MI355X: 4 to 16 are within
 // 0.1 % of each other on the BERT-large list, 1 is 3 % slower).  RAFHIP_LANS_ROUND_SLICES overrides.
 constexpr int kDefaultRoundSlices = 8;
@@ -516,10 +519,16 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
         for (int64_t u = 0; u < units_a_of(numel[t]); ++u) phased_a.push_back(make_item(t, kPhaseA, u));
       p->n_items_a = (int64_t)phased_a.size();
       // Resident workgroups per CU: never more than fit (every workgroup must be running), and by
-      // default three: a larger window of in-flight items measured slower on MI355X (it crowds the
-      // Infinity Cache).  RAFHIP_LANS_BLOCKS_PER_CU overrides the default downwards or up to the fit.
+      // default three; a larger window of in-flight items measured slower on MI355X (it crowds the
+      // Infinity Cache).  Lists whose bulk is in long tensors (GPT-2's 8-10 M element matrices)
+      // measured 3 % faster with two, lists of shorter tensors (BERT: up to 4 M) 1-2 % slower.
+      // RAFHIP_LANS_BLOCKS_PER_CU overrides the choice downwards or up to the fit.
       const int fit = pipelined_blocks_per_cu(grad_dtype);
-      int per_cu = fit > 0 ? (fit < 3 ? fit : 3) : 2;
+      int64_t in_long_tensors = 0;
+      for (int32_t t = 0; t < n_tensors; ++t)
+        if (numel[t] >= kLongTensorElems) in_long_tensors += numel[t];
+      const int wanted = 2 * in_long_tensors > total ? 2 : 3;
+      int per_cu = fit > 0 ? (fit < wanted ? fit : wanted) : 2;
       if (const char* e = std::getenv("RAFHIP_LANS_BLOCKS_PER_CU")) {
         const int want = std::atoi(e);
         if (want > 0) per_cu = (fit > 0 && want > fit) ? fit : want;

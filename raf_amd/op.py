@@ -260,6 +260,102 @@ def traced_sgd_update(w, dx, v, learning_rate, momentum, return_ir=False):
     return (w, upd.ir_before, upd.ir_after) if return_ir else w
 
 
+class _TracedOptimizer:
+    """Common part of the two traced optimizers below: the optimizer graph is built for the given
+    parameter lists, taken through the FuseDialect pass (the hip dialect's graph rewrites first,
+    its patterns after), and every call of the resulting graph gets an OpEnv; ``__call__`` runs them
+    in order, in place on the tensors.  ``ir_before`` / ``ir_after`` hold the graph's text on either
+    side of the pass, ``ops`` what the fused graph calls (a leading ``!`` marks an operator that
+    stayed unfused and has no backend here)."""
+
+    _KIND = None
+
+    def _make(self, lists, step, zero_is_constant, hyper, allow_partial):
+        lib = _lib.dialect()
+        self._keep: list = [lists, step]
+        self._n = len(lists[1])
+        self._allow_partial = int(bool(allow_partial))
+
+        def array(ts):
+            if ts is None:
+                return None
+            if len(ts) != self._n:
+                raise ValueError("the tensor lists differ in length")
+            return (TensorDesc * max(self._n, 1))(*[_desc(t, self._keep) for t in ts])
+
+        self._descs = [array(ts) for ts in lists]
+        self._step = ctypes.byref(_desc(step, self._keep)) if step is not None else None
+        hy = (ctypes.c_double * len(hyper))(*[float(x) for x in hyper])
+        h = c_void_p(None)
+        status = lib.rafhip_raf_traced_optimizer_make(self._KIND, self._n, *self._descs, self._step,
+                                                      int(bool(zero_is_constant)), hy, len(hyper),
+                                                      self._allow_partial, ctypes.byref(h))
+        self._env = _Env(h) if h.value else None  # also set on failure: it then holds the graphs
+        check_raf(status)
+        self._first = lists[1][0]
+        self._execute = lib.rafhip_raf_traced_optimizer_execute
+
+    def __call__(self):
+        stream = _stream(self._first)
+        ws = _workspace(self._env, self._first, stream) if self._env.workspace_bytes > 0 else None
+        check_raf(self._execute(self._env.handle, self._n, *self._descs, self._step, self._allow_partial,
+                                ws.data if ws else None, self._env.workspace_bytes, stream))
+
+    def _text(self, fused: int) -> str:
+        buf = ctypes.create_string_buffer(1 << 22)
+        check_raf(_lib.dialect().rafhip_raf_env_ir_text(self._env.handle, fused, buf, len(buf)))
+        return buf.value.decode()
+
+    @property
+    def ir_before(self) -> str:
+        return self._text(0)
+
+    @property
+    def ir_after(self) -> str:
+        return self._text(1)
+
+    @property
+    def ops(self) -> List[str]:
+        buf = ctypes.create_string_buffer(1 << 16)
+        check_raf(_lib.dialect().rafhip_raf_env_graph_ops(self._env.handle, buf, len(buf)))
+        return [x for x in buf.value.decode().split(";") if x]
+
+
+class TracedSgdOptimizer(_TracedOptimizer):
+    """The optimizer part of what the reference's traced SGD optimizer builds for a whole model
+    (python/raf/optim/sgd.py:187-215): per parameter ``add(multiply(momentum, v), dx, out=v)`` and
+    ``subtract(w, multiply(learning_rate, new_v), out=w)`` (with ``cast(dx, "float32")`` in front
+    for a 16-bit gradient) and, with ``p`` (a half-precision model with fp32 master weights ``w``),
+    ``add(cast(new_w, dtype), zero, out=p)``.  The hip dialect gathers all of it into one
+    multi-tensor call.  ``zero_is_constant=False`` leaves the optimizer's zero tensor a free
+    variable, as traced: the cast and the copy then stay unfused (and, with ``allow_partial``, are
+    left out when the graph is run, since this library has no backend for them)."""
+
+    _KIND = 0
+
+    def __init__(self, w, dx, v, learning_rate, momentum, p=None, zero_is_constant=True, allow_partial=False):
+        self._make([list(dx), list(w), None, list(v), list(p) if p is not None else None], None,
+                   zero_is_constant, [learning_rate, momentum], allow_partial)
+
+
+class TracedLansOptimizer(_TracedOptimizer):
+    """The optimizer part of what the reference's traced LANS optimizer builds for a half-precision
+    model (python/raf/optim/lans.py:244-312): ``group_cast(g, "float32")``, ``raf.op.lans`` over
+    ``[g32..., w..., m..., v...]``, and per parameter ``cast(new_w, dtype)`` and
+    ``add(_, zero, out=p)``.  The hip dialect folds all of it into one ``raf.op.hip.lans_mixed``
+    call; with ``zero_is_constant=False`` only the group_cast folds (``raf.op.hip.lans`` on the half
+    gradients)."""
+
+    _KIND = 1
+
+    def __init__(self, g, w, m, v, p, step, learning_rate=1e-3, beta1=0.9, beta2=0.999, eps=1e-6,
+                 bias_correction=True, weight_decay=0.01, grad_averaging=True, mode=True, normalize_grad=True,
+                 zero_is_constant=True, allow_partial=False):
+        self._make([list(g), list(w), list(m), list(v), list(p)], step, zero_is_constant,
+                   [learning_rate, beta1, beta2, eps, int(bias_correction), weight_decay, int(grad_averaging),
+                    int(mode), int(bool(normalize_grad))], allow_partial)
+
+
 def sgd_multi(tensor_list: Sequence[torch.Tensor], learning_rate, mu):
     """Extension op: momentum SGD over a parameter list ``[x..., dx..., v...]`` in place (x and v
     are updated, the list is returned), one launch; per element the four roundings of ``sgd``."""
