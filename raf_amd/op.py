@@ -142,14 +142,21 @@ class _Marshalled:
         self.keep: list = []
         self.descs = (TensorDesc * max(len(tensors), 1))(*[_desc(t, self.keep) for t in tensors])
         self.sig = tuple(_sig(t) for t in tensors)
-        self.refs = [weakref.ref(t) for t in tensors]
-        self.ptrs = [t.data_ptr() for t in tensors]
+        # Once one of the tensors has died its id may be handed to another object: the weak
+        # references notice, and the entry is never trusted again.
+        self.alive = True
+        self.refs = [weakref.ref(t, self._one_died) for t in tensors]
+        self.ptrs = list(map(torch.Tensor.data_ptr, tensors))
         self.slot = 0
 
+    def _one_died(self, _ref) -> None:
+        self.alive = False
+
     def still_describes(self, tensors) -> bool:
-        # the same live objects (a weak reference cannot be fooled by a recycled id) at the same
-        # addresses: their shapes and dtypes cannot have changed either
-        return all(r() is t and t.data_ptr() == p for r, t, p in zip(self.refs, tensors, self.ptrs))
+        # The caller found this entry under the ids of `tensors`, and all of the original objects
+        # are alive, so these are the same objects; their shapes and dtypes cannot have changed,
+        # their storage can (x.data = ..., set_, resize_): the addresses are compared, at C speed.
+        return self.alive and list(map(torch.Tensor.data_ptr, tensors)) == self.ptrs
 
 
 _marshalled: Dict[Tuple, _Marshalled] = {}
