@@ -75,7 +75,8 @@ __host__ __device__ inline int chunk_shift_for(int64_t numel) {  // chunks are p
   return numel < kSmallTensorBelow ? 12 : 13;
 }
 __host__ __device__ inline int chunk_elems_for(int64_t numel) { return 1 << chunk_shift_for(numel); }
-static_assert(kSmallChunk == 1 << 12 && kChunk == 1 << 13, "chunk_shift_for must match the chunk sizes");
+constexpr int kChunkShift = 13;  // log2 of the largest chunk
+static_assert(kSmallChunk == 1 << 12 && kChunk == 1 << kChunkShift, "chunk_shift_for must match the chunk sizes");
 
 struct TensorRec {  // 64 bytes, one per tensor
   const void* g;
@@ -173,9 +174,11 @@ void launch_prepare(hipStream_t s, const LansDeviceArgs& a, const float* step_de
 // so the passes add the partials themselves and the two finish launches are skipped.
 constexpr int kInlineFinishChunks = 32;
 // The first pass also writes the step scalars: no set-up launch in this schedule.
+// `apply_slice_shift`: a streaming list's last pass works in slices of 2^that many elements
+// (10 to the chunk shift), 0 for whole chunks.
 void launch_phased(int grad_dtype, bool streaming, bool inline_finish, hipStream_t s,
                    const LansDeviceArgs& a, const float* step_dev, int32_t step_host,
-                   HParamsPod hp, hipEvent_t* marks);
+                   HParamsPod hp, hipEvent_t* marks, int apply_slice_shift);
 void launch_pipelined(int grad_dtype, unsigned grid, hipStream_t s, const LansDeviceArgs& a);
 // Resident workgroups per CU of the pipelined kernel (occupancy query), 0 on failure.
 int pipelined_blocks_per_cu(int grad_dtype);

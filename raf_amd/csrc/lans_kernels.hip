@@ -739,26 +739,45 @@ __global__ __launch_bounds__(kLansBlock) void lans_norm_u(LansDeviceArgs a) {
   }
 }
 
+// `slice_shift` > 0: a chunk is applied in slices of 2^slice_shift elements, one workgroup each
+// (pass C adds nothing up, so how a chunk is cut changes no result); the grid provides
+// kChunk >> slice_shift workgroups per chunk, and those beyond a shorter chunk's end do nothing.
+// A workgroup that makes one short trip and ends never holds loads back behind its own stores:
+// with 1024-element slices the streaming pass runs 3.5 % (BERT-large) to 6 % (BERT-base) faster.
 template <typename G, int kMode>
-__global__ __launch_bounds__(kLansBlock) void lans_apply(LansDeviceArgs a) {
+__global__ __launch_bounds__(kLansBlock) void lans_apply(LansDeviceArgs a, int slice_shift) {
   constexpr CachePolicy kP = kMode == kModeStreaming ? kPhasedPolicy : kResidentPolicy;
   __shared__ double red[4][kLansWaves];
   if (step_is_skipped(a)) return;
   const float unscale = grad_unscale_of(a);
   WaitCtx no_wait{nullptr, 0, nullptr};
   const StepScalars k = *a.scalars;
-  for (int64_t c = blockIdx.x; c < a.n_chunks; c += gridDim.x) {
+  const int split_shift = slice_shift > 0 ? kChunkShift - slice_shift : 0;
+  const int64_t n_slices = a.n_chunks << split_shift;
+  for (int64_t b = blockIdx.x; b < n_slices; b += gridDim.x) {
+    const int64_t c = b >> split_shift;
     const WorkItem it = a.items[c];
     const TensorRec tr = a.tensors[it.tensor];
     const uint32_t chunk = it.chunk_phase & kChunkMask;
-    const ChunkView cv = chunk_view(tr, chunk, (int)sizeof(G));
+    ChunkView cv = chunk_view(tr, chunk, (int)sizeof(G));
+    if (split_shift > 0) {
+      const int begin = (int)(b & ((1 << split_shift) - 1)) << slice_shift;
+      if (begin >= cv.len) continue;
+      cv.g = static_cast<const char*>(cv.g) + (int64_t)begin * (int)sizeof(G);
+      cv.w += begin;
+      cv.m += begin;
+      cv.v += begin;
+      if (cv.p) cv.p += begin;
+      const int slice = 1 << slice_shift;
+      cv.len = cv.len - begin < slice ? cv.len - begin : slice;
+    }
     ApplyParams p;
     if constexpr (kMode == kModeResidentInline) {
       double tot[3];
       tensor_totals<3, false>(a.partials + kPartialSlots * (int64_t)tr.first_chunk, 1, chunks_of(tr), 1,
                               tot, red, no_wait);
       p.inv_gdiv = a.stats[it.tensor].inv_grad_div;  // left by pass B
-      if (chunk == 0 && threadIdx.x == 0)
+      if (chunk == 0 && b == (c << split_shift) && threadIdx.x == 0)
         stats_after_b(&a.stats[it.tensor], tot, k, p.rm, p.rg);
       else
         (void)trust_ratios(tot, k, p.rm, p.rg);
@@ -935,7 +954,8 @@ void launch_prepare(hipStream_t s, const LansDeviceArgs& a, const float* step_de
 namespace {
 template <typename G, int kMode>
 void launch_phased_t(hipStream_t s, const LansDeviceArgs& a, const float* step_dev,
-                     int32_t step_host, const HParamsPod& hp, hipEvent_t* marks) {
+                     int32_t step_host, const HParamsPod& hp, hipEvent_t* marks,
+                     int apply_slice_shift) {
   const unsigned grid = (unsigned)(a.n_chunks < (1 << 20) ? a.n_chunks : (1 << 20));
   const unsigned grid_a = (unsigned)(a.n_items_a < (1 << 20) ? a.n_items_a : (1 << 20));
   auto mark = [&](int i) {
@@ -954,22 +974,27 @@ void launch_phased_t(hipStream_t s, const LansDeviceArgs& a, const float* step_d
   if (kFinishLaunches)
     hipLaunchKernelGGL(lans_finish, dim3((unsigned)a.n_tensors), dim3(kLansBlock), 0, s, a, 1);
   mark(4);
-  hipLaunchKernelGGL((lans_apply<G, kMode>), dim3(grid), dim3(kLansBlock), 0, s, a);
+  // Slices only where the pass streams from HBM: a cache-resident list is short of parallelism,
+  // not of bandwidth, and finer items cost it 30 % of the pass.
+  const int slice_shift = kMode == kModeStreaming ? apply_slice_shift : 0;
+  const int64_t slices = (int64_t)a.n_chunks << (slice_shift > 0 ? kChunkShift - slice_shift : 0);
+  const unsigned grid_c = (unsigned)(slices < (1 << 24) ? slices : (1 << 24));
+  hipLaunchKernelGGL((lans_apply<G, kMode>), dim3(grid_c), dim3(kLansBlock), 0, s, a, slice_shift);
   mark(5);
 }
 }  // namespace
 
 void launch_phased(int grad_dtype, bool streaming, bool inline_finish, hipStream_t s,
                    const LansDeviceArgs& a, const float* step_dev, int32_t step_host,
-                   HParamsPod hp, hipEvent_t* marks) {
+                   HParamsPod hp, hipEvent_t* marks, int apply_slice_shift) {
   auto go = [&](auto tag) {
     using G = decltype(tag);
     if (streaming)
-      launch_phased_t<G, kModeStreaming>(s, a, step_dev, step_host, hp, marks);
+      launch_phased_t<G, kModeStreaming>(s, a, step_dev, step_host, hp, marks, apply_slice_shift);
     else if (inline_finish)
-      launch_phased_t<G, kModeResidentInline>(s, a, step_dev, step_host, hp, marks);
+      launch_phased_t<G, kModeResidentInline>(s, a, step_dev, step_host, hp, marks, apply_slice_shift);
     else
-      launch_phased_t<G, kModeResident>(s, a, step_dev, step_host, hp, marks);
+      launch_phased_t<G, kModeResident>(s, a, step_dev, step_host, hp, marks, apply_slice_shift);
   };
   if (grad_dtype == RAFHIP_F16)
     go(_Float16{});

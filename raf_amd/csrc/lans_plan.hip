@@ -325,6 +325,8 @@ struct rafhip_lans_plan {
   int64_t n_chunks = 0;
   int64_t total_elements = 0;
   uint32_t spin_limit = 1u << 22;
+  int64_t resident_bytes = kResidentBytes;  // lists up to this size use temporal accesses throughout
+  int apply_slice_shift = 10;  // phased schedule, streaming lists: log2 of the last pass's slice
   bool short_tensors_only = false;  // no tensor has more than kInlineFinishChunks chunks
   uint32_t n_pipeline_items = 0;
   unsigned pipeline_grid = 0;
@@ -491,6 +493,10 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
       total += numel[t];
     }
     p->short_tensors_only = longest <= kInlineFinishChunks;
+    p->resident_bytes = (int64_t)env_count("RAFHIP_LANS_RESIDENT_MIB", (int)(kResidentBytes >> 20)) << 20;
+    p->apply_slice_shift = env_count("RAFHIP_LANS_APPLY_SLICE_SHIFT", 10);
+    if (p->apply_slice_shift != 0 && (p->apply_slice_shift < 10 || p->apply_slice_shift >= kChunkShift))
+      p->apply_slice_shift = 0;
     p->n_chunks = chunks;
     p->total_elements = total;
     p->schedule = schedule_setting(total);
@@ -766,8 +772,9 @@ int launch_step(const char* who, rafhip_lans_plan* plan, int32_t p_dtype, const 
       for (int i = 2; i < 6; ++i) RAFHIP_HIP_TRY(hipEventRecord(marks[i], s));
   } else {
     const int64_t bytes_per_elt = plan->grad_dtype == RAFHIP_F32 ? 16 : 14;
-    launch_phased(plan->grad_dtype, plan->total_elements * bytes_per_elt > kResidentBytes,
-                  plan->short_tensors_only, s, a, step_dev, step_host, pod, marks);
+    launch_phased(plan->grad_dtype, plan->total_elements * bytes_per_elt > plan->resident_bytes,
+                  plan->short_tensors_only, s, a, step_dev, step_host, pod, marks,
+                  plan->apply_slice_shift);
   }
   RAFHIP_HIP_TRY(hipGetLastError());
   plan->steps_done++;

@@ -104,7 +104,10 @@ __global__ __launch_bounds__(kSgdBlock) void sgd_scalar_kernel(
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // ------------------------------------------------------------------ multi-tensor, in place
-constexpr int kSgdChunkShiftDefault = 12;  // 4096 elements per work item
+// 1024 elements per work item: a workgroup makes one trip (one 16-byte access per lane and array)
+// and ends, so no wavefront ever holds loads back behind its own stores.  Measured on the
+// BERT-large list: 6.29 TB/s, against 5.80-5.86 with 2048 and 5.67-5.85 with 4096 elements per item.
+constexpr int kSgdChunkShiftDefault = 10;
 
 struct SgdRec {  // 48 bytes, one per parameter
   float* x;      // fp32 (master) weight, updated in place
@@ -228,11 +231,17 @@ extern "C" int rafhip_sgd_f32(const float* x, const float* dx, const float* v, f
   int64_t done = 0;
   if (vec && n >= 4) {
     const int64_t n4 = n / 4;
-    static const int unroll = env_int("RAFHIP_SGD_UNROLL", 8);
+    static const int unroll_short = env_int("RAFHIP_SGD_UNROLL", 8);
     static const int per_cu = env_int("RAFHIP_SGD_BLOCKS_PER_CU", 8);
+    // A long tensor is better served by workgroups that make one trip and end (see the
+    // multi-tensor kernel): 6.4 against 6.2 TB/s at 16 Mi elements, 6.15 against 5.5 at 256 Mi.
+    // A short one is launch-bound and wants few, deep workgroups.
+    static const int64_t one_trip_from = (int64_t)env_knob("RAFHIP_SGD_ONE_TRIP_FROM_MI", 16) << 20;
+    const bool one_trip = n >= one_trip_from;
+    const int unroll = one_trip ? 1 : unroll_short;
     const int64_t per_block = (int64_t)kSgdBlock * unroll;
     int64_t blocks = (n4 + per_block - 1) / per_block;
-    const int64_t gcap = (int64_t)cap / 8 * per_cu;
+    const int64_t gcap = one_trip ? (int64_t)1 << 30 : (int64_t)cap / 8 * per_cu;
     if (blocks > gcap) blocks = gcap;
     auto go = [&](auto kernel) {
       hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kSgdBlock), 0, s,
@@ -308,7 +317,7 @@ extern "C" int rafhip_sgd_plan_create(int32_t n_tensors, const int64_t* numel, i
     p->grad_dtype = grad_dtype;
     p->chunk_shift = env_int("RAFHIP_SGD_CHUNK_SHIFT", kSgdChunkShiftDefault);
     if (p->chunk_shift < 10 || p->chunk_shift > 20) p->chunk_shift = kSgdChunkShiftDefault;
-    p->unroll = env_int("RAFHIP_SGD_MULTI_UNROLL", 4);
+    p->unroll = env_int("RAFHIP_SGD_MULTI_UNROLL", 1);
     p->blocks_per_cu = std::getenv("RAFHIP_SGD_MULTI_BLOCKS_PER_CU") ? std::atoi(std::getenv("RAFHIP_SGD_MULTI_BLOCKS_PER_CU")) : 0;
     const int64_t kSgdChunk = (int64_t)1 << p->chunk_shift;
     std::vector<SgdItem> items;

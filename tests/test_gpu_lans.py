@@ -296,6 +296,48 @@ def test_pipelined_schedule_is_bitwise_equal_to_phased(native_libs, monkeypatch,
         _assert_norms(results["pipelined"][1], on)
 
 
+@pytest.mark.parametrize("copy16", [False, True])
+def test_sliced_last_pass_of_streaming_lists_is_bitwise_equal(native_libs, monkeypatch, copy16):
+    """Lists beyond the cache run the phased schedule's last pass in 1024-element slices of a chunk,
+    one workgroup each.  Forced onto short ragged lists (resident limit 0), every slice size gives
+    the unsliced pass's bits, which are the pipelined schedule's; unaligned tensors (scalar path)
+    and the 16-bit weight copies included."""
+    from raf_amd import kernels
+
+    sizes = [1, 3, 4, 5, 0, 255, 1023, 1024, 1025, 4095, 4097, 8191, 8192, 8193, 16385, 65537, 100003,
+             (1 << 20) + 1029, 12345]
+    g, w, m, v = lans_inputs(sizes, cfg=81, g16=True)
+    hp = LansHParams(grad_unscale=1 / 1024)
+    monkeypatch.setenv("RAFHIP_LANS_RESIDENT_MIB", "0")
+    results = {}
+    for variant in ("pipelined", "0", "10", "11", "12"):
+        if variant != "pipelined":
+            monkeypatch.setenv("RAFHIP_LANS_APPLY_SLICE_SHIFT", variant)
+        tg, tw, tm, tv = _to_dev(g), _to_dev(w), _to_dev(m), _to_dev(v)
+        # every third tensor starts 4 bytes off a 16-byte boundary
+        backing = [torch.zeros(n + 1, device=DEV) for n in sizes]
+        for i in range(0, len(sizes), 3):
+            off = backing[i][1:]
+            off.copy_(tw[i])
+            tw[i] = off
+        tp = [torch.zeros(n, dtype=torch.float16, device=DEV) for n in sizes] if copy16 else None
+        plan = kernels.LansPlan(sizes, tg[0].dtype, DEV)
+        plan.set_schedule("pipelined" if variant == "pipelined" else "phased")
+        for step in (1, 2):
+            plan.step(tg, tw, tm, tv, step, _khp(hp), p=tp)
+        torch.cuda.synchronize()
+        plan.read_norms()
+        results[variant] = [t.cpu().numpy() for t in tw + tm + tv + (tp or [])]
+        plan.close()
+    for variant in ("0", "10", "11", "12"):
+        for i, (a, b) in enumerate(zip(results["pipelined"], results[variant])):
+            assert np.array_equal(a, b), (variant, i)
+    ow, om, ov = w, m, v
+    for step in (1, 2):
+        ow, om, ov, _ = lans_f64.lans_step(g, ow, om, ov, step, hp)
+    _assert_close(results["10"][:3 * len(sizes)], ow + om + ov, TOL_1, "sliced")
+
+
 def test_random_lists_groupings_and_slicings_agree_bitwise(native_libs, monkeypatch):
     """Whatever the list looks like and however the pipelined work list is cut (cache-group size,
     slices per round, resident workgroups), the result is the phased schedule's, bit for bit, and no
