@@ -189,6 +189,33 @@ def test_fp16_gradient_unscale_is_applied_first():
     np.testing.assert_allclose(a[0], sw, rtol=1e-12)
 
 
+def test_dynamic_scale_is_an_exact_unscale_or_no_step_at_all():
+    """The dynamic-loss-scaling form (an extension with no counterpart in the reference): with a
+    power-of-two scale it is the plain step on the exactly unscaled gradients, bit for bit; a set
+    overflow flag returns w, m, v untouched, whatever the gradients hold; a scale that is not a
+    power of two is rounded to fp32 once, like a device word would hold it."""
+    sizes = [7, 130]
+    g, w, m, v = lans_inputs(sizes, cfg=33)
+    g512 = [(x * np.float32(512)).astype(np.float32) for x in g]
+    a = lans_f64.lans_step_dynamic_scale(g512, w, m, v, 3, LansHParams(), 1.0 / 512, 0.0)
+    b = lans_f64.lans_step(g, w, m, v, 3, LansHParams())
+    for xs, ys in zip(a[:3], b[:3]):
+        for x, y in zip(xs, ys):
+            assert np.array_equal(x, y)
+    np.testing.assert_array_equal(a[3], b[3])
+    poisoned = [np.full_like(x, np.inf) for x in g]
+    sw, sm, sv, sn = lans_f64.lans_step_dynamic_scale(poisoned, w, m, v, 3, LansHParams(), 1.0 / 512, 1.0)
+    for xs, ys in zip((sw, sm, sv), (w, m, v)):
+        for x, y in zip(xs, ys):
+            assert np.array_equal(x, y) and x is not y
+    assert np.isnan(sn).all()
+    third = lans_f64.lans_step_dynamic_scale(g, w, m, v, 3, LansHParams(), 1.0 / 3.0, 0.0)
+    same = lans_f64.lans_step(g, w, m, v, 3, LansHParams(grad_unscale=float(np.float32(1.0 / 3.0))))
+    assert all(np.array_equal(x, y) for x, y in zip(third[0], same[0]))
+    assert np.array_equal(third[3], same[3])
+    assert not np.array_equal(third[3], b[3])  # and the scale is applied at all
+
+
 # ------------------------------------------------------------------ invariants and special cases
 def test_tensor_independence_and_list_order():
     sizes = [5, 1, 130, 17]
