@@ -56,16 +56,19 @@ def lans_kernel_bytes_per_elt(g_bytes: int):
 SGD_BYTES_PER_ELT = 20  # read x, dx, v; write v1, x1
 
 
+_COMMENTS = re.compile(r"//[^\n]*|/\*.*?\*/", re.S)
+
+
 def kernel_sources_digest() -> str:
-    """Digest of the HIP sources the kernel library is built from: a traffic figure measured with
-    rocprofv3 belongs to the kernels it was measured on."""
+    """Digest of the HIP sources the kernel library is built from, comments and white space aside: a
+    traffic figure measured with rocprofv3 belongs to the kernels it was measured on."""
     from raf_amd import build
 
     h = hashlib.sha256()
     files = sorted([build.CSRC / s for s in build.OPTIM_SOURCES] + list(build.CSRC.glob("*.h")))
     for f in files:
         h.update(f.name.encode())
-        h.update(f.read_bytes())
+        h.update(" ".join(_COMMENTS.sub(" ", f.read_text()).split()).encode())
     return h.hexdigest()[:16]
 
 

@@ -60,8 +60,8 @@ inline int64_t units_a_of(int64_t numel) {
 // same group left in the 256 MB Infinity Cache one round earlier.
 constexpr int64_t kDefaultGroupElems = 13 * 1000 * 1000;
 // Lists at least this long run pipelined by default; shorter ones are launch- and latency-bound
-// and do better with one launch per pass (measured on prefixes of the BERT-large list: equal at
-// 50 M elements, pipelined 4 % faster at 76 M, 5 % at 100 M, phased 7 % faster at 25 M).
+// and do better with one launch per pass (measured on prefixes of the BERT-large list: phased 9 %
+// faster at 26 M elements, 2 % at 51 M, pipelined 1-3 % faster at 65 M, 4 % at 80 M).
 constexpr int64_t kPipelinedFromElems = 64 * 1024 * 1024;
 // Lists whose g, w, m, v together stay under this many bytes fit in the cache: temporal accesses.
 constexpr int64_t kResidentBytes = 192LL << 20;
