@@ -282,7 +282,9 @@ int rafhip_lans_read_norms(const rafhip_lans_plan* plan, const void* workspace, 
  * kernels on the step's stream into slot (step_index % slots); slots == 0 turns it off.
  * rafhip_lans_timing_read waits for that slot's last event and returns five durations in
  * milliseconds.  Phased schedule: [0] norm of g  [1] finish  [2] norms of u_m, u_g, w  [3] finish
- * [4] apply.  Pipelined schedule: [0] set-up  [1] the persistent kernel  [2..4] zero.
+ * [4] apply ([1] and [3] zero for a list of short tensors, which has no finish launches).
+ * Pipelined schedule: [0] set-up  [1] the persistent kernel  [2..4] zero.  Only the events that
+ * delimit a launch are recorded: each costs a few microseconds of the step.
  */
 int rafhip_lans_timing_enable(rafhip_lans_plan* plan, int32_t slots);
 int rafhip_lans_timing_read(rafhip_lans_plan* plan, int32_t slot, float* ms_out5);

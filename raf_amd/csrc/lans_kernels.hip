@@ -966,14 +966,16 @@ void launch_phased_t(hipStream_t s, const LansDeviceArgs& a, const float* step_d
   hipLaunchKernelGGL((lans_norm_g<G, kMode>), dim3(grid_a), dim3(kLansBlock), 0, s, a, step_dev,
                      step_host, hp);
   mark(1);
-  if (kFinishLaunches)
+  if (kFinishLaunches) {
     hipLaunchKernelGGL(lans_finish, dim3((unsigned)a.n_tensors), dim3(kLansBlock), 0, s, a, 0);
-  mark(2);
+    mark(2);
+  }
   hipLaunchKernelGGL((lans_norm_u<G, kMode>), dim3(grid), dim3(kLansBlock), 0, s, a);
   mark(3);
-  if (kFinishLaunches)
+  if (kFinishLaunches) {
     hipLaunchKernelGGL(lans_finish, dim3((unsigned)a.n_tensors), dim3(kLansBlock), 0, s, a, 1);
-  mark(4);
+    mark(4);
+  }
   // Slices only where the pass streams from HBM: a cache-resident list is short of parallelism,
   // not of bandwidth, and finer items cost it 30 % of the pass.
   const int slice_shift = kMode == kModeStreaming ? apply_slice_shift : 0;

@@ -365,6 +365,7 @@ struct rafhip_lans_plan {
 
   // Optional per-kernel timing: slots x 6 events.
   std::vector<std::array<hipEvent_t, 6>> timing;
+  std::vector<int> timing_marks;  // which events the slot's last step recorded (each costs microseconds)
   int64_t steps_done = 0;
 };
 
@@ -375,6 +376,7 @@ void destroy_timing(rafhip_lans_plan* p) {
     for (auto& e : slot)
       if (e) (void)hipEventDestroy(e);
   p->timing.clear();
+  p->timing_marks.clear();
 }
 
 void free_plan(rafhip_lans_plan* p) {
@@ -760,16 +762,22 @@ int launch_step(const char* who, rafhip_lans_plan* plan, int32_t p_dtype, const 
   pod.normalize_grad = hp->normalize_grad ? 1 : 0;
 
   hipEvent_t* marks = nullptr;
-  if (!plan->timing.empty())
-    marks = plan->timing[plan->steps_done % (int64_t)plan->timing.size()].data();
+  if (!plan->timing.empty()) {
+    const size_t slot = (size_t)(plan->steps_done % (int64_t)plan->timing.size());
+    marks = plan->timing[slot].data();
+    // bit j: event j is recorded in this step (a launch that is skipped needs no event after it)
+    const int64_t bytes_per_elt = plan->grad_dtype == RAFHIP_F32 ? 16 : 14;
+    const bool inline_finish =
+        plan->short_tensors_only && plan->total_elements * bytes_per_elt <= plan->resident_bytes;
+    plan->timing_marks[slot] = plan->schedule == RAFHIP_LANS_PIPELINED ? 0x07 : inline_finish ? 0x2B : 0x3F;
+  }
 
   if (plan->schedule == RAFHIP_LANS_PIPELINED) {
     if (marks) RAFHIP_HIP_TRY(hipEventRecord(marks[0], s));
     launch_prepare(s, a, step_dev, step_host, pod);
     if (marks) RAFHIP_HIP_TRY(hipEventRecord(marks[1], s));
     launch_pipelined(plan->grad_dtype, plan->pipeline_grid, s, a);
-    if (marks)
-      for (int i = 2; i < 6; ++i) RAFHIP_HIP_TRY(hipEventRecord(marks[i], s));
+    if (marks) RAFHIP_HIP_TRY(hipEventRecord(marks[2], s));
   } else {
     const int64_t bytes_per_elt = plan->grad_dtype == RAFHIP_F32 ? 16 : 14;
     launch_phased(plan->grad_dtype, plan->total_elements * bytes_per_elt > plan->resident_bytes,
@@ -930,6 +938,7 @@ int rafhip_lans_timing_enable(rafhip_lans_plan* plan, int32_t slots) {
     destroy_timing(plan);
     plan->steps_done = 0;
     plan->timing.resize((size_t)slots);
+    plan->timing_marks.assign((size_t)slots, 0);
     for (auto& slot : plan->timing) slot.fill(nullptr);
     for (auto& slot : plan->timing)
       for (auto& e : slot) {
@@ -950,8 +959,17 @@ int rafhip_lans_timing_read(rafhip_lans_plan* plan, int32_t slot, float* ms_out5
   if (slot < 0 || (size_t)slot >= plan->timing.size() || plan->steps_done <= slot)
     return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_timing_read: slot %d holds no step", slot);
   auto& ev = plan->timing[(size_t)slot];
-  RAFHIP_HIP_TRY(hipEventSynchronize(ev[5]));
-  for (int i = 0; i < 5; ++i) RAFHIP_HIP_TRY(hipEventElapsedTime(&ms_out5[i], ev[i], ev[i + 1]));
+  const int recorded = plan->timing_marks[(size_t)slot];
+  if ((recorded & 1) == 0) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_timing_read: slot %d holds no step", slot);
+  int last = 0;
+  for (int j = 1; j < 6; ++j) {
+    ms_out5[j - 1] = 0.0f;
+    if (recorded & (1 << j)) {  // the interval that ends at event j started at the last recorded event
+      RAFHIP_HIP_TRY(hipEventSynchronize(ev[j]));
+      RAFHIP_HIP_TRY(hipEventElapsedTime(&ms_out5[j - 1], ev[last], ev[j]));
+      last = j;
+    }
+  }
   return RAFHIP_OK;
 }
 

@@ -709,3 +709,33 @@ def test_two_lists_alternating_on_two_streams_through_one_plan(native_libs):
         _assert_close([t.cpu().numpy() for t in tw], ow, TOL_1, "w")
         _assert_close([t.cpu().numpy() for t in tv], ov, TOL_1, "v")
     plan.close()
+
+
+def test_per_kernel_timing_slots(native_libs):
+    """rafhip_lans_timing_*: five intervals per step, zero where the schedule launches nothing."""
+    from raf_amd import kernels
+
+    hp = LansHParams()
+    cases = [("pipelined", [1 << 20, 70001], [True, True, False, False, False]),
+             ("phased", [1 << 20, 70001], [True] * 5),          # a long tensor: the two finish launches run
+             ("phased", [70001, 5, 4096], [True, False, True, False, True])]  # short tensors: they do not
+    for schedule, sizes, nonzero in cases:
+        g, w, m, v = lans_inputs(sizes, cfg=95)
+        tg, tw, tm, tv = _to_dev(g), _to_dev(w), _to_dev(m), _to_dev(v)
+        plan = kernels.LansPlan(sizes, torch.float32, DEV)
+        plan.set_schedule(schedule)
+        plan.timing_enable(2)
+        with pytest.raises(native_libs.RafHipError, match="holds no step"):
+            plan.timing_read(0)
+        for step in (1, 2, 3):
+            plan.step(tg, tw, tm, tv, step, _khp(hp))
+        torch.cuda.synchronize()
+        for slot in (0, 1):
+            ms = plan.timing_read(slot)
+            assert len(ms) == 5 and all(x >= 0.0 for x in ms)
+            assert [x > 0.0 for x in ms] == nonzero, (schedule, sizes, ms)
+            assert sum(ms) < 50.0
+        plan.timing_enable(0)
+        plan.step(tg, tw, tm, tv, 4, _khp(hp))
+        torch.cuda.synchronize()
+        plan.close()
