@@ -41,6 +41,8 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import List, Sequence, Tuple
 
+import math
+
 import numpy as np
 
 from oracle.halfs import narrow_weight, widen_grad
@@ -115,10 +117,10 @@ def l2norm(x: np.ndarray) -> float:
     return float(np.sqrt(np.dot(x, x)))
 
 
-def lans_directions(g, w, m, v, sc: LansScalars, hp: LansHParams):
+def lans_directions(g, w, m, v, sc: LansScalars, hp: LansHParams, repeat: int = 1):
     """Stage 1 for one tensor; float64 in, float64 out.
-    Returns (m1, v1, u_m, u_g, grad_norm)."""
-    gn = l2norm(g)
+    Returns (m1, v1, u_m, u_g, grad_norm).  ``repeat``: see lans_tensor_step."""
+    gn = l2norm(g) * math.sqrt(repeat)
     sg = g / (gn + sc.eps) if (hp.normalize_grad and gn != 0.0) else g
     wp = w if sc.wd != 0.0 else np.zeros_like(w)
     if int(hp.mode) == 0:
@@ -136,18 +138,24 @@ def lans_directions(g, w, m, v, sc: LansScalars, hp: LansHParams):
     return m1, v1, u_m, u_g, gn
 
 
-def lans_tensor_step(g, w, m, v, step, hp: LansHParams):
+def lans_tensor_step(g, w, m, v, step, hp: LansHParams, repeat: int = 1):
     """One LANS step on one tensor.  Inputs are used at float64 (g through
     ``grad_to_f64``); returns float64 ``(w1, m1, v1, norms)`` where ``norms`` =
-    (||g||, ||w||, ||u_m||, ||u_g||)."""
+    (||g||, ||w||, ||u_m||, ||u_g||).
+
+    ``repeat`` = k > 1 stands for a tensor that consists of k copies of the
+    given arrays back to back (a way to state what the step does to a tensor
+    of billions of elements without holding it): each of its norms is sqrt(k)
+    times the pattern's, and every copy gets the pattern's result."""
     sc = lans_scalars(hp, step)
     g64 = grad_to_f64(g, hp).ravel()
     w64 = np.asarray(w, dtype=np.float64).ravel()
     m64 = np.asarray(m, dtype=np.float64).ravel()
     v64 = np.asarray(v, dtype=np.float64).ravel()
-    pn = l2norm(w64)
-    m1, v1, u_m, u_g, gn = lans_directions(g64, w64, m64, v64, sc, hp)
-    un_m, un_g = l2norm(u_m), l2norm(u_g)
+    rep = math.sqrt(repeat)
+    pn = l2norm(w64) * rep
+    m1, v1, u_m, u_g, gn = lans_directions(g64, w64, m64, v64, sc, hp, repeat)
+    un_m, un_g = l2norm(u_m) * rep, l2norm(u_g) * rep
     r_m = sc.lr * (pn / un_m) if (un_m != 0.0 and pn != 0.0) else sc.lr
     r_g = sc.lr * (pn / un_g) if (un_g != 0.0 and pn != 0.0) else sc.lr
     r_m *= sc.beta1

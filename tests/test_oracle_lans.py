@@ -216,6 +216,26 @@ def test_dynamic_scale_is_an_exact_unscale_or_no_step_at_all():
     assert not np.array_equal(third[3], b[3])  # and the scale is applied at all
 
 
+def test_repeat_stands_for_a_tensor_of_back_to_back_copies():
+    """lans_tensor_step(..., repeat=k) against the step on the pattern tiled k times explicitly: the
+    norms are sqrt(k) times the pattern's and every copy gets the same result (to the rounding of the
+    differently ordered sums); repeat=1 changes no bit."""
+    g, w, m, v = lans_inputs([257], cfg=34)
+    hp = LansHParams()
+    for k in (2, 3, 7):
+        tiled = [np.tile(a[0], k) for a in (g, w, m, v)]
+        w1, m1, v1, n1 = lans_f64.lans_tensor_step(*tiled, 4, hp)
+        wr, mr, vr, nr = lans_f64.lans_tensor_step(g[0], w[0], m[0], v[0], 4, hp, repeat=k)
+        np.testing.assert_allclose(nr, n1, rtol=1e-13)
+        for big, pat in ((w1, wr), (m1, mr), (v1, vr)):
+            for j in range(k):
+                np.testing.assert_allclose(big[j * 257:(j + 1) * 257], pat, rtol=1e-12, atol=0)
+        assert not np.allclose(nr, lans_f64.lans_tensor_step(g[0], w[0], m[0], v[0], 4, hp)[3])
+    a = lans_f64.lans_tensor_step(g[0], w[0], m[0], v[0], 4, hp, repeat=1)
+    b = lans_f64.lans_tensor_step(g[0], w[0], m[0], v[0], 4, hp)
+    assert all(np.array_equal(x, y) for x, y in zip(a[:3], b[:3])) and a[3] == b[3]
+
+
 # ------------------------------------------------------------------ invariants and special cases
 def test_tensor_independence_and_list_order():
     sizes = [5, 1, 130, 17]
