@@ -234,9 +234,10 @@ extern "C" int rafhip_sgd_f32(const float* x, const float* dx, const float* v, f
     static const int unroll_short = env_int("RAFHIP_SGD_UNROLL", 8);
     static const int per_cu = env_int("RAFHIP_SGD_BLOCKS_PER_CU", 8);
     // A long tensor is better served by workgroups that make one trip and end (see the
-    // multi-tensor kernel): 6.4 against 6.2 TB/s at 16 Mi elements, 6.15 against 5.5 at 256 Mi.
-    // A short one is launch-bound and wants few, deep workgroups.
-    static const int64_t one_trip_from = (int64_t)env_knob("RAFHIP_SGD_ONE_TRIP_FROM_MI", 16) << 20;
+    // multi-tensor kernel): 6.2 against 6.0 TB/s at 16 Mi elements, 6.15 against 5.5 at 256 Mi,
+    // equal at 8 Mi.  A short one is launch-bound and wants few, deep workgroups (4 Mi elements:
+    // 5.8 against 5.3 TB/s).
+    static const int64_t one_trip_from = (int64_t)env_knob("RAFHIP_SGD_ONE_TRIP_FROM_MI", 8) << 20;
     const bool one_trip = n >= one_trip_from;
     const int unroll = one_trip ? 1 : unroll_short;
     const int64_t per_block = (int64_t)kSgdBlock * unroll;
