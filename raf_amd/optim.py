@@ -26,6 +26,8 @@ class SGD:
         if momentum < 0.0:
             raise ValueError("Invalid momentum value: {}".format(momentum))
         self.params = []
+        self._lists = None  # the weight and velocity lists of all parameters, made on first use
+        self._model = None  # (data pointers, aliases of the half-precision parameters' data)
         self._lr = learning_rate
         self._momentum = momentum
         params = list(params)
@@ -52,11 +54,27 @@ class SGD:
                 x0.data.copy_(x1)
                 v0.copy_(v1)
             return
-        tensor_list = [w for _, w, _ in live] + [x.grad for x, _, _ in live] + [v for _, _, v in live]
+        if len(live) == len(self.params):
+            # every parameter has a gradient: the weight and velocity lists made once, and one
+            # attribute read per parameter
+            if self._lists is None:
+                self._lists = ([w for _, w, _ in self.params], [v for _, _, v in self.params])
+            ws, vs = self._lists
+        else:
+            ws, vs = [w for _, w, _ in live], [v for _, _, v in live]
+        tensor_list = ws + [x.grad for x, _, _ in live] + vs
         if self.mixed:
-            _op.sgd_multi_mixed(tensor_list + [x.data for x, _, _ in live], self._lr, self._momentum)
+            _op.sgd_multi_mixed(tensor_list + self._model_data(live), self._lr, self._momentum)
         else:
             _op.sgd_multi(tensor_list, self._lr, self._momentum)
+
+    def _model_data(self, live):
+        """Aliases of the half-precision parameters' data, kept while the storages stay the same."""
+        xs = [x for x, _, _ in live]
+        ptrs = list(map(torch.Tensor.data_ptr, xs))
+        if self._model is None or self._model[0] != ptrs:
+            self._model = (ptrs, [x.data for x in xs])
+        return self._model[1]
 
 
 class LANS:
@@ -85,6 +103,8 @@ class LANS:
         # `step` array (lans.py:228, :240): making a fresh device scalar from the host every step
         # would block on the previous step's kernels.
         self._step_dev = None
+        self._lists = None  # the w, m, v lists of all parameters, made on first use
+        self._model = None  # (data pointers, aliases of the half-precision parameters' data)
         params = list(params)
         halves = {x.dtype for x in params if isinstance(x, torch.Tensor)} & {torch.float16, torch.bfloat16}
         self.mixed = bool(halves)
@@ -98,15 +118,22 @@ class LANS:
 
     def step(self):
         """Update the parameters with gradients."""
-        g_list, x_list, m_list, v_list, p_list = [], [], [], [], []
-        for x, w, m, v in self.params:
-            if x.grad is None:
-                continue
-            g_list.append(x.grad)
-            x_list.append(w)
-            m_list.append(m)
-            v_list.append(v)
-            p_list.append(x.data)
+        params = self.params
+        grads = [x.grad for x, _, _, _ in params]
+        if any(g is None for g in grads):  # the reference skips parameters without a gradient (lans.py:81-83)
+            live = [i for i, g in enumerate(grads) if g is not None]
+            g_list = [grads[i] for i in live]
+            x_list = [params[i][1] for i in live]
+            m_list = [params[i][2] for i in live]
+            v_list = [params[i][3] for i in live]
+            p_list = [params[i][0].data for i in live] if self.mixed else []
+        else:
+            # The common case costs one attribute read per parameter: the state lists are the ones
+            # made at construction, and so are the aliases of the half-precision parameters' data
+            # (new ones only if a parameter's storage has been replaced since).
+            g_list = grads
+            x_list, m_list, v_list = self._state_lists()
+            p_list = self._model_data() if self.mixed else []
         if not x_list:
             self._advance()
             return
@@ -121,6 +148,18 @@ class LANS:
         else:
             _op.lans(tensor_list, step, *hyper)
         self._advance()
+
+    def _state_lists(self):
+        if self._lists is None:
+            self._lists = tuple([t[i] for t in self.params] for i in (1, 2, 3))
+        return self._lists
+
+    def _model_data(self):
+        xs = [t[0] for t in self.params]
+        ptrs = list(map(torch.Tensor.data_ptr, xs))
+        if self._model is None or self._model[0] != ptrs:
+            self._model = (ptrs, [x.data for x in xs])
+        return self._model[1]
 
     def _advance(self):
         self._step += 1

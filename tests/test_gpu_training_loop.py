@@ -88,3 +88,111 @@ def test_lans_training_follows_the_oracle(native_libs):
             assert np.max(np.abs(got - want) / np.maximum(np.abs(want), 1e-30)) <= 1e-5 * step, name
         # the next step starts from the model's own weights on both sides: one step at a time is compared
         ow = [p.detach().cpu().numpy().ravel().copy() for p in params]
+
+
+# ------------------------------------------------------------------ the optimizer objects' own bookkeeping
+def _lans_reference(g, w, m, v, step, **kw):
+    ow, om, ov, _ = lans_f64.lans_step(g, w, m, v, step, LansHParams(**kw))
+    return ow, om, ov
+
+
+def test_parameters_without_a_gradient_are_skipped(native_libs):
+    """Like the reference (python/raf/optim/lans.py:81-83, sgd.py:53-56): a parameter whose grad is
+    None is left out of the step, and joins again once it has one; the state of the others does
+    not care."""
+    from raf_amd import optim
+
+    rng = np.random.default_rng(7)
+    sizes = [1000, 77, 4097, 5]
+    init = [rng.normal(0, 0.02, n).astype(np.float32) for n in sizes]
+    grads = [rng.normal(0, 1e-3, n).astype(np.float32) for n in sizes]
+    params = [torch.from_numpy(a.copy()).to(DEV).requires_grad_() for a in init]
+    opt = optim.LANS(params)
+    for p, g in zip(params, grads):
+        p.grad = torch.from_numpy(g).to(DEV)
+    params[1].grad = None
+    opt.step()  # step 1 without parameter 1
+    params[1].grad = torch.from_numpy(grads[1]).to(DEV)
+    opt.step()  # step 2 with all four
+    torch.cuda.synchronize()
+    zeros = [np.zeros_like(a) for a in init]
+    live = [0, 2, 3]
+    w1, m1, v1 = _lans_reference([grads[i] for i in live], [init[i] for i in live], [zeros[i] for i in live],
+                                 [zeros[i] for i in live], 1)
+    w, m, v = list(init), list(zeros), list(zeros)
+    for j, i in enumerate(live):
+        w[i], m[i], v[i] = w1[j], m1[j], v1[j]
+    w2, _, _ = _lans_reference(grads, w, m, v, 2)
+    for p, want in zip(params, w2):
+        got = p.detach().cpu().numpy()
+        assert np.max(np.abs(got - want) / np.maximum(np.abs(want), 1e-12)) <= 1e-5
+
+    sgd_params = [torch.from_numpy(a.copy()).to(DEV).requires_grad_() for a in init]
+    sgd = optim.SGD(sgd_params, 0.1, 0.9)
+    for p, g in zip(sgd_params, grads):
+        p.grad = torch.from_numpy(g).to(DEV)
+    sgd_params[2].grad = None
+    sgd.step()
+    torch.cuda.synchronize()
+    assert np.array_equal(sgd_params[2].detach().cpu().numpy(), init[2])
+    assert not np.array_equal(sgd_params[0].detach().cpu().numpy(), init[0])
+
+
+def test_half_precision_model_whose_storage_is_replaced(native_libs):
+    """The optimizer keeps aliases of the half-precision parameters' data between steps; a parameter
+    whose storage has been swapped (x.data = ...) must receive the next weights in its new storage."""
+    from raf_amd import optim
+
+    torch.manual_seed(3)
+    params = [torch.randn(n, device=DEV).mul_(0.02).half().requires_grad_() for n in (3000, 17, 9000)]
+    opt = optim.LANS(params)
+    for p in params:
+        p.grad = (torch.randn(p.shape, device=DEV) * 1e-3).half()
+    opt.step()
+    old_storage = params[1].data
+    before = old_storage.clone()
+    params[1].data = params[1].data.clone()  # same values, new storage
+    opt.step()
+    torch.cuda.synchronize()
+    assert torch.equal(old_storage, before)  # the old storage is no longer written
+    master = opt.params[1][1]
+    assert torch.equal(params[1].data, master.half())  # the new one holds the narrowed master weight
+    assert not torch.equal(params[1].data, before)
+
+
+def test_optimizer_step_replayed_from_a_hip_graph(native_libs):
+    """A model of many small tensors is host-bound in eager mode (one attribute read and one address
+    check per tensor and step); captured once, `LANS.step()` replays with no Python at all and gives
+    the eager results."""
+    from raf_amd import optim, shapes
+
+    sizes = shapes.log_uniform_numels(300, seed=21)
+    torch.manual_seed(5)
+    init = [torch.randn(n, device=DEV).mul_(0.02) for n in sizes]
+    grads = [torch.randn(n, device=DEV).mul_(1e-3) for n in sizes]
+
+    def fresh():
+        ps = [t.clone().requires_grad_() for t in init]
+        for p, g in zip(ps, grads):
+            p.grad = g.clone()
+        return ps, optim.LANS(ps)
+
+    eager_params, eager = fresh()
+    for _ in range(6):
+        eager.step()
+    params, opt = fresh()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up: plan, tables and workspace exist before the capture
+        opt.step()
+        opt.step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        opt.step()  # step 3 is recorded, not run
+    for _ in range(4):  # replays: steps 3 to 6 (the step counter lives on the device)
+        graph.replay()
+    torch.cuda.synchronize()
+    for a, b in zip(params, eager_params):
+        assert torch.equal(a.detach(), b.detach())
