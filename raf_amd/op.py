@@ -133,6 +133,7 @@ def clear_op_env_cache() -> None:
     _env_cache.clear()
     _marshalled.clear()
     _slots.clear()
+    _sig_tokens.clear()
 
 
 class _Marshalled:
@@ -142,6 +143,9 @@ class _Marshalled:
         self.keep: list = []
         self.descs = (TensorDesc * max(len(tensors), 1))(*[_desc(t, self.keep) for t in tensors])
         self.sig = tuple(_sig(t) for t in tensors)
+        # A small number that stands for the signature in OpEnv keys: hashing a tuple of thousands
+        # of (shape, dtype, device) entries at every dictionary operation costs tens of microseconds.
+        self.sig_token = _sig_tokens.setdefault(self.sig, len(_sig_tokens))
         # Once one of the tensors has died its id may be handed to another object: the weak
         # references notice, and the entry is never trusted again.
         self.alive = True
@@ -160,8 +164,9 @@ class _Marshalled:
 
 
 _marshalled: Dict[Tuple, _Marshalled] = {}
+_sig_tokens: Dict[Tuple, int] = {}  # signature of a tensor list -> its number (never reused)
 _SLOTS_PER_SIGNATURE = 4
-_slots: Dict[Tuple, list] = {}  # signature -> identities (id tuples) of the lists seen, by slot
+_slots: Dict[int, list] = {}  # signature number -> identities (id tuples) of the lists seen, by slot
 
 
 def _marshal_list(tensors: list) -> _Marshalled:
@@ -174,7 +179,7 @@ def _marshal_list(tensors: list) -> _Marshalled:
         if len(_marshalled) >= 8:
             _marshalled.clear()
         m = _marshalled[key] = _Marshalled(tensors)
-        known = _slots.setdefault(m.sig, [])
+        known = _slots.setdefault(m.sig_token, [])
         if key not in known:
             if len(known) >= _SLOTS_PER_SIGNATURE:
                 known.pop()
@@ -382,7 +387,7 @@ def _sgd_multi(mixed, tensor_list, learning_rate, mu):
     n = len(tensor_list)
     m = _marshal_list(tensor_list)
     descs = m.descs
-    key = ("sgd_multi", mixed, m.sig, m.slot, float(mu))
+    key = ("sgd_multi", mixed, m.sig_token, m.slot, float(mu))
     env = _env_cache.get(key)
     if env is None:
         h = c_void_p(None)
@@ -430,7 +435,7 @@ def _lans(op_name, tensor_list, step, learning_rate, beta1, beta2, eps, bias_cor
     # All but the learning rate and the loss scaling.  `m.slot` tells lists of equal signature
     # apart (two models of one architecture): each keeps an OpEnv, and with it a plan whose device
     # pointer table follows that list alone.
-    key = (op_name, m.sig, m.slot, _sig(step), hp[1:])
+    key = (op_name, m.sig_token, m.slot, _sig(step), hp[1:])
     env = _env_cache.get(key)
     if env is None:
         h = c_void_p(None)
