@@ -76,6 +76,39 @@ def test_order_invariants(native_libs, group):
         _check(kernels.pipeline_order(sizes, group), sizes, lib)
 
 
+def test_order_invariants_on_random_lists(native_libs):
+    """The same invariants over a few hundred random lists: every mix of empty, one-chunk, small-chunk,
+    large-chunk and cache-exceeding tensors, with random cache-group sizes."""
+    import numpy as np
+
+    from raf_amd import kernels
+
+    lib = native_libs.optim()
+    rng = np.random.default_rng(31)
+    for case in range(300):
+        n = int(rng.integers(1, 25))
+        kinds = rng.integers(0, 6, n)
+        sizes = []
+        for k in kinds:
+            if k == 0:
+                sizes.append(int(rng.integers(0, 3)))                    # empty or tiny
+            elif k == 1:
+                sizes.append(int(rng.integers(1, 4097)))                 # one chunk
+            elif k == 2:
+                sizes.append(int(rng.integers(4097, 1 << 19)))           # small chunks
+            elif k == 3:
+                sizes.append(int(rng.integers(1 << 19, 6_000_000)))      # large chunks
+            elif k == 4:
+                sizes.append(int(rng.integers(6_000_000, 22_000_000)))   # long, still cached
+            else:
+                sizes.append(int(rng.integers(22_400_000, 60_000_000)))  # streamed
+        group = int(rng.choice([0, 1, 50_000, 3_000_000, 13_000_000, 10**12]))
+        try:
+            _check(kernels.pipeline_order(sizes, group), sizes, lib)
+        except AssertionError as e:
+            raise AssertionError(f"case {case}: sizes {sizes}, group {group}: {e}") from e
+
+
 def test_groups_bound_the_reuse_distance(native_libs):
     """Between a tensor's pass-A chunks and its pass-C chunks lie at most a few groups' worth of
     other tensors' work, which is what keeps the tensor in the Infinity Cache."""
