@@ -361,6 +361,10 @@ def test_random_lists_groupings_and_slicings_agree_bitwise(native_libs, monkeypa
                 monkeypatch.setenv("RAFHIP_LANS_GROUP_ELEMS", str(int(rng.choice([1, 50_000, 400_000, 3_000_000]))))
                 monkeypatch.setenv("RAFHIP_LANS_ROUND_SLICES", str(int(rng.choice([1, 2, 8, 64, 4096]))))
                 monkeypatch.setenv("RAFHIP_LANS_BLOCKS_PER_CU", str(int(rng.choice([1, 2, 3]))))
+                # tensors from this size on are treated as too large for the cache: their items are
+                # marked streaming and merged into the list of the cached groups
+                monkeypatch.setenv("RAFHIP_LANS_STREAM_FROM_ELEMS", str(int(rng.choice([50_000, 600_000, 10**9]))))
+                monkeypatch.setenv("RAFHIP_LANS_STREAM_HOLD_ITEMS", str(int(rng.choice([0, 7, 3072]))))
             tg, tw, tm, tv = _to_dev(g), _to_dev(w), _to_dev(m), _to_dev(v)
             plan = kernels.LansPlan(sizes, tg[0].dtype, DEV)
             plan.set_schedule(schedule)

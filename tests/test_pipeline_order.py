@@ -22,7 +22,7 @@ def _normalise(order):
     return out, streamed
 
 
-def _check(order, sizes, lib):
+def _check(order, sizes, lib, stream_from=(256 << 20) // 12):
     # a tensor's chunk size (and first-pass unit) depends on its own element count
     n_chunks = [-(-n // lib.rafhip_lans_chunk_elements(n)) for n in sizes]
     n_units = [-(-n // lib.rafhip_lans_pass_a_unit_elements(n)) for n in sizes]
@@ -33,7 +33,7 @@ def _check(order, sizes, lib):
         assert (kind, t, c) not in seen, "duplicate work item"
         seen[(kind, t, c)] = pos
     for t in streamed:
-        assert sizes[t] * 12 >= 256 << 20, "only tensors beyond the cache are streamed"
+        assert sizes[t] >= stream_from, "only tensors beyond the cache are streamed"
     for t, nc in enumerate(n_chunks):
         if nc == 0:
             continue
@@ -76,9 +76,10 @@ def test_order_invariants(native_libs, group):
         _check(kernels.pipeline_order(sizes, group), sizes, lib)
 
 
-def test_order_invariants_on_random_lists(native_libs):
+def test_order_invariants_on_random_lists(native_libs, monkeypatch):
     """The same invariants over a few hundred random lists: every mix of empty, one-chunk, small-chunk,
-    large-chunk and cache-exceeding tensors, with random cache-group sizes."""
+    large-chunk and cache-exceeding tensors, with random cache-group sizes, streaming thresholds and
+    hold lengths."""
     import numpy as np
 
     from raf_amd import kernels
@@ -103,8 +104,11 @@ def test_order_invariants_on_random_lists(native_libs):
             else:
                 sizes.append(int(rng.integers(22_400_000, 60_000_000)))  # streamed
         group = int(rng.choice([0, 1, 50_000, 3_000_000, 13_000_000, 10**12]))
+        stream_from = int(rng.choice([(256 << 20) // 12, 30_000, 1_000_000, 10**12]))
+        monkeypatch.setenv("RAFHIP_LANS_STREAM_FROM_ELEMS", str(stream_from))
+        monkeypatch.setenv("RAFHIP_LANS_STREAM_HOLD_ITEMS", str(int(rng.choice([0, 3, 3072, 10**6]))))
         try:
-            _check(kernels.pipeline_order(sizes, group), sizes, lib)
+            _check(kernels.pipeline_order(sizes, group), sizes, lib, stream_from)
         except AssertionError as e:
             raise AssertionError(f"case {case}: sizes {sizes}, group {group}: {e}") from e
 
