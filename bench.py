@@ -73,6 +73,7 @@ def kernel_sources_digest() -> str:
 
 
 _TRAFFIC_LINE = re.compile(r"^traffic: workload=(\S+) kernel=(\S+) bytes_per_launch=(\d+) kernel_sources=(\w+)\s*$")
+_NO_TRAFFIC_LINE = re.compile(r"^no traffic figure: workload=(\S+) reason=(.+)$")
 
 
 def measured_traffic(workload: str, kernel: str):
@@ -92,6 +93,9 @@ def measured_traffic(workload: str, kernel: str):
                 if m.group(4) == now:
                     return int(m.group(3)), f"profiles/{md.name} (rocprofv3 FETCH_SIZE + WRITE_SIZE, kernel sources {now})"
                 stale = f"profiles/{md.name} holds a figure for other kernel sources ({m.group(4)}, tree is {now}): not quoted"
+            m = _NO_TRAFFIC_LINE.match(line.strip())
+            if m and m.group(1) == workload and stale is None:
+                stale = f"not measured: {m.group(2)} (profiles/{md.name})"
     return None, stale or "not measured"
 
 
