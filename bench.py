@@ -133,6 +133,8 @@ def workloads():
         "sgd_multi_bert_large_fp32": dict(kind="sgd_multi", sizes=shapes.numels(shapes.bert_large_shapes())),
         # the traced optimizer's per-parameter op sequence after dialect fusion: one multi-tensor call
         "traced_sgd_fused_bert_large_fp32": dict(kind="traced_sgd", sizes=shapes.numels(shapes.bert_large_shapes())),
+        # the traced LANS optimizer of a half-precision model after the graph rewrite: one lans_mixed call
+        "traced_lans_mixed_bert_large_fp16": dict(kind="traced_lans", sizes=shapes.numels(shapes.bert_large_shapes())),
         # neighbours of the optimizer step that reuse its machinery
         "l2norm_bert_large_flat_fp32": dict(kind="l2norm", n=sum(shapes.numels(shapes.bert_large_shapes()))),
         "fuse_bert_large_fp32": dict(kind="fuse", sizes=shapes.numels(shapes.bert_large_shapes()), gather=True),
@@ -711,6 +713,42 @@ def bench_traced_sgd(name, wl, args):
     return res
 
 
+def bench_traced_lans(name, wl, args):
+    """One step = the optimizer part of the reference's traced LANS optimizer for a half-precision
+    model (group_cast, raf.op.lans, and per parameter cast + add(out=p)), taken through the
+    FuseDialect pass: the hip dialect's graph rewrite folds all of it into one raf.op.hip.lans_mixed
+    call, executed through the C window; the step counter is advanced on the device."""
+    import torch
+
+    from raf_amd import op
+
+    dev = torch.device("cuda:0")
+    sizes = wl["sizes"]
+    total = sum(sizes)
+    g, w, m, v = gen_lans(sizes, True, True, dev)
+    p16 = [torch.empty(n, dtype=torch.float16, device=dev) for n in sizes]
+    step_t = torch.full((), 1.0, dtype=torch.float32, device=dev)
+    op.set_lans_grad_unscale(1.0 / 1024)
+    opt = op.TracedLansOptimizer(g, w, m, v, p16, step_t)
+    calls = opt.ops
+
+    def one_step(i):
+        opt()
+        step_t.add_(1.0)
+
+    wall_ms, dev_ms = _timed(one_step, args)
+    op.set_lans_grad_unscale(1.0)
+    a, b, c = lans_bytes_per_elt(2)
+    bytes_step = total * (a + b + c + 2)
+    res = _line("traced mixed-precision LANS optimizer after the dialect's graph rewrite: algorithmic bandwidth "
+                "(48 B per element / step time)", name, "f64", bytes_step, wall_ms, dev_ms,
+                "lans step (all launches)", args,
+                {"tensors": len(sizes), "elements": total, "bytes_per_element": a + b + c + 2,
+                 "calls_in_fused_graph": calls,
+                 "unfused_ops_per_step": 2 + 2 * len(sizes)})
+    return res
+
+
 def _config_entry(line):
     """What the "configs" block keeps of a workload's full line."""
     cfg, roof = line["config"], line["roofline"]
@@ -831,7 +869,7 @@ def main():
             out = bench_sgd(args.workload, wl, args, parity=not args.no_parity)
         else:
             fn = {"copy": bench_copy, "l2norm": bench_l2norm, "fuse": bench_fuse, "sgd_multi": bench_sgd_multi,
-                  "traced_sgd": bench_traced_sgd}[wl["kind"]]
+                  "traced_sgd": bench_traced_sgd, "traced_lans": bench_traced_lans}[wl["kind"]]
             out = fn(args.workload, wl, args)
     print(json.dumps(out), flush=True)
     parity = out.get("parity")

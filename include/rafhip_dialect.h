@@ -215,7 +215,9 @@ int rafhip_raf_env_set_learning_rate(rafhip_raf_env* env, double learning_rate);
  * _set_dynamic_scale: device-resident one-element float32 tensors holding that factor (the
  * reciprocal of the current loss scale) and an overflow flag; the kernels read them when they
  * start, and a non-zero flag turns the step into a no-op.  Either descriptor may be NULL.  None
- * of this identifies the OpEnv: a scale change keeps the OpEnv, its plan and its tables. */
+ * of this identifies the OpEnv: a scale change keeps the OpEnv, its plan and its tables.  On the
+ * env of a traced optimizer (rafhip_raf_traced_optimizer_make) they reach every call of the graph
+ * that takes a gradient scale. */
 int rafhip_raf_env_set_grad_unscale(rafhip_raf_env* env, float factor);
 int rafhip_raf_env_set_dynamic_scale(rafhip_raf_env* env, const rafhip_tensor_desc* grad_unscale,
                                      const rafhip_tensor_desc* found_inf);

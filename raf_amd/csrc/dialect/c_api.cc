@@ -975,6 +975,11 @@ int rafhip_raf_env_set_learning_rate(rafhip_raf_env* env, double learning_rate) 
 int rafhip_raf_env_set_grad_unscale(rafhip_raf_env* env, float factor) {
   return Guard([&] {
     if (!env) throw Error("rafhip_raf_env_set_grad_unscale: env is NULL");
+    if (!env->graph_calls.empty()) {  // a traced optimizer: every call of the graph that takes one
+      for (auto& gc : env->graph_calls)
+        if (auto* t = dynamic_cast<hip::HasGradScaling*>(gc.env.get())) t->SetGradUnscale(factor);
+      return;
+    }
     if (!env->env) return;  // declared as a no-op
     auto* target = dynamic_cast<hip::HasGradScaling*>(env->env.get());
     if (!target) throw Error("rafhip_raf_env_set_grad_unscale: " + env->name + " takes no gradient scale");
@@ -986,9 +991,10 @@ int rafhip_raf_env_set_dynamic_scale(rafhip_raf_env* env, const rafhip_tensor_de
                                      const rafhip_tensor_desc* found_inf) {
   return Guard([&] {
     if (!env) throw Error("rafhip_raf_env_set_dynamic_scale: env is NULL");
-    if (!env->env) return;  // declared as a no-op
-    auto* target = dynamic_cast<hip::HasGradScaling*>(env->env.get());
-    if (!target) throw Error("rafhip_raf_env_set_dynamic_scale: " + env->name + " takes no gradient scale");
+    const bool graph = !env->graph_calls.empty();
+    if (!graph && !env->env) return;  // declared as a no-op
+    auto* target = graph ? nullptr : dynamic_cast<hip::HasGradScaling*>(env->env.get());
+    if (!graph && !target) throw Error("rafhip_raf_env_set_dynamic_scale: " + env->name + " takes no gradient scale");
     auto word = [&](const rafhip_tensor_desc* d, const char* what) -> const float* {
       if (!d) return nullptr;
       const TensorView t = FromDesc(d, what)->tensor;
@@ -998,7 +1004,14 @@ int rafhip_raf_env_set_dynamic_scale(rafhip_raf_env* env, const rafhip_tensor_de
         throw Error(std::string(what) + " must live on the OpEnv's device");
       return static_cast<const float*>(t.data);
     };
-    target->SetDynamicScale(word(grad_unscale, "grad_unscale"), word(found_inf, "found_inf"));
+    const float* unscale_word = word(grad_unscale, "grad_unscale");
+    const float* found_inf_word = word(found_inf, "found_inf");
+    if (graph) {
+      for (auto& gc : env->graph_calls)
+        if (auto* t = dynamic_cast<hip::HasGradScaling*>(gc.env.get())) t->SetDynamicScale(unscale_word, found_inf_word);
+      return;
+    }
+    target->SetDynamicScale(unscale_word, found_inf_word);
   });
 }
 

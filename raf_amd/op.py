@@ -309,6 +309,8 @@ class _TracedOptimizer:
 
     def __call__(self):
         stream = _stream(self._first)
+        if self._KIND == 1:  # the loss scaling in force reaches the LANS call of the graph
+            self._env.set_grad_scaling(_lans_grad_unscale, _lans_dynamic_scale)
         ws = _workspace(self._env, self._first, stream) if self._env.workspace_bytes > 0 else None
         check_raf(self._execute(self._env.handle, self._n, *self._descs, self._step, self._allow_partial,
                                 ws.data if ws else None, self._env.workspace_bytes, stream))

@@ -149,3 +149,44 @@ def test_traced_lans_with_a_free_zero_tensor_folds_the_group_cast_only(native_li
         assert max_rel_err(tw[t].cpu().numpy(), ow[t]) <= 1e-5
         assert max_rel_err(tm[t].cpu().numpy(), om[t]) <= 1e-5
         assert max_rel_err(tv[t].cpu().numpy(), ov[t]) <= 1e-5
+
+
+def test_traced_lans_optimizer_takes_the_loss_scaling_in_force(native_libs):
+    """The loss scaling set for LANS calls reaches the lans_mixed call inside a traced optimizer's
+    graph: a static inverse scale, then a device-resident one with an overflow flag that skips a step."""
+    from raf_amd import op
+
+    sizes = [int(np.prod(s)) for s in SHAPES]
+    g, w, m, v = lans_inputs(sizes, cfg=314, g16=True, loss_scale=1024.0)
+    tg, tw, tm, tv = ([_dev(a) for a in x] for x in (g, w, m, v))
+    tp = [torch.zeros(n, dtype=torch.float16, device=DEV) for n in sizes]
+    step = torch.ones((), device=DEV)
+    opt = op.TracedLansOptimizer(tg, tw, tm, tv, tp, step)
+    hp = LansHParams(grad_unscale=1.0 / 1024)
+    try:
+        op.set_lans_grad_unscale(1.0 / 1024)
+        opt()
+        torch.cuda.synchronize()
+        ow, om, ov, _ = lans_f64.lans_step(g, w, m, v, 1, hp)
+        for t in range(len(sizes)):
+            assert max_rel_err(tw[t].cpu().numpy(), ow[t]) <= 1e-5
+        # dynamic: the scale word says 1/1024 too, the flag skips step 2, step 3 runs as step 2 would
+        op.set_lans_grad_unscale(1.0)
+        inv_scale = torch.full((), 1.0 / 1024, device=DEV)
+        found_inf = torch.ones((), device=DEV)
+        op.set_lans_dynamic_scale(inv_scale, found_inf)
+        step.fill_(2.0)
+        before = [t.clone() for t in tw + tm + tv + tp]
+        opt()
+        torch.cuda.synchronize()
+        assert all(torch.equal(a, b) for a, b in zip(before, tw + tm + tv + tp))
+        found_inf.zero_()
+        opt()
+        torch.cuda.synchronize()
+        ow2, _, _, _ = lans_f64.lans_step(g, ow, om, ov, 2, hp)
+        for t in range(len(sizes)):
+            assert max_rel_err(tw[t].cpu().numpy(), ow2[t]) <= 1e-5
+            assert torch.equal(tp[t], tw[t].half())
+    finally:
+        op.set_lans_grad_unscale(1.0)
+        op.set_lans_dynamic_scale(None, None)
