@@ -632,7 +632,8 @@ def bench_fuse(name, wl, args):
     wall_ms, dev_ms = _timed(step, args)
     moved = 2 * plan.total_bytes
     res = _line(f"{what} achieved HBM bandwidth (bytes read + written / time)", name, "u8", moved, wall_ms, dev_ms,
-                kernel, args, {"tensors": len(sizes), "bytes_read_per_step": plan.total_bytes,
+                kernel, args, {"tensors": len(sizes), "elements": sum(sizes), "bytes_per_element": 8,
+                               "bytes_read_per_step": plan.total_bytes,
                                "bytes_written_per_step": plan.total_bytes, "launches_per_step": 1})
     if not args.no_cpu_baseline:
         from oracle import tensor_ops
@@ -822,6 +823,32 @@ def run_suite(table, args):
         via["overhead_vs_c_abi_us"] = round((via["ms_per_step"] - direct["ms_per_step"]) * 1e3, 1)
         via["overhead_vs_c_abi_pct"] = round(100 * (via["ms_per_step"] / direct["ms_per_step"] - 1), 2)
     out["configs"] = configs
+
+    # The callers and neighbours either side of the path, timed in the same run (no parity here:
+    # the GPU tests pin their bits): the traced optimizers after the dialect's graph rewrites beside
+    # the C-ABI calls they end in, and the list operators.
+    neighbours = {}
+    quick = copy.copy(args)
+    quick.no_cpu_baseline = True
+    for name in ("sgd_multi_bert_large_fp32", "traced_sgd_fused_bert_large_fp32", "lans_bert_large_mixed_fp16",
+                 "traced_lans_mixed_bert_large_fp16", "l2norm_bert_large_flat_fp32", "fuse_bert_large_fp32",
+                 "defuse_bert_large_fp32"):
+        wl = table[name]
+        if wl["kind"] == "lans":
+            line = bench_lans(name, wl, quick, parity=False, cpu_baseline=False)
+        else:
+            fn = {"l2norm": bench_l2norm, "fuse": bench_fuse, "sgd_multi": bench_sgd_multi,
+                  "traced_sgd": bench_traced_sgd, "traced_lans": bench_traced_lans}[wl["kind"]]
+            line = fn(name, wl, quick)
+        neighbours[name] = _config_entry(line)
+        if "calls_in_fused_graph" in line["config"]:
+            neighbours[name]["calls_in_fused_graph"] = line["config"]["calls_in_fused_graph"]
+        release()
+    for traced, direct in (("traced_sgd_fused_bert_large_fp32", "sgd_multi_bert_large_fp32"),
+                           ("traced_lans_mixed_bert_large_fp16", "lans_bert_large_mixed_fp16")):
+        neighbours[traced]["overhead_vs_c_abi_pct"] = round(
+            100 * (neighbours[traced]["ms_per_step"] / neighbours[direct]["ms_per_step"] - 1), 2)
+    out["neighbours"] = neighbours
     parity["ok"] = all(p is None or p.get("ok", False) for p in parity.values())
     out["parity"] = parity
     return out
