@@ -349,16 +349,37 @@ def bench_lans(name, wl, args, entry="c_abi", parity=True, cpu_baseline=True):
             step_t.add_(1.0)  # the step counter lives on the device, as in the reference's traced optimizer
     else:
         # raf.op.lans(tensor_list, step, ...) as the reference's LANS.step calls it
-        # (python/raf/optim/lans.py:74-103): schema -> declare -> dialect dispatch -> OpEnv -> Execute
+        # (python/raf/optim/lans.py:74-103): schema -> declare -> dialect dispatch -> OpEnv -> Execute.
+        #   dialect              the list as a TensorList handle (the tuple value RAF's callers hold)
+        #   dialect_list         a plain Python list of the same tensor objects every step
+        #   dialect_fresh_grads  a plain list whose gradient objects are new at every step (same storage)
+        #   vm_fresh_tuple       Execute receives a NEW TupleValue over the same tensor values at every
+        #                        step, as the VM allocates one per iteration (src/impl/vm/vm.cc:764-769)
+        #   vm_moving_grads      that, and the gradients alternate between two allocations every step,
+        #                        as per-iteration allocation gives them (vm.cc:1099-1105)
         if args.schedule != "auto":
             os.environ["RAFHIP_LANS_SCHEDULE"] = args.schedule
         op.clear_op_env_cache()
         op.set_lans_grad_unscale(hp.grad_unscale)
-        tensor_list = g + w + m + v + (p16 or [])
+        op.set_executor("vm" if entry.startswith("vm_") else "interpreter")
+        rest = w + m + v + (p16 or [])
         call = op.lans_mixed if copy16 else op.lans
         schedule = args.schedule
+        if entry == "dialect_list":
+            lists = [g + rest]
+        elif entry == "dialect_fresh_grads":
+            # new tensor objects over the same gradient storage for every step, made before the clock starts
+            lists = [[t.detach() for t in g] + rest for _ in range(args.warmup + args.steps + 4)]
+        elif entry == "vm_moving_grads":
+            first = op.TensorList(g + rest)
+            lists = [first, first.replaced(0, [t.clone() for t in g])]  # same values at another address
+        else:
+            lists = [op.TensorList(g + rest)]
+        calls_made = [0]
 
         def one_step():
+            tensor_list = lists[calls_made[0] % len(lists)]
+            calls_made[0] += 1
             call(tensor_list, step_t, hp.learning_rate, hp.beta1, hp.beta2, hp.eps, True, hp.weight_decay,
                  True, True, True)
             step_t.add_(1.0)
@@ -462,6 +483,7 @@ def bench_lans(name, wl, args, entry="c_abi", parity=True, cpu_baseline=True):
         out["parity"] = checker.check(steps_done, g, w, m, v, one_step)
     if entry != "c_abi":
         op.set_lans_grad_unscale(1.0)
+        op.set_executor("interpreter")
         op.clear_op_env_cache()
         os.environ.pop("RAFHIP_LANS_SCHEDULE", None)
     if plan is not None:
@@ -750,30 +772,47 @@ def bench_traced_lans(name, wl, args):
     return res
 
 
+def _short_traffic_source(source: str) -> str:
+    """One token for the line the driver keeps; the full sentence is in profiles/ and DESIGN.md."""
+    if "other kernel sources" in source:
+        return "stale"
+    if source.startswith("profiles/"):
+        return source.split(" ")[0]
+    return "unmeasured"
+
+
 def _config_entry(line):
-    """What the "configs" block keeps of a workload's full line."""
+    """What the "configs" block keeps of a workload's full line: step time, the dominant kernel and
+    its time from HIP events, and its fraction of the 8 TB/s peak by algorithmic bytes (`frac`), by
+    compulsory bytes (`frac_c`: every operand read once, every result written once) and by the
+    traffic rocprofv3 measured (`traffic`, bytes per launch, or null)."""
     cfg, roof = line["config"], line["roofline"]
     comp = cfg.get("compulsory_bytes_per_element")
     launch_s = roof["avg_launch_ms"] * 1e-3
-    entry = {
-        "entry": cfg.get("entry", "c_abi"), "elements": cfg["elements"], "tensors": cfg.get("tensors", 1),
-        "schedule": cfg.get("schedule"), "ms_per_step": line["ms_per_step"], "steps": line["steps"],
-        "algorithmic_GBps": line["value"], "bytes_per_element": cfg["bytes_per_element"],
-        "kernel": roof["kernel"], "kernel_ms": roof["avg_launch_ms"],
-        "frac_by_algorithmic_bytes": roof["frac"],
-        "frac_by_compulsory_bytes": roof.get("frac_by_compulsory_bytes"),
-        "traffic": roof["traffic"], "traffic_source": roof["traffic_source"],
-    }
-    if entry["frac_by_compulsory_bytes"] is None and comp and roof["kernel"] not in ("lans_apply",):
-        entry["frac_by_compulsory_bytes"] = round(cfg["elements"] * comp / launch_s / 1e9 / HBM_PEAK_GBPS, 4)
-    if "kernels_ms" in line:
+    entry = {"ms": line["ms_per_step"], "kernel": roof["kernel"], "kernel_ms": roof["avg_launch_ms"],
+             "frac": roof["frac"], "frac_c": roof.get("frac_by_compulsory_bytes"), "traffic": roof["traffic"]}
+    if entry["frac_c"] is None and comp and roof["kernel"] not in ("lans_apply",):
+        entry["frac_c"] = round(cfg["elements"] * comp / launch_s / 1e9 / HBM_PEAK_GBPS, 4)
+    if "kernels_ms" in line and cfg.get("schedule") == "phased":
         entry["kernels_ms"] = line["kernels_ms"]
     return entry
 
 
+def _parity_entry(p):
+    if p is None:
+        return None
+    if "w" not in p:  # SGD: bit-exact
+        return {"ok": p["ok"], "n": p["elements_checked"], "ne": p["not_bit_equal"]}
+    return {"ok": p["ok"], "n": p["elements_checked"], "tol": p["tolerance"],
+            "max_rel": max(p[q]["max_rel"] for q in "wmv"), "over_tol": sum(p[q]["over_tol"] for q in "wmv"),
+            "ne": sum(p[q]["not_bit_equal"] for q in "wmv")}
+
+
 def run_suite(table, args):
     """Every benchmark configuration in one process, one after the other, each with its parity
-    check; the headline workload first, and its line is the one whose fields go to the top level."""
+    check; the headline workload first, and its line is the one whose fields go to the top level.
+    The line stays well under 8 KB so that a log tail of that size holds all of it; per-workload
+    detail is printed by `--workload NAME`."""
     import copy
     import gc
 
@@ -786,7 +825,14 @@ def run_suite(table, args):
     headline = "lans_bert_large_fp16grad"
     out = bench_lans(headline, table[headline], args, entry="c_abi", parity=True, cpu_baseline=True)
     configs = {headline: _config_entry(out)}
-    parity = {headline: out.pop("parity", None)}
+    parity = {headline: _parity_entry(out.pop("parity", None))}
+    out["roofline"]["traffic_source"] = _short_traffic_source(out["roofline"]["traffic_source"])
+    out["config"] = {k: out["config"][k] for k in ("workload", "entry", "tensors", "elements", "bytes_per_element",
+                                                   "kernel_bytes_per_element", "compulsory_bytes_per_element",
+                                                   "schedule", "launches_per_step")}
+    out["metric"] = "LANS optimizer step, algorithmic bandwidth (46 B per element by the three-pass model / step time)"
+    if "cpu_baseline" in out:
+        out["cpu_baseline"]["sample"] = out["cpu_baseline"]["sample"].split(", float64")[0]
     release()
 
     def more_steps(k):
@@ -797,32 +843,40 @@ def run_suite(table, args):
     def add(name, line):
         configs[name] = _config_entry(line)
         if "parity" in line:
-            parity[name] = line["parity"]
+            parity[name] = _parity_entry(line["parity"])
         release()
 
-    # the operator front end on the headline list: raf.op.lans -> dialect dispatch -> OpEnv -> Execute
-    line = bench_lans(headline, table[headline], args, entry="dialect", parity=True, cpu_baseline=False)
-    add(headline + "@dialect", line)
     add("sgd_4m_fp32", bench_sgd("sgd_4m_fp32", table["sgd_4m_fp32"], more_steps(4), parity=True, cpu_baseline=False))
     add("lans_bert_base_fp32", bench_lans("lans_bert_base_fp32", table["lans_bert_base_fp32"], args, cpu_baseline=False))
     small = "lans_2000_small_tensors"
-    quiet = copy.copy(args)
-    quiet.no_kernel_events = True  # per-kernel events cost a fifth of this 0.1 ms step
-    line = bench_lans(small, table[small], more_steps(4), cpu_baseline=False)
-    add(small, line)
-    quiet.steps = line["steps"]
-    add(small + "@c_abi_no_events", bench_lans(small, table[small], quiet, parity=False, cpu_baseline=False))
-    add(small + "@dialect", bench_lans(small, table[small], quiet, entry="dialect", cpu_baseline=False))
+    add(small, bench_lans(small, table[small], more_steps(4), cpu_baseline=False))
     big = copy.copy(args)
-    big.steps, big.warmup = min(args.steps, 20), min(args.warmup, 5)  # 11.5 ms per step, 25 GB resident
+    big.steps, big.warmup = min(args.steps, 20), min(args.warmup, 5)  # 10 ms per step, 25 GB resident
     add("lans_gpt2_1p5b_fp32", bench_lans("lans_gpt2_1p5b_fp32", table["lans_gpt2_1p5b_fp32"], big, cpu_baseline=False))
-
-    for base in (headline, small):
-        direct = configs[base + "@c_abi_no_events"] if base == small else configs[base]
-        via = configs[base + "@dialect"]
-        via["overhead_vs_c_abi_us"] = round((via["ms_per_step"] - direct["ms_per_step"]) * 1e3, 1)
-        via["overhead_vs_c_abi_pct"] = round(100 * (via["ms_per_step"] / direct["ms_per_step"] - 1), 2)
     out["configs"] = configs
+
+    # The ways into the same step, ms per step each and percent over the C ABI (no per-kernel events
+    # in either, they cost a fifth of the 0.1 ms step): the operator front end with a TensorList
+    # handle, with a plain list, with new gradient objects every step, and the VM's calling pattern.
+    quiet = copy.copy(args)
+    quiet.no_kernel_events = True
+    entries = {}
+    for base, steps_factor, variants in (
+            (headline, 1, ("dialect", "vm_fresh_tuple", "vm_moving_grads")),
+            (small, 4, ("dialect", "dialect_list", "dialect_fresh_grads", "vm_fresh_tuple", "vm_moving_grads"))):
+        quiet.steps = max(1, int(args.steps * steps_factor))
+        direct = bench_lans(base, table[base], quiet, parity=False, cpu_baseline=False)["ms_per_step"]
+        release()
+        block = {"c_abi": direct}
+        for entry in variants:
+            line = bench_lans(base, table[base], quiet, entry=entry, parity=entry != "dialect_list", cpu_baseline=False)
+            block[entry] = line["ms_per_step"]
+            block[entry + "_pct"] = round(100 * (line["ms_per_step"] / direct - 1), 1)
+            if "parity" in line:
+                parity[f"{base}@{entry}"] = _parity_entry(line["parity"])
+            release()
+        entries[base] = block
+    out["entries"] = entries
 
     # The callers and neighbours either side of the path, timed in the same run (no parity here:
     # the GPU tests pin their bits): the traced optimizers after the dialect's graph rewrites beside
@@ -840,14 +894,8 @@ def run_suite(table, args):
             fn = {"l2norm": bench_l2norm, "fuse": bench_fuse, "sgd_multi": bench_sgd_multi,
                   "traced_sgd": bench_traced_sgd, "traced_lans": bench_traced_lans}[wl["kind"]]
             line = fn(name, wl, quick)
-        neighbours[name] = _config_entry(line)
-        if "calls_in_fused_graph" in line["config"]:
-            neighbours[name]["calls_in_fused_graph"] = line["config"]["calls_in_fused_graph"]
+        neighbours[name] = {"ms": line["ms_per_step"], "frac": line["roofline"]["frac"]}
         release()
-    for traced, direct in (("traced_sgd_fused_bert_large_fp32", "sgd_multi_bert_large_fp32"),
-                           ("traced_lans_mixed_bert_large_fp16", "lans_bert_large_mixed_fp16")):
-        neighbours[traced]["overhead_vs_c_abi_pct"] = round(
-            100 * (neighbours[traced]["ms_per_step"] / neighbours[direct]["ms_per_step"] - 1), 2)
     out["neighbours"] = neighbours
     parity["ok"] = all(p is None or p.get("ok", False) for p in parity.values())
     out["parity"] = parity
@@ -861,8 +909,13 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="all",
                     help="a workload name, or 'all' (default): the headline line plus every configuration and parity")
-    ap.add_argument("--entry", default="c_abi", choices=["c_abi", "dialect"],
-                    help="LANS workloads: call the C ABI (bound plan) or the operator front end raf_amd.op.lans")
+    ap.add_argument("--entry", default="c_abi",
+                    choices=["c_abi", "dialect", "dialect_list", "dialect_fresh_grads", "vm_fresh_tuple",
+                             "vm_moving_grads"],
+                    help="LANS workloads: call the C ABI (bound plan), or the operator front end raf_amd.op.lans "
+                         "with a TensorList handle (dialect), a plain list, a list with new gradient objects "
+                         "every step, or the way RAF's VM calls an OpEnv (a new tuple value every step; "
+                         "gradients alternating between two allocations)")
     ap.add_argument("--schedule", default="auto", choices=["auto", "phased", "pipelined"],
                     help="LANS launch schedule (bit-identical results); auto = the library's choice")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline leg")

@@ -74,6 +74,28 @@ int rafhip_raf_lans_execute(rafhip_raf_env* env, int32_t list_len,
                             const rafhip_tensor_desc* tensor_list, const rafhip_tensor_desc* step,
                             void* workspace, int64_t workspace_bytes, void* stream);
 
+/* A tensor list held as a value: RAF's TupleValue of TensorValues (include/raf/value.h), which is
+ * what its executors keep between calls -- the interpreter in the argument object, the VM in its
+ * registers (src/impl/vm/vm.cc:764-769) -- so that no call converts the list again.  Immutable.
+ * _replace makes a new tuple that shares every field of `base` except [first, first + count),
+ * which are made from `fields`: one step's list against the previous one when only the gradients
+ * were allocated anew. */
+typedef struct rafhip_raf_tuple rafhip_raf_tuple;
+int rafhip_raf_tuple_make(int32_t n, const rafhip_tensor_desc* fields, rafhip_raf_tuple** tuple_out);
+int rafhip_raf_tuple_replace(const rafhip_raf_tuple* base, int32_t first, int32_t count,
+                             const rafhip_tensor_desc* fields, rafhip_raf_tuple** tuple_out);
+int32_t rafhip_raf_tuple_size(const rafhip_raf_tuple* tuple); /* -1 on NULL */
+int rafhip_raf_tuple_destroy(rafhip_raf_tuple* tuple);
+/* rafhip_raf_lans_execute / rafhip_raf_sgd_multi_execute on a tuple made beforehand.  as_vm != 0
+ * hands Execute a NEW TupleValue over the same tensor values, which is what the VM does at every
+ * iteration (vm.cc:764-769 allocates the tuple afresh from its registers); 0 hands over the
+ * tuple itself, as the interpreter does with the call's argument. */
+int rafhip_raf_lans_execute_tuple(rafhip_raf_env* env, const rafhip_raf_tuple* tensor_list,
+                                  const rafhip_tensor_desc* step, void* workspace,
+                                  int64_t workspace_bytes, void* stream, int32_t as_vm);
+int rafhip_raf_sgd_multi_execute_tuple(rafhip_raf_env* env, const rafhip_raf_tuple* tensor_list,
+                                       void* stream, int32_t as_vm);
+
 /* Extension ops raf.op.sgd_multi(tensor_list, learning_rate, mu) with tensor_list = x..., dx...,
  * v... (3n descriptors) and raf.op.sgd_multi_mixed with a fourth block p... (the model's float16 /
  * bfloat16 parameters): momentum SGD over the whole list, in place on x and v, per element the

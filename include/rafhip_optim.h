@@ -182,6 +182,14 @@ int64_t rafhip_lans_workspace_bytes(const rafhip_lans_plan* plan);
 int32_t rafhip_lans_plan_num_tensors(const rafhip_lans_plan* plan);
 int64_t rafhip_lans_plan_num_chunks(const rafhip_lans_plan* plan);
 int64_t rafhip_lans_plan_total_elements(const rafhip_lans_plan* plan);
+/* A plan keeps RAFHIP_TABLE_SLOTS device tables of tensor pointers, each with the pointer lists it
+ * was last sent; a step whose lists equal one of them sends nothing, any other replaces the least
+ * recently used through pinned staging memory of its own, without waiting for the device.  An
+ * executor whose gradients alternate between two allocations (the reference's VM allocates them
+ * per iteration, src/impl/vm/vm.cc:1099-1105) therefore stops uploading after two steps.  This
+ * counts the uploads made so far (-1 on NULL). */
+#define RAFHIP_TABLE_SLOTS 4
+int64_t rafhip_lans_plan_table_uploads(const rafhip_lans_plan* plan);
 
 /*
  * One LANS step, in place on w/m/v; g is read-only (the reference overwrites it with an

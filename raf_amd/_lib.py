@@ -13,6 +13,7 @@ from pathlib import Path
 LIB_DIR = Path(__file__).resolve().parent / "lib"
 OPTIM_LIB = LIB_DIR / "libraf_hip_optim.so"
 DIALECT_LIB = LIB_DIR / "libraf_hip_dialect.so"
+GLUE_LIB = LIB_DIR / "_torch_glue.so"
 
 RAFHIP_OK = 0
 RAFHIP_ERR_INVALID_ARG = 1
@@ -81,6 +82,7 @@ OPTIM_SYMBOLS = {
     "rafhip_lans_plan_num_tensors": (c_int32, [c_void_p]),
     "rafhip_lans_plan_num_chunks": (c_int64, [c_void_p]),
     "rafhip_lans_plan_total_elements": (c_int64, [c_void_p]),
+    "rafhip_lans_plan_table_uploads": (c_int64, [c_void_p]),
     "rafhip_lans_step": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
                                  POINTER(c_void_p), c_void_p, c_int32, POINTER(LansHParams),
                                  c_void_p, c_int64, c_void_p]),
@@ -141,6 +143,13 @@ DIALECT_SYMBOLS = {
                                      c_int32, POINTER(c_void_p)]),
     "rafhip_raf_lans_execute": (c_int, [c_void_p, c_int32, POINTER(TensorDesc),
                                         POINTER(TensorDesc), c_void_p, c_int64, c_void_p]),
+    "rafhip_raf_tuple_make": (c_int, [c_int32, POINTER(TensorDesc), POINTER(c_void_p)]),
+    "rafhip_raf_tuple_replace": (c_int, [c_void_p, c_int32, c_int32, POINTER(TensorDesc), POINTER(c_void_p)]),
+    "rafhip_raf_tuple_size": (c_int32, [c_void_p]),
+    "rafhip_raf_tuple_destroy": (c_int, [c_void_p]),
+    "rafhip_raf_lans_execute_tuple": (c_int, [c_void_p, c_void_p, POINTER(TensorDesc), c_void_p, c_int64,
+                                              c_void_p, c_int32]),
+    "rafhip_raf_sgd_multi_execute_tuple": (c_int, [c_void_p, c_void_p, c_void_p, c_int32]),
     "rafhip_raf_sgd_multi_make": (c_int, [c_int32, c_int32, POINTER(TensorDesc), c_double, c_double,
                                           POINTER(c_void_p)]),
     "rafhip_raf_sgd_multi_execute": (c_int, [c_void_p, c_int32, POINTER(TensorDesc), c_void_p]),
@@ -217,6 +226,7 @@ DEVICE_SYMBOLS = {
 
 _optim = None
 _dialect = None
+_glue = None
 
 
 def _bind(lib, table):
@@ -262,6 +272,25 @@ def dialect():
         _bind(lib, DIALECT_SYMBOLS)
         _dialect = lib
     return _dialect
+
+
+def glue():
+    """The CPython module that reads lists of torch tensors for the operator front end."""
+    global _glue
+    if _glue is None:
+        if not GLUE_LIB.exists():
+            raise RuntimeError(f"{GLUE_LIB} is missing: build it with `python -m raf_amd.build`")
+        import importlib.machinery
+        import importlib.util
+
+        import torch  # noqa: F401  (the module resolves its symbols in torch's libraries)
+
+        loader = importlib.machinery.ExtensionFileLoader("_torch_glue", str(GLUE_LIB))
+        spec = importlib.util.spec_from_loader("_torch_glue", loader)
+        module = importlib.util.module_from_spec(spec)
+        loader.exec_module(module)
+        _glue = module
+    return _glue
 
 
 class RafError(RuntimeError):

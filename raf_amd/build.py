@@ -3,9 +3,10 @@
     python -m raf_amd.build            # build everything
     python -m raf_amd.build --check    # exit 1 if a library is missing or older than its sources
 
-Two shared objects land in raf_amd/lib/:
+Three shared objects land in raf_amd/lib/:
   libraf_hip_optim.so    HIP kernels + the C ABI declared in include/rafhip_optim.h
   libraf_hip_dialect.so  C++ host layer: OpEnv / dialect registry mirror + the `hip` dialect ops
+  _torch_glue.so         CPython module that reads lists of torch tensors for the Python front end
 """
 from __future__ import annotations
 
@@ -73,9 +74,33 @@ def build_dialect() -> Path:
     return out
 
 
+def glue_lib() -> Path:
+    return LIB / "_torch_glue.so"
+
+
+def build_glue() -> Path:
+    """The only piece that sees torch's headers: host C++ built with the host compiler against the
+    installed torch (its C++ ABI setting included) and this interpreter's headers."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension
+
+    LIB.mkdir(parents=True, exist_ok=True)
+    out = glue_lib()
+    torch_lib = Path(torch.__file__).resolve().parent / "lib"
+    incs = [f"-I{p}" for p in cpp_extension.include_paths()] + [f"-I{sysconfig.get_paths()['include']}"]
+    _run([os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall",
+          f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}", f"-I{INCLUDE}", *incs,
+          "-o", out, CSRC / "torch_glue.cpp", f"-L{torch_lib}", "-ltorch_python", "-ltorch_cpu", "-lc10",
+          f"-Wl,-rpath,{torch_lib}"])
+    return out
+
+
 def build_all() -> None:
     build_optim()
     build_dialect()
+    build_glue()
 
 
 def stale() -> list:
@@ -84,6 +109,7 @@ def stale() -> list:
     deps = {
         optim_lib(): [CSRC / s for s in OPTIM_SOURCES] + list(CSRC.glob("*.h")) + list(INCLUDE.glob("*.h")),
         dialect_lib(): [CSRC / s for s in DIALECT_SOURCES] + list((CSRC / "dialect").glob("*.h")) + list(INCLUDE.glob("*.h")),
+        glue_lib(): [CSRC / "torch_glue.cpp", INCLUDE / "rafhip_dialect.h"],
     }
     for lib, srcs in deps.items():
         if not lib.exists() or any(s.stat().st_mtime > lib.stat().st_mtime for s in srcs if s.exists()):

@@ -17,6 +17,10 @@ struct rafhip_raf_memory {
   std::shared_ptr<memory_pool::Memory> mem;
 };
 
+struct rafhip_raf_tuple {
+  value::TupleValue value;
+};
+
 struct rafhip_raf_env {
   OpEnvPtr env;
   CallValues call;
@@ -479,6 +483,79 @@ int rafhip_raf_lans_execute(rafhip_raf_env* env, int32_t list_len,
     std::vector<value::Value> inputs = {tuple, FromDesc(step, "step")};
     OpEnv::SetStreamForAllBackends(env->call->device, stream);
     WorkspaceBinding bind(env->env.get(), workspace, workspace_bytes);
+    env->env->Execute(inputs, tuple);  // output aliases the inputs
+  });
+}
+
+int rafhip_raf_tuple_make(int32_t n, const rafhip_tensor_desc* fields, rafhip_raf_tuple** tuple_out) {
+  return Guard([&] {
+    if (!tuple_out) throw Error("rafhip_raf_tuple_make: tuple_out is NULL");
+    *tuple_out = nullptr;
+    if (n < 0 || (n > 0 && !fields)) throw Error("rafhip_raf_tuple_make: bad field list");
+    std::vector<value::Value> values;
+    values.reserve((size_t)n);
+    for (int32_t i = 0; i < n; ++i) values.push_back(FromDesc(&fields[i], "tuple field"));
+    *tuple_out = new rafhip_raf_tuple{value::MakeTuple(std::move(values))};
+  });
+}
+
+int rafhip_raf_tuple_replace(const rafhip_raf_tuple* base, int32_t first, int32_t count,
+                             const rafhip_tensor_desc* fields, rafhip_raf_tuple** tuple_out) {
+  return Guard([&] {
+    if (!tuple_out) throw Error("rafhip_raf_tuple_replace: tuple_out is NULL");
+    *tuple_out = nullptr;
+    if (!base) throw Error("rafhip_raf_tuple_replace: base is NULL");
+    const int64_t n = (int64_t)base->value->fields.size();
+    if (first < 0 || count < 0 || (int64_t)first + count > n || (count > 0 && !fields))
+      throw Error("rafhip_raf_tuple_replace: range [" + std::to_string(first) + ", " +
+                  std::to_string((int64_t)first + count) + ") does not fit a tuple of " + std::to_string(n));
+    std::vector<value::Value> values = base->value->fields;  // shares the tensor values
+    for (int32_t i = 0; i < count; ++i) values[(size_t)first + (size_t)i] = FromDesc(&fields[i], "tuple field");
+    *tuple_out = new rafhip_raf_tuple{value::MakeTuple(std::move(values))};
+  });
+}
+
+int32_t rafhip_raf_tuple_size(const rafhip_raf_tuple* tuple) {
+  return tuple ? (int32_t)tuple->value->fields.size() : -1;
+}
+
+int rafhip_raf_tuple_destroy(rafhip_raf_tuple* tuple) {
+  return Guard([&] { delete tuple; });
+}
+
+namespace {
+// The value Execute receives for a tuple handle: the tuple itself, or (as_vm) a new TupleValue
+// over the same tensor values, as the VM's AllocTuple makes one per iteration (vm.cc:764-769).
+value::Value TupleArgument(const rafhip_raf_tuple* tuple, int32_t as_vm, const char* who) {
+  if (!tuple) throw Error(std::string(who) + ": tensor_list is NULL");
+  if (!as_vm) return tuple->value;
+  return value::MakeTuple(tuple->value->fields);
+}
+}  // namespace
+
+int rafhip_raf_lans_execute_tuple(rafhip_raf_env* env, const rafhip_raf_tuple* tensor_list,
+                                  const rafhip_tensor_desc* step, void* workspace,
+                                  int64_t workspace_bytes, void* stream, int32_t as_vm) {
+  return Guard([&] {
+    if (!env) throw Error("rafhip_raf_lans_execute_tuple: env is NULL");
+    if (!env->env) return;  // declared as a no-op
+    value::Value tuple = TupleArgument(tensor_list, as_vm, "rafhip_raf_lans_execute_tuple");
+    std::vector<value::Value> inputs = {tuple, FromDesc(step, "step")};
+    OpEnv::SetStreamForAllBackends(env->call->device, stream);
+    WorkspaceBinding bind(env->env.get(), workspace, workspace_bytes);
+    env->env->Execute(inputs, tuple);  // output aliases the inputs
+  });
+}
+
+int rafhip_raf_sgd_multi_execute_tuple(rafhip_raf_env* env, const rafhip_raf_tuple* tensor_list,
+                                       void* stream, int32_t as_vm) {
+  return Guard([&] {
+    if (!env) throw Error("rafhip_raf_sgd_multi_execute_tuple: env is NULL");
+    if (!env->env) return;  // declared as a no-op
+    value::Value tuple = TupleArgument(tensor_list, as_vm, "rafhip_raf_sgd_multi_execute_tuple");
+    std::vector<value::Value> inputs = {tuple};
+    OpEnv::SetStreamForAllBackends(env->call->device, stream);
+    WorkspaceBinding bind(env->env.get(), nullptr, 0);
     env->env->Execute(inputs, tuple);  // output aliases the inputs
   });
 }

@@ -16,7 +16,9 @@
 // arguments are reported through error_msgs so dispatch can fall through to another dialect.
 #include "hip_dialect.h"
 
+#include <cstring>
 #include <sstream>
+#include <typeinfo>
 
 #include "raf_iface.h"
 #include "rafhip_optim.h"
@@ -43,6 +45,22 @@ bool IsF16(const DType& t) { return t.code == kDLFloat && t.bits == 16; }
 bool IsBF16(const DType& t) { return t.code == kDLBfloat && t.bits == 16; }
 int32_t KernelDType(const DType& t) {
   return IsF32(t) ? RAFHIP_F32 : IsF16(t) ? RAFHIP_F16 : IsBF16(t) ? RAFHIP_BF16 : -1;
+}
+
+// The data pointers of a tuple's tensor fields into out[fields.size()].  This runs for every field
+// at every Execute, so it costs one type comparison and one pointer read per field: no reference
+// counting, and the exact-type test first (inside RAF the downcast is a type-index comparison,
+// `field.as<TensorValueObj>()`); only a subclass would take the dynamic_cast.
+void CollectDataPointers(const std::vector<Value>& fields, void** out, const std::string& op) {
+  for (size_t i = 0; i < fields.size(); ++i) {
+    const value::ValueObj* f = fields[i].get();
+    const value::TensorValueObj* t = nullptr;
+    if (f != nullptr)
+      t = typeid(*f) == typeid(value::TensorValueObj) ? static_cast<const value::TensorValueObj*>(f)
+                                                      : dynamic_cast<const value::TensorValueObj*>(f);
+    if (!t) throw Error(op + ": field " + std::to_string(i) + " of tensor_list is not a tensor");
+    out[i] = t->tensor.data;
+  }
 }
 
 }  // namespace
@@ -182,9 +200,9 @@ class SgdMultiHipEnv : public OpEnv, public HasLearningRate {
     auto tuple = AsTuple(inputs[0]);
     RAF_CHECK((int64_t)tuple->fields.size() == (int64_t)blocks_ * (int64_t)n_,
               op_ + ": tensor_list length changed since the OpEnv was made");
-    std::vector<void*> ptrs(tuple->fields.size());
-    for (size_t i = 0; i < ptrs.size(); ++i) ptrs[i] = AsTensor(tuple->fields[i])->tensor.data;
-    void** p = ptrs.data();
+    ptrs_.resize(tuple->fields.size());
+    CollectDataPointers(tuple->fields, ptrs_.data(), op_);
+    void** p = ptrs_.data();
     void* stream = DeviceAPI::Get(DevType::kROCM())->GetStream();
     int st = rafhip_sgd_multi_step(plan_, reinterpret_cast<float* const*>(p),
                                    reinterpret_cast<const void* const*>(p + n_),
@@ -209,6 +227,7 @@ class SgdMultiHipEnv : public OpEnv, public HasLearningRate {
   int32_t n_ = 0;
   int32_t copy_dtype_ = RAFHIP_F16;
   rafhip_sgd_plan* plan_ = nullptr;
+  std::vector<void*> ptrs_;  // this call's addresses (kept: no allocation per call)
 };
 
 // ---------------------------------------------------------------------------------------- LANS
@@ -319,13 +338,16 @@ class LansHipEnv : public OpEnv, public HasLearningRate, public HasGradScaling {
     RAF_CHECK(IsF32(step.dtype), "step must be float32");
     RAF_CHECK(workspace_ != nullptr || workspace_bytes_ == 0,
               "raf.op.hip.lans: the executor did not provide the requested workspace");
-    // An executor that hands over the very same tuple object again (a loop over fixed storage)
-    // finds the plan already bound to its tensors: no walk over the 4n or 5n fields, no table
-    // to compare or send.  Any other tuple is walked and bound afresh.  Only a weak reference is
-    // kept, so the OpEnv never prolongs the life of a caller's tensors.
-    if (bound_tuple_.expired() || bound_tuple_.lock() != tuple) {
-      ptrs_.resize(tuple->fields.size());
-      for (size_t i = 0; i < ptrs_.size(); ++i) ptrs_[i] = AsTensor(tuple->fields[i])->tensor.data;
+    // Executors hand over a new TupleValue at every call (the VM allocates one per iteration,
+    // src/impl/vm/vm.cc:764-769; the interpreter overload above makes one too) and a tuple's
+    // fields and a tensor's storage may be replaced between calls, so nothing is concluded from
+    // the identity of the tuple: its fields are walked, one pointer read each, and the plan is
+    // bound afresh only when an address differs from the last call's.
+    now_.resize(tuple->fields.size());
+    CollectDataPointers(tuple->fields, now_.data(), op_);
+    if (!bound_ || std::memcmp(now_.data(), ptrs_.data(), sizeof(void*) * now_.size()) != 0) {
+      bound_ = false;
+      ptrs_.swap(now_);
       void** p = ptrs_.data();
       int st = rafhip_lans_plan_bind(plan_, reinterpret_cast<const void* const*>(p),
                                      reinterpret_cast<float* const*>(p + n_),
@@ -333,7 +355,7 @@ class LansHipEnv : public OpEnv, public HasLearningRate, public HasGradScaling {
                                      reinterpret_cast<float* const*>(p + 3 * n_),
                                      blocks_ == 5 ? p + 4 * n_ : nullptr, copy_dtype_);
       if (st != RAFHIP_OK) throw Error(KernelError("rafhip_lans_plan_bind", st));
-      bound_tuple_ = tuple;
+      bound_ = true;
     }
     void* stream = DeviceAPI::Get(DevType::kROCM())->GetStream();
     int st = rafhip_lans_step_bound(plan_, static_cast<const float*>(step.data), 0, &hp_, workspace_,
@@ -363,8 +385,9 @@ class LansHipEnv : public OpEnv, public HasLearningRate, public HasGradScaling {
   rafhip_lans_plan* plan_ = nullptr;
   void* workspace_ = nullptr;  // bound by the executor around each Execute
   int64_t workspace_bytes_ = 0;
-  std::weak_ptr<value::TupleValueObj> bound_tuple_;  // the tuple whose tensors the plan is bound to
-  std::vector<void*> ptrs_;
+  std::vector<void*> ptrs_;  // the addresses the plan is bound to (g, w, m, v[, p] blocks)
+  std::vector<void*> now_;   // this call's addresses
+  bool bound_ = false;
 };
 
 // -------------------------------------------------------------------------------------- l2norm

@@ -36,8 +36,8 @@ constexpr int kCopyBlock = 256;
 // then the stores, then the workgroup ends.  Measured on the BERT-large list (1.34 GB): 6.3 TB/s,
 // against 6.1-6.2 for items of 16-32 KiB and 5.5 for 4 KiB items or for a grid-stride loop over
 // CUs x 8 workgroups.
-constexpr int64_t kCopyChunkDefault = 8 * 1024;  // bytes per work item
-constexpr int kCopyInFlightDefault = 2;          // 16-byte accesses in flight per lane per trip
+constexpr int64_t kCopyChunk = 8 * 1024;  // bytes per work item
+constexpr int kCopyInFlight = 2;          // 16-byte accesses in flight per lane per trip
 
 struct Segment {  // 32 bytes, one per tensor
   char* part;     // the tensor
@@ -51,7 +51,7 @@ struct CopyItem {
   int32_t chunk;
 };
 
-template <bool kNT, int kCopyInFlight>
+template <bool kNT>
 __device__ __forceinline__ void copy_bytes(char* dst, const char* src, int64_t n) {
   // head: bring dst to a 16-byte boundary
   int64_t head = (int64_t)((16u - (unsigned)(reinterpret_cast<uintptr_t>(dst) & 15u)) & 15u);
@@ -94,10 +94,10 @@ __device__ __forceinline__ void copy_bytes(char* dst, const char* src, int64_t n
 }
 
 // gather != 0: parts -> flat buffer (fuse); gather == 0: flat buffer -> parts (defuse).
-template <bool kNT, int kCopyInFlight>
+template <bool kNT>
 __global__ __launch_bounds__(kCopyBlock) void fuse_copy(const Segment* segments,
                                                         const CopyItem* items, int64_t n_items,
-                                                        char* flat, int gather, int64_t kCopyChunk) {
+                                                        char* flat, int gather) {
   for (int64_t it = blockIdx.x; it < n_items; it += gridDim.x) {
     const CopyItem item = items[it];
     const Segment seg = segments[item.segment];
@@ -107,9 +107,9 @@ __global__ __launch_bounds__(kCopyBlock) void fuse_copy(const Segment* segments,
     char* in_part = seg.part + begin;
     char* in_flat = flat + seg.offset + begin;
     if (gather)
-      copy_bytes<kNT, kCopyInFlight>(in_flat, in_part, len);
+      copy_bytes<kNT>(in_flat, in_part, len);
     else
-      copy_bytes<kNT, kCopyInFlight>(in_part, in_flat, len);
+      copy_bytes<kNT>(in_part, in_flat, len);
   }
 }
 
@@ -126,20 +126,17 @@ struct rafhip_fuse_plan {
   std::vector<int64_t> nbytes, offset;
   int64_t total_bytes = 0;
   int64_t n_items = 0;
-  int64_t chunk_bytes = kCopyChunkDefault;
-  int in_flight = kCopyInFlightDefault;
-  int blocks_per_cu = 0;  // grid cap per CU; 0 = one workgroup per item
   void* d_tables = nullptr;
-  Segment* d_segments = nullptr;
   CopyItem* d_items = nullptr;
-  RecordUploader<Segment> segments;
+  RecordTables<Segment> tables;  // device segment tables that follow the caller's pointers
+  std::vector<Segment> segs;     // this call's segments, built in place: a call allocates nothing
 };
 
 namespace {
 
 void free_plan(rafhip_fuse_plan* p) {
   if (!p) return;
-  p->segments.release();
+  p->tables.release();
   if (p->d_tables) (void)hipFree(p->d_tables);
   delete p;
 }
@@ -152,30 +149,25 @@ int run(rafhip_fuse_plan* plan, const char* what, void* const* parts, void* flat
   if (int st = check_plan_device(what, plan->device)) return st;
   if (!parts || !flat) return fail(RAFHIP_ERR_INVALID_ARG, "%s: null pointer argument", what);
   return guarded(what, [&]() -> int {
-    std::vector<Segment> segs((size_t)plan->n);
+    std::vector<Segment>& segs = plan->segs;  // already n long
     for (int32_t i = 0; i < plan->n; ++i) {
       if (plan->nbytes[i] > 0 && !parts[i])
         return fail(RAFHIP_ERR_INVALID_ARG, "%s: tensor %d has a null data pointer", what, i);
       segs[i] = Segment{static_cast<char*>(parts[i]), plan->offset[i], plan->nbytes[i], 0};
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    RAFHIP_HIP_TRY(plan->segments.sync(segs, s));
-    const int64_t cap = plan->blocks_per_cu > 0 ? (int64_t)streaming_grid_cap() / 8 * plan->blocks_per_cu
-                                                : (int64_t)1 << 30;
-    const unsigned grid = (unsigned)(plan->n_items < cap ? plan->n_items : cap);
+    const Segment* table = nullptr;
+    RAFHIP_HIP_TRY(plan->tables.sync(segs, s, &table));
+    // One workgroup per item; the kernel strides over what a launch cannot hold.
+    const unsigned grid = (unsigned)(plan->n_items < kMaxGridBlocks ? plan->n_items : kMaxGridBlocks);
     auto go = [&](auto kernel) {
-      hipLaunchKernelGGL(kernel, dim3(grid), dim3(kCopyBlock), 0, s, plan->d_segments, plan->d_items,
-                         plan->n_items, static_cast<char*>(flat), gather ? 1 : 0, plan->chunk_bytes);
+      hipLaunchKernelGGL(kernel, dim3(grid), dim3(kCopyBlock), 0, s, table, plan->d_items,
+                         plan->n_items, static_cast<char*>(flat), gather ? 1 : 0);
     };
-    const bool nt = plan->total_bytes > kStreamFromBytes;
-    if (plan->in_flight == 8)
-      nt ? go(fuse_copy<true, 8>) : go(fuse_copy<false, 8>);
-    else if (plan->in_flight == 2)
-      nt ? go(fuse_copy<true, 2>) : go(fuse_copy<false, 2>);
-    else if (plan->in_flight == 1)
-      nt ? go(fuse_copy<true, 1>) : go(fuse_copy<false, 1>);
+    if (plan->total_bytes > kStreamFromBytes)
+      go(fuse_copy<true>);
     else
-      nt ? go(fuse_copy<true, 4>) : go(fuse_copy<false, 4>);
+      go(fuse_copy<false>);
     RAFHIP_HIP_TRY(hipGetLastError());
     return RAFHIP_OK;
   });
@@ -194,11 +186,6 @@ int rafhip_fuse_plan_create(int32_t n_tensors, const int64_t* nbytes, rafhip_fus
   return guarded("rafhip_fuse_plan_create", [&]() -> int {
     std::unique_ptr<rafhip_fuse_plan, void (*)(rafhip_fuse_plan*)> p(new rafhip_fuse_plan(), free_plan);
     p->n = n_tensors;
-    const int kib = env_knob("RAFHIP_FUSE_CHUNK_KIB", (int)(kCopyChunkDefault >> 10));
-    if (kib >= 4 && kib <= 4096 && (kib & (kib - 1)) == 0) p->chunk_bytes = (int64_t)kib << 10;
-    p->in_flight = env_knob("RAFHIP_FUSE_IN_FLIGHT", kCopyInFlightDefault);
-    p->blocks_per_cu = env_knob("RAFHIP_FUSE_BLOCKS_PER_CU", 0);
-    const int64_t kCopyChunk = p->chunk_bytes;
     std::vector<CopyItem> items;
     for (int32_t i = 0; i < n_tensors; ++i) {
       if (nbytes[i] < 0)
@@ -221,12 +208,11 @@ int rafhip_fuse_plan_create(int32_t n_tensors, const int64_t* nbytes, rafhip_fus
       (void)hipGetLastError();
       return fail(RAFHIP_ERR_NO_DEVICE, "rafhip_fuse_plan_create: no HIP device available");
     }
-    const size_t seg_bytes = (sizeof(Segment) * (size_t)n_tensors + 255) / 256 * 256;
-    hipError_t e = hipMalloc(&p->d_tables, seg_bytes + sizeof(CopyItem) * items.size());
+    p->segs.resize((size_t)n_tensors);
+    hipError_t e = hipMalloc(&p->d_tables, sizeof(CopyItem) * items.size());
     if (e == hipSuccess) {
-      p->d_segments = static_cast<Segment*>(p->d_tables);
-      p->d_items = reinterpret_cast<CopyItem*>(static_cast<char*>(p->d_tables) + seg_bytes);
-      e = p->segments.init(p->d_segments, (size_t)n_tensors);
+      p->d_items = static_cast<CopyItem*>(p->d_tables);
+      e = p->tables.init((size_t)n_tensors);
     }
     if (e == hipSuccess) {
       e = hipMemcpy(p->d_items, items.data(), sizeof(CopyItem) * items.size(), hipMemcpyHostToDevice);

@@ -980,7 +980,7 @@ void launch_phased_t(hipStream_t s, const LansDeviceArgs& a, const float* step_d
   // not of bandwidth, and finer items cost it 30 % of the pass.
   const int slice_shift = kMode == kModeStreaming ? apply_slice_shift : 0;
   const int64_t slices = (int64_t)a.n_chunks << (slice_shift > 0 ? kChunkShift - slice_shift : 0);
-  const unsigned grid_c = (unsigned)(slices < (1 << 24) ? slices : (1 << 24));
+  const unsigned grid_c = (unsigned)(slices < (1 << 24) ? slices : (1 << 24) - 1);  // 2^32 threads are refused
   hipLaunchKernelGGL((lans_apply<G, kMode>), dim3(grid_c), dim3(kLansBlock), 0, s, a, slice_shift);
   mark(5);
 }

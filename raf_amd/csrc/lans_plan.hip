@@ -20,6 +20,8 @@
 
 using namespace rafhip;
 
+static_assert(RecordTables<TensorRec>::kSlots == RAFHIP_TABLE_SLOTS, "header and table cache disagree");
+
 // Scratch memory of rafhip_lans_step_noalloc, the step for callers that cannot allocate: the
 // step scalars, per-tensor statistics, chunk partial sums and ticket words that the other step
 // entry points find in the caller's workspace.  Every GPU the library runs on holds its own copy
@@ -334,9 +336,8 @@ struct rafhip_lans_plan {
   std::vector<int32_t> first_chunk;
   WorkspaceLayout ws{};
 
-  // Device tables in one allocation: [TensorRec x n][chunk items][pipeline items][pass-A items].
+  // Work lists in one allocation: [chunk items][pipeline items][pass-A items].
   void* d_tables = nullptr;
-  TensorRec* d_tensors = nullptr;
   WorkItem* d_items = nullptr;
   WorkItem* d_items_a = nullptr;
   int64_t n_items_a = 0;
@@ -347,12 +348,12 @@ struct rafhip_lans_plan {
   uint32_t* host_error = nullptr;
   uint32_t* host_error_dev = nullptr;  // the device's address of the same word
 
-  RecordUploader<TensorRec> tensors;  // a step whose pointers did not move sends nothing
+  RecordTables<TensorRec> tensors;  // device tensor tables; a step whose pointers are known sends nothing
   std::vector<TensorRec> recs;        // this call's records, built in place: a step allocates nothing
   // rafhip_lans_plan_bind: records of tensors that stay where they are, built and checked once.
   std::vector<TensorRec> bound;
   bool bound_valid = false;
-  bool bound_on_device = false;  // the device table holds `bound` (no other step intervened)
+  bool bound_on_device = false;  // the table used last holds `bound` (no other step intervened)
   int32_t bound_p_dtype = RAFHIP_F16;
   // rafhip_lans_plan_set_dynamic_scale: optional device words read by every kernel of a step.
   const float* unscale_dev = nullptr;
@@ -547,22 +548,18 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
       p->n_pipeline_items = (uint32_t)pipeline.size();
       if (p->pipeline_grid > p->n_pipeline_items) p->pipeline_grid = p->n_pipeline_items;
 
-      const size_t tensors_bytes = (size_t)align_up((int64_t)sizeof(TensorRec) * n_tensors);
       const size_t phased_bytes = (size_t)align_up((int64_t)sizeof(WorkItem) * (int64_t)phased.size());
       const size_t pipe_bytes = (size_t)align_up((int64_t)sizeof(WorkItem) * (int64_t)pipeline.size());
       const size_t a_bytes = (size_t)align_up((int64_t)sizeof(WorkItem) * (int64_t)phased_a.size());
-      hipError_t e =
-          hipMalloc(&p->d_tables, tensors_bytes + phased_bytes + pipe_bytes + a_bytes + kAlign);
-      if (e == hipSuccess)
-        e = p->tensors.init(static_cast<TensorRec*>(p->d_tables), (size_t)n_tensors);
+      hipError_t e = hipMalloc(&p->d_tables, phased_bytes + pipe_bytes + a_bytes + kAlign);
+      if (e == hipSuccess) e = p->tensors.init((size_t)n_tensors);
       if (e != hipSuccess)
         return fail(RAFHIP_ERR_HIP, "rafhip_lans_plan_create: allocation failed: %s",
                     hipGetErrorString(e));
       char* base = static_cast<char*>(p->d_tables);
-      p->d_tensors = reinterpret_cast<TensorRec*>(base);
-      p->d_items = reinterpret_cast<WorkItem*>(base + tensors_bytes);
-      p->d_pipeline = reinterpret_cast<WorkItem*>(base + tensors_bytes + phased_bytes);
-      p->d_items_a = reinterpret_cast<WorkItem*>(base + tensors_bytes + phased_bytes + pipe_bytes);
+      p->d_items = reinterpret_cast<WorkItem*>(base);
+      p->d_pipeline = reinterpret_cast<WorkItem*>(base + phased_bytes);
+      p->d_items_a = reinterpret_cast<WorkItem*>(base + phased_bytes + pipe_bytes);
       if (!phased_a.empty())
         e = hipMemcpy(p->d_items_a, phased_a.data(), sizeof(WorkItem) * phased_a.size(),
                       hipMemcpyHostToDevice);
@@ -617,6 +614,10 @@ int64_t rafhip_lans_plan_num_chunks(const rafhip_lans_plan* plan) {
 }
 int64_t rafhip_lans_plan_total_elements(const rafhip_lans_plan* plan) {
   return plan ? plan->total_elements : -1;
+}
+
+int64_t rafhip_lans_plan_table_uploads(const rafhip_lans_plan* plan) {
+  return plan ? plan->tensors.uploads() : -1;
 }
 
 int rafhip_lans_step(rafhip_lans_plan* plan, const void* const* g, float* const* w,
@@ -723,14 +724,15 @@ int build_records(const char* who, const rafhip_lans_plan* plan, const void* con
   return RAFHIP_OK;
 }
 
-// Enqueues the kernels of one step on `s`; the device tensor table is up to date for that stream.
-int launch_step(const char* who, rafhip_lans_plan* plan, int32_t p_dtype, const float* step_dev,
-                int32_t step_host, const rafhip_lans_hparams* hp, void* workspace,
-                int64_t workspace_bytes, hipStream_t s) {
+// Enqueues the kernels of one step on `s`; `table` is the device tensor table to read, up to date
+// for that stream.
+int launch_step(const char* who, rafhip_lans_plan* plan, const TensorRec* table, int32_t p_dtype,
+                const float* step_dev, int32_t step_host, const rafhip_lans_hparams* hp,
+                void* workspace, int64_t workspace_bytes, hipStream_t s) {
   (void)who;
   char* ws = static_cast<char*>(workspace);
   LansDeviceArgs a;
-  a.tensors = plan->d_tensors;
+  a.tensors = table;
   a.n_tensors = plan->n_tensors;
   a.items = plan->d_items;
   a.n_chunks = plan->n_chunks;
@@ -813,9 +815,10 @@ int lans_step_impl(rafhip_lans_plan* plan, const void* const* g, float* const* w
     if (int st = check_workspace(who, plan, workspace, workspace_bytes)) return st;
     if (int st = build_records(who, plan, g, w, m, v, p, p_dtype, plan->recs)) return st;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    RAFHIP_HIP_TRY(plan->tensors.sync(plan->recs, s));
-    plan->bound_on_device = false;  // whatever was bound, the device table now follows this call
-    return launch_step(who, plan, p_dtype, step_dev, step_host, hp, workspace, workspace_bytes, s);
+    const TensorRec* table = nullptr;
+    RAFHIP_HIP_TRY(plan->tensors.sync(plan->recs, s, &table));
+    plan->bound_on_device = false;  // whatever was bound, the table used last now follows this call
+    return launch_step(who, plan, table, p_dtype, step_dev, step_host, hp, workspace, workspace_bytes, s);
   });
 }
 
@@ -852,14 +855,15 @@ int rafhip_lans_step_bound(rafhip_lans_plan* plan, const float* step_dev, int32_
   return guarded(who, [&]() -> int {
     if (int st = check_workspace(who, plan, workspace, workspace_bytes)) return st;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    const TensorRec* table = nullptr;
     if (plan->bound_on_device) {
-      RAFHIP_HIP_TRY(plan->tensors.follow(s));  // nothing to build, compare or send
+      RAFHIP_HIP_TRY(plan->tensors.follow(s, &table));  // nothing to build, compare or send
     } else {
       plan->recs = plan->bound;  // same size: a copy, no allocation
-      RAFHIP_HIP_TRY(plan->tensors.sync(plan->recs, s));
+      RAFHIP_HIP_TRY(plan->tensors.sync(plan->recs, s, &table));
       plan->bound_on_device = true;
     }
-    return launch_step(who, plan, plan->bound_p_dtype, step_dev, step_host, hp, workspace,
+    return launch_step(who, plan, table, plan->bound_p_dtype, step_dev, step_host, hp, workspace,
                        workspace_bytes, s);
   });
 }

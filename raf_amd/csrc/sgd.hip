@@ -35,15 +35,7 @@ namespace rafhip {
 namespace {
 
 constexpr int kSgdBlock = 256;
-constexpr int kSgdUnroll = 2;  // float4 groups in flight per lane per trip (multi-tensor default)
-
-int env_int(const char* name, int fallback) {
-  if (const char* e = std::getenv(name)) {
-    const int v = std::atoi(e);
-    if (v > 0) return v;
-  }
-  return fallback;
-}
+constexpr int kSgdUnroll = 2;  // float4 groups in flight per lane per trip (cache-resident lists)
 
 __device__ __forceinline__ void sgd_elem(float x0, float dx, float v0, float lr, float mu,
                                          float& v1, float& x1) {
@@ -107,7 +99,7 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 // 1024 elements per work item: a workgroup makes one trip (one 16-byte access per lane and array)
 // and ends, so no wavefront ever holds loads back behind its own stores.  Measured on the
 // BERT-large list: 6.29 TB/s, against 5.80-5.86 with 2048 and 5.67-5.85 with 4096 elements per item.
-constexpr int kSgdChunkShiftDefault = 10;
+constexpr int kSgdChunkShift = 10;
 
 struct SgdRec {  // 48 bytes, one per parameter
   float* x;      // fp32 (master) weight, updated in place
@@ -189,23 +181,16 @@ __global__ __launch_bounds__(kSgdBlock) void sgd_multi_kernel(const SgdRec* recs
 constexpr int64_t kSgdStreamFromBytes = 160LL << 20;
 
 template <typename G>
-void launch_sgd_multi(bool stream_nt, int unroll, unsigned grid, hipStream_t s, const SgdRec* recs,
-                      const SgdItem* items, int64_t n_items, float lr, float mu, int p_is_bf16,
-                      int chunk_shift) {
+void launch_sgd_multi(bool stream_nt, unsigned grid, hipStream_t s, const SgdRec* recs,
+                      const SgdItem* items, int64_t n_items, float lr, float mu, int p_is_bf16) {
   auto go = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(kSgdBlock), 0, s, recs, items, n_items, lr, mu,
-                       p_is_bf16, chunk_shift);
+                       p_is_bf16, kSgdChunkShift);
   };
-  if (stream_nt) {
-    if (unroll >= 4)
-      go(sgd_multi_kernel<G, true, 4>);
-    else if (unroll == 1)
-      go(sgd_multi_kernel<G, true, 1>);
-    else
-      go(sgd_multi_kernel<G, true, 2>);
-  } else {
+  if (stream_nt)
+    go(sgd_multi_kernel<G, true, 1>);  // 1024-element items: one access per lane and array
+  else
     go(sgd_multi_kernel<G, false, kSgdUnroll>);
-  }
 }
 
 }  // namespace
@@ -231,18 +216,18 @@ extern "C" int rafhip_sgd_f32(const float* x, const float* dx, const float* v, f
   int64_t done = 0;
   if (vec && n >= 4) {
     const int64_t n4 = n / 4;
-    static const int unroll_short = env_int("RAFHIP_SGD_UNROLL", 8);
-    static const int per_cu = env_int("RAFHIP_SGD_BLOCKS_PER_CU", 8);
+    constexpr int unroll_short = 8;
+    constexpr int per_cu = 8;
     // A long tensor is better served by workgroups that make one trip and end (see the
     // multi-tensor kernel): 6.2 against 6.0 TB/s at 16 Mi elements, 6.15 against 5.5 at 256 Mi,
     // equal at 8 Mi.  A short one is launch-bound and wants few, deep workgroups (4 Mi elements:
     // 5.8 against 5.3 TB/s).
-    static const int64_t one_trip_from = (int64_t)env_knob("RAFHIP_SGD_ONE_TRIP_FROM_MI", 8) << 20;
+    constexpr int64_t one_trip_from = (int64_t)8 << 20;
     const bool one_trip = n >= one_trip_from;
     const int unroll = one_trip ? 1 : unroll_short;
     const int64_t per_block = (int64_t)kSgdBlock * unroll;
     int64_t blocks = (n4 + per_block - 1) / per_block;
-    const int64_t gcap = one_trip ? (int64_t)1 << 30 : (int64_t)cap / 8 * per_cu;
+    const int64_t gcap = one_trip ? kMaxGridBlocks : (int64_t)cap / 8 * per_cu;
     if (blocks > gcap) blocks = gcap;
     auto go = [&](auto kernel) {
       hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kSgdBlock), 0, s,
@@ -250,14 +235,10 @@ extern "C" int rafhip_sgd_f32(const float* x, const float* dx, const float* v, f
                          reinterpret_cast<const f32x4*>(v), reinterpret_cast<f32x4*>(v_out),
                          reinterpret_cast<f32x4*>(x_out), n4, lr32, mu32);
     };
-    if (unroll == 1)
+    if (one_trip)
       go(sgd_vec4_kernel<1>);
-    else if (unroll == 4)
-      go(sgd_vec4_kernel<4>);
-    else if (unroll == 8)
-      go(sgd_vec4_kernel<8>);
     else
-      go(sgd_vec4_kernel<2>);
+      go(sgd_vec4_kernel<unroll_short>);
     RAFHIP_HIP_TRY(hipGetLastError());
     done = n4 * 4;
   }
@@ -280,19 +261,16 @@ struct rafhip_sgd_plan {
   std::vector<int64_t> numel;
   int64_t total_elements = 0;
   int64_t n_items = 0;
-  int chunk_shift = 12;
-  int unroll = 2;
-  int blocks_per_cu = 8;  // grid cap per CU; 0 = one workgroup per item
   void* d_tables = nullptr;
-  rafhip::SgdRec* d_recs = nullptr;
   rafhip::SgdItem* d_items = nullptr;
-  rafhip::RecordUploader<rafhip::SgdRec> recs;
+  rafhip::RecordTables<rafhip::SgdRec> tables;  // device record tables that follow the caller's pointers
+  std::vector<rafhip::SgdRec> recs;             // this call's records, built in place: a step allocates nothing
 };
 
 namespace {
 void free_sgd_plan(rafhip_sgd_plan* p) {
   if (!p) return;
-  p->recs.release();
+  p->tables.release();
   if (p->d_tables) (void)hipFree(p->d_tables);
   delete p;
 }
@@ -316,11 +294,7 @@ extern "C" int rafhip_sgd_plan_create(int32_t n_tensors, const int64_t* numel, i
     std::unique_ptr<rafhip_sgd_plan, void (*)(rafhip_sgd_plan*)> p(new rafhip_sgd_plan(), free_sgd_plan);
     p->n = n_tensors;
     p->grad_dtype = grad_dtype;
-    p->chunk_shift = env_int("RAFHIP_SGD_CHUNK_SHIFT", kSgdChunkShiftDefault);
-    if (p->chunk_shift < 10 || p->chunk_shift > 20) p->chunk_shift = kSgdChunkShiftDefault;
-    p->unroll = env_int("RAFHIP_SGD_MULTI_UNROLL", 1);
-    p->blocks_per_cu = std::getenv("RAFHIP_SGD_MULTI_BLOCKS_PER_CU") ? std::atoi(std::getenv("RAFHIP_SGD_MULTI_BLOCKS_PER_CU")) : 0;
-    const int64_t kSgdChunk = (int64_t)1 << p->chunk_shift;
+    const int64_t kSgdChunk = (int64_t)1 << kSgdChunkShift;
     std::vector<SgdItem> items;
     for (int32_t t = 0; t < n_tensors; ++t) {
       if (numel[t] < 0)
@@ -342,12 +316,11 @@ extern "C" int rafhip_sgd_plan_create(int32_t n_tensors, const int64_t* numel, i
       (void)hipGetLastError();
       return fail(RAFHIP_ERR_NO_DEVICE, "rafhip_sgd_plan_create: no HIP device available");
     }
-    const size_t rec_bytes = (sizeof(SgdRec) * (size_t)n_tensors + 255) / 256 * 256;
-    hipError_t e = hipMalloc(&p->d_tables, rec_bytes + sizeof(SgdItem) * items.size());
+    p->recs.resize((size_t)n_tensors);
+    hipError_t e = hipMalloc(&p->d_tables, sizeof(SgdItem) * items.size());
     if (e == hipSuccess) {
-      p->d_recs = static_cast<SgdRec*>(p->d_tables);
-      p->d_items = reinterpret_cast<SgdItem*>(static_cast<char*>(p->d_tables) + rec_bytes);
-      e = p->recs.init(p->d_recs, (size_t)n_tensors);
+      p->d_items = static_cast<SgdItem*>(p->d_tables);
+      e = p->tables.init((size_t)n_tensors);
     }
     if (e == hipSuccess)
       e = hipMemcpy(p->d_items, items.data(), sizeof(SgdItem) * items.size(), hipMemcpyHostToDevice);
@@ -377,7 +350,7 @@ extern "C" int rafhip_sgd_multi_step(rafhip_sgd_plan* plan, float* const* x, con
   if (!x || !dx || !v) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_sgd_multi_step: null pointer list");
   return guarded("rafhip_sgd_multi_step", [&]() -> int {
     const uintptr_t g_elem = plan->grad_dtype == RAFHIP_F32 ? 4 : 2;
-    std::vector<SgdRec> recs((size_t)plan->n);
+    std::vector<SgdRec>& recs = plan->recs;  // already n long
     for (int32_t t = 0; t < plan->n; ++t) {
       SgdRec& r = recs[t];
       r = SgdRec{x[t], dx[t], v[t], p ? p[t] : nullptr, plan->numel[t], 0, 0};
@@ -390,21 +363,21 @@ extern "C" int rafhip_sgd_multi_step(rafhip_sgd_plan* plan, float* const* x, con
                  aligned_to(r.p, 8);
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    RAFHIP_HIP_TRY(plan->recs.sync(recs, s));
+    const SgdRec* table = nullptr;
+    RAFHIP_HIP_TRY(plan->tables.sync(recs, s, &table));
     // One rounding double -> fp32, as for the single-tensor op.
     const float lr32 = static_cast<float>(learning_rate);
     const float mu32 = static_cast<float>(mu);
-    const int64_t cap = plan->blocks_per_cu > 0 ? (int64_t)streaming_grid_cap() / 8 * plan->blocks_per_cu
-                                                : (int64_t)1 << 20;
-    const unsigned grid = (unsigned)(plan->n_items < cap ? plan->n_items : cap);
+    // One workgroup per item; the kernel strides over what a launch cannot hold.
+    const unsigned grid = (unsigned)(plan->n_items < kMaxGridBlocks ? plan->n_items : kMaxGridBlocks);
     const bool nt = plan->total_elements * (int64_t)(8 + g_elem) > kSgdStreamFromBytes;
     const int bf = p_dtype == RAFHIP_BF16 ? 1 : 0;
     if (plan->grad_dtype == RAFHIP_F16)
-      launch_sgd_multi<_Float16>(nt, plan->unroll, grid, s, plan->d_recs, plan->d_items, plan->n_items, lr32, mu32, bf, plan->chunk_shift);
+      launch_sgd_multi<_Float16>(nt, grid, s, table, plan->d_items, plan->n_items, lr32, mu32, bf);
     else if (plan->grad_dtype == RAFHIP_BF16)
-      launch_sgd_multi<Bf16>(nt, plan->unroll, grid, s, plan->d_recs, plan->d_items, plan->n_items, lr32, mu32, bf, plan->chunk_shift);
+      launch_sgd_multi<Bf16>(nt, grid, s, table, plan->d_items, plan->n_items, lr32, mu32, bf);
     else
-      launch_sgd_multi<float>(nt, plan->unroll, grid, s, plan->d_recs, plan->d_items, plan->n_items, lr32, mu32, bf, plan->chunk_shift);
+      launch_sgd_multi<float>(nt, grid, s, table, plan->d_items, plan->n_items, lr32, mu32, bf);
     RAFHIP_HIP_TRY(hipGetLastError());
     return RAFHIP_OK;
   });

@@ -30,16 +30,6 @@ inline int check_plan_device(const char* who, int plan_device) {
   return RAFHIP_OK;
 }
 
-// A tuning knob from the environment: a non-negative integer, or `fallback` when unset or malformed.
-inline int env_knob(const char* name, int fallback) {
-  if (const char* e = std::getenv(name)) {
-    char* end = nullptr;
-    const long v = std::strtol(e, &end, 10);
-    if (end != e && *end == '\0' && v >= 0 && v <= (1 << 30)) return (int)v;
-  }
-  return fallback;
-}
-
 // No C++ exception may cross the C boundary: entry points that allocate host memory (work lists,
 // tables) run their body through this and report a failure as RAFHIP_ERR_HOST instead.
 template <typename F>

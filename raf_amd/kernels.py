@@ -245,6 +245,11 @@ class LansPlan:
     def schedule(self) -> str:
         return {0: "phased", 1: "pipelined"}[self.lib.rafhip_lans_plan_schedule(self._h)]
 
+    @property
+    def table_uploads(self) -> int:
+        """How often a pointer table had to be sent to the device so far."""
+        return self.lib.rafhip_lans_plan_table_uploads(self._h)
+
     def close(self):
         if self._h:
             self.lib.rafhip_lans_plan_destroy(self._h)

@@ -13,7 +13,6 @@ from __future__ import annotations
 
 import collections
 import ctypes
-import weakref
 from ctypes import c_int64, c_void_p
 from typing import Dict, List, Sequence, Tuple
 
@@ -131,61 +130,142 @@ _env_cache = _EnvCache()
 
 def clear_op_env_cache() -> None:
     _env_cache.clear()
-    _marshalled.clear()
-    _slots.clear()
-    _sig_tokens.clear()
+    _recent_lists.clear()
 
 
-class _Marshalled:
-    """Descriptors, signature and identity of a tensor list that has been handed to an op before."""
+class TensorList:
+    """A tensor list held the way RAF's callers hold one: as an immutable tuple value
+    (``TupleValue`` of ``TensorValue``s, include/raf/value.h).  The descriptors, the addresses and
+    the C++ tuple are made once; ``lans`` / ``lans_mixed`` / ``sgd_multi`` accept the handle
+    wherever they accept a list, and a call with it marshals nothing.
 
-    def __init__(self, tensors):
-        self.keep: list = []
-        self.descs = (TensorDesc * max(len(tensors), 1))(*[_desc(t, self.keep) for t in tensors])
-        self.sig = tuple(_sig(t) for t in tensors)
-        # A small number that stands for the signature in OpEnv keys: hashing a tuple of thousands
-        # of (shape, dtype, device) entries at every dictionary operation costs tens of microseconds.
-        self.sig_token = _sig_tokens.setdefault(self.sig, len(_sig_tokens))
-        # Once one of the tensors has died its id may be handed to another object: the weak
-        # references notice, and the entry is never trusted again.
-        self.alive = True
-        self.refs = [weakref.ref(t, self._one_died) for t in tensors]
-        self.ptrs = list(map(torch.Tensor.data_ptr, tensors))
-        self.slot = 0
+    The handle records where the tensors' storage was when it was made.  Unless ``track=False``
+    every use checks, in one pass at C speed, that each tensor still lives there (``x.data = ...``,
+    ``set_()`` and ``resize_()`` move a tensor without replacing the Python object) and rebuilds
+    the handle if not, so it is never silently stale; ``rebuilds`` counts that.  With
+    ``track=False`` the caller vouches for it, as for a ``TupleValue``, which nothing re-reads.
+    Either way the handle keeps the tensors alive."""
 
-    def _one_died(self, _ref) -> None:
-        self.alive = False
+    def __init__(self, tensors, track: bool = True, _share=None):
+        self._tensors = list(tensors)
+        self.track = bool(track)
+        self.rebuilds = 0
+        self._handle = c_void_p(None)
+        self._build(_share)
 
-    def still_describes(self, tensors) -> bool:
-        # The caller found this entry under the ids of `tensors`, and all of the original objects
-        # are alive, so these are the same objects; their shapes and dtypes cannot have changed,
-        # their storage can (x.data = ..., set_, resize_): the addresses are compared, at C speed.
-        return self.alive and list(map(torch.Tensor.data_ptr, tensors)) == self.ptrs
+    def _build(self, share=None) -> None:
+        lib, glue = _lib.dialect(), _lib.glue()
+        n = len(self._tensors)
+        if share is None:
+            self._descs = (TensorDesc * max(n, 1))()
+            self._ptrs = (ctypes.c_uint64 * max(n, 1))()
+            self._shapes = (c_int64 * max(8 * n, 1))()
+            try:
+                glue.describe(self._tensors, ctypes.addressof(self._descs), ctypes.addressof(self._shapes),
+                              len(self._shapes), ctypes.addressof(self._ptrs))
+            except ValueError as e:
+                if "shape buffer" not in str(e):
+                    raise
+                self._shapes = (c_int64 * max(sum(t.dim() for t in self._tensors), 1))()
+                glue.describe(self._tensors, ctypes.addressof(self._descs), ctypes.addressof(self._shapes),
+                              len(self._shapes), ctypes.addressof(self._ptrs))
+            h = c_void_p(None)
+            check_raf(lib.rafhip_raf_tuple_make(n, self._descs, ctypes.byref(h)))
+        else:
+            # Everything outside [first, end) is the other handle's: its descriptors are copied, its
+            # tensor values shared; only the fields in the range are described and made anew.
+            base, first, end = share
+            k = end - first
+            self._descs = (TensorDesc * max(n, 1))()
+            ctypes.memmove(self._descs, base._descs, ctypes.sizeof(TensorDesc) * n)
+            self._ptrs = (ctypes.c_uint64 * max(n, 1))()
+            ctypes.memmove(self._ptrs, base._ptrs, 8 * n)
+            part = (c_int64 * max(8 * k, 1))()
+            glue.describe(self._tensors[first:end], ctypes.addressof(self._descs) + ctypes.sizeof(TensorDesc) * first,
+                          ctypes.addressof(part), len(part), ctypes.addressof(self._ptrs) + 8 * first)
+            self._shapes = (base._shapes, part)  # both stay alive: the descriptors point into them
+            h = c_void_p(None)
+            check_raf(lib.rafhip_raf_tuple_replace(base._handle, first, k,
+                                                   ctypes.cast(ctypes.addressof(self._descs) +
+                                                               ctypes.sizeof(TensorDesc) * first,
+                                                               ctypes.POINTER(TensorDesc)), ctypes.byref(h)))
+        old, self._handle = self._handle, h
+        if old:
+            lib.rafhip_raf_tuple_destroy(old)
+        # What identifies an OpEnv made for this list: every tensor's dtype, device and shape.  A
+        # bytes object, so that a dictionary compares two lists' signatures with one memcmp and
+        # the handle's own signature by identity.
+        self.signature = glue.signature(ctypes.addressof(self._descs), n)
+
+    def current(self) -> bool:
+        """Whether every tensor's storage is where it was when the handle was made."""
+        return _lib.glue().same_storage(self._tensors, ctypes.addressof(self._ptrs))
+
+    def refresh(self) -> "TensorList":
+        """Brings the handle up to date with its tensors if their storage moved."""
+        if not self.current():
+            self._build()
+            self.rebuilds += 1
+        return self
+
+    def replaced(self, first: int, tensors) -> "TensorList":
+        """A new handle that differs from this one in the tensors from ``first`` on (as many as
+        given): the list of the next step when, say, only the gradients were allocated anew."""
+        tensors = list(tensors)
+        end = first + len(tensors)
+        if first < 0 or end > len(self._tensors):
+            raise IndexError("replacement range outside the list")
+        merged = self._tensors[:first] + tensors + self._tensors[end:]
+        return TensorList(merged, self.track, _share=(self, first, end))
+
+    def __len__(self):
+        return len(self._tensors)
+
+    def __getitem__(self, i):
+        return self._tensors[i]
+
+    def __iter__(self):
+        return iter(self._tensors)
+
+    def __del__(self):
+        try:
+            if self._handle:
+                _lib.dialect().rafhip_raf_tuple_destroy(self._handle)
+        except Exception:
+            pass
 
 
-_marshalled: Dict[Tuple, _Marshalled] = {}
-_sig_tokens: Dict[Tuple, int] = {}  # signature of a tensor list -> its number (never reused)
-_SLOTS_PER_SIGNATURE = 4
-_slots: Dict[int, list] = {}  # signature number -> identities (id tuples) of the lists seen, by slot
+_recent_lists: "collections.deque[TensorList]" = collections.deque(maxlen=8)
 
 
-def _marshal_list(tensors: list) -> _Marshalled:
-    """Marshalling a list of hundreds of tensors costs milliseconds of Python; a training loop passes
-    the same tensors every step, so the last marshalling of every distinct list is kept.  Lists of
-    equal signature get different ``slot`` numbers (up to a few; beyond that they share the last)."""
-    key = tuple(map(id, tensors))
-    m = _marshalled.get(key)
-    if m is None or not m.still_describes(tensors):
-        if len(_marshalled) >= 8:
-            _marshalled.clear()
-        m = _marshalled[key] = _Marshalled(tensors)
-        known = _slots.setdefault(m.sig_token, [])
-        if key not in known:
-            if len(known) >= _SLOTS_PER_SIGNATURE:
-                known.pop()
-            known.append(key)
-        m.slot = known.index(key)
-    return m
+def _tensor_list(tensors) -> TensorList:
+    """The handle behind a ``tensor_list`` argument.  A ``TensorList`` is used as it is (checked
+    against its tensors unless it was made with ``track=False``).  A plain sequence is looked up
+    among the handles made for recent calls by the identity of its elements -- a training loop
+    passes the same tensor objects every step -- and when only a stretch of it differs (fresh
+    gradient tensors, say) the new handle shares the rest with the old one."""
+    if isinstance(tensors, TensorList):
+        return tensors.refresh() if tensors.track else tensors
+    lst = tensors if type(tensors) is list else list(tensors)
+    glue = _lib.glue()
+    nearest = None
+    for h in _recent_lists:
+        if len(h) != len(lst):
+            continue
+        first, end = glue.diff_range(lst, h._tensors)
+        if first < 0:
+            if h is not _recent_lists[0]:
+                _recent_lists.remove(h)
+                _recent_lists.appendleft(h)
+            return h.refresh()
+        if nearest is None or end - first < nearest[2] - nearest[1]:
+            nearest = (h, first, end)
+    if nearest is not None and 2 * (nearest[2] - nearest[1]) <= len(lst) and nearest[0].current():
+        h = nearest[0].replaced(nearest[1], lst[nearest[1]:nearest[2]])
+    else:
+        h = TensorList(lst)
+    _recent_lists.appendleft(h)
+    return h
 
 
 def _sig(t: torch.Tensor):
@@ -385,21 +465,19 @@ def sgd_multi_mixed(tensor_list: Sequence[torch.Tensor], learning_rate, mu):
 
 def _sgd_multi(mixed, tensor_list, learning_rate, mu):
     lib = _lib.dialect()
-    tensor_list = list(tensor_list)
-    n = len(tensor_list)
-    m = _marshal_list(tensor_list)
-    descs = m.descs
-    key = ("sgd_multi", mixed, m.sig_token, m.slot, float(mu))
+    tl = _tensor_list(tensor_list)
+    n = len(tl)
+    key = ("sgd_multi", mixed, tl.signature, float(mu))
     env = _env_cache.get(key)
     if env is None:
         h = c_void_p(None)
-        check_raf(lib.rafhip_raf_sgd_multi_make(int(mixed), n, descs, float(learning_rate), float(mu),
+        check_raf(lib.rafhip_raf_sgd_multi_make(int(mixed), n, tl._descs, float(learning_rate), float(mu),
                                                 ctypes.byref(h)))
         env = _env_cache[key] = _Env(h)
         env.learning_rate = float(learning_rate)
     if n:
         env.set_learning_rate(float(learning_rate))
-    check_raf(lib.rafhip_raf_sgd_multi_execute(env.handle, n, descs, _stream(tensor_list[0]) if n else None))
+    check_raf(lib.rafhip_raf_sgd_multi_execute_tuple(env.handle, tl._handle, _stream(tl[0]) if n else None, _as_vm))
     return tensor_list
 
 
@@ -426,32 +504,29 @@ def lans_mixed(tensor_list: Sequence[torch.Tensor], step: torch.Tensor, learning
 def _lans(op_name, tensor_list, step, learning_rate, beta1, beta2, eps, bias_correction,
           weight_decay, grad_averaging, mode, normalize_grad):
     lib = _lib.dialect()
-    tensor_list = list(tensor_list)
     keep: list = []
-    n4 = len(tensor_list)
-    m = _marshal_list(tensor_list)
-    descs = m.descs
+    tl = _tensor_list(tensor_list)
+    n4 = len(tl)
     dstep = _desc(step, keep)
     hp = (float(learning_rate), float(beta1), float(beta2), float(eps), int(bias_correction),
           float(weight_decay), int(grad_averaging), int(mode), int(bool(normalize_grad)))
-    # All but the learning rate and the loss scaling.  `m.slot` tells lists of equal signature
-    # apart (two models of one architecture): each keeps an OpEnv, and with it a plan whose device
-    # pointer table follows that list alone.
-    key = (op_name, m.sig_token, m.slot, _sig(step), hp[1:])
+    # All but the learning rate and the loss scaling.  Lists of equal signature (two models of one
+    # architecture) share an OpEnv: its plan keeps a device pointer table per recent list.
+    key = (op_name, tl.signature, _sig(step), hp[1:])
     env = _env_cache.get(key)
     if env is None:
         h = c_void_p(None)
         make = lib.rafhip_raf_lans_make if op_name == "lans" else lib.rafhip_raf_lans_mixed_make
-        check_raf(make(n4, descs, dstep, *hp, ctypes.byref(h)))
+        check_raf(make(n4, tl._descs, dstep, *hp, ctypes.byref(h)))
         env = _env_cache[key] = _Env(h)
         env.learning_rate = hp[0]
     if n4:
         env.set_learning_rate(hp[0])
         env.set_grad_scaling(_lans_grad_unscale, _lans_dynamic_scale)
-    stream = _stream(tensor_list[0]) if n4 else None
-    ws = _workspace(env, tensor_list[0], stream) if env.workspace_bytes > 0 else None
-    check_raf(lib.rafhip_raf_lans_execute(env.handle, n4, descs, dstep, ws.data if ws else None,
-                                          env.workspace_bytes, stream))
+    stream = _stream(tl[0]) if n4 else None
+    ws = _workspace(env, tl[0], stream) if env.workspace_bytes > 0 else None
+    check_raf(lib.rafhip_raf_lans_execute_tuple(env.handle, tl._handle, dstep, ws.data if ws else None,
+                                                env.workspace_bytes, stream, _as_vm))
     return tensor_list
 
 
@@ -536,6 +611,16 @@ def defuse_tensor(data: torch.Tensor, sizes, shapes, shape_indices):
 
 _lans_grad_unscale = 1.0
 _lans_dynamic_scale = (None, None)
+_as_vm = 0
+
+
+def set_executor(kind: str) -> None:
+    """Which of RAF's executors the multi-tensor ops imitate when they hand a tensor list to an
+    OpEnv: "interpreter" passes the list's tuple value itself (src/impl/interpreter.cc:286-325),
+    "vm" a newly allocated ``TupleValue`` over the same tensor values at every call, which is what
+    the VM's AllocTuple instruction produces per iteration (src/impl/vm/vm.cc:764-769)."""
+    global _as_vm
+    _as_vm = {"interpreter": 0, "vm": 1}[kind]
 
 
 def set_lans_grad_unscale(factor: float) -> None:
@@ -561,6 +646,11 @@ def set_lans_dynamic_scale(grad_unscale: torch.Tensor = None, found_inf: torch.T
                               or not t.is_cuda):
             raise TypeError(f"{name} must be a one-element float32 GPU tensor")
     _lans_dynamic_scale = (grad_unscale, found_inf)
+
+
+def get_lans_dynamic_scale():
+    """The (grad_unscale, found_inf) tensors in force, either of them possibly None."""
+    return _lans_dynamic_scale
 
 
 def dispatch_list(base_op: str, device_type: int = DEV_ROCM) -> List[Tuple[str, str, int]]:

@@ -162,6 +162,14 @@ class LANS:
         return self._model[1]
 
     def _advance(self):
+        """``_step`` counts the calls made; the counter the kernels read lives on the device and
+        counts the steps that were applied: with dynamic loss scaling in force
+        (``op.set_lans_dynamic_scale(found_inf=...)``) a step the kernels skipped because of an
+        overflow leaves it where it was, so the bias corrections stay in step with m and v."""
         self._step += 1
         if self._step_dev is not None:
-            self._step_dev.add_(1.0)
+            found_inf = _op.get_lans_dynamic_scale()[1]
+            if found_inf is None:
+                self._step_dev.add_(1.0)
+            else:
+                self._step_dev.add_((found_inf == 0).to(torch.float32).reshape(()))

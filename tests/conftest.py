@@ -35,7 +35,7 @@ def native_libs():
     """The in-tree HIP libraries; built on first use only if nothing is built yet."""
     from raf_amd import _lib, build
 
-    if not _lib.OPTIM_LIB.exists() or not _lib.DIALECT_LIB.exists():
+    if not _lib.OPTIM_LIB.exists() or not _lib.DIALECT_LIB.exists() or not _lib.GLUE_LIB.exists():
         build.build_all()
     return _lib
 

@@ -715,6 +715,38 @@ def test_two_lists_alternating_on_two_streams_through_one_plan(native_libs):
     plan.close()
 
 
+def test_alternating_pointer_lists_stop_uploading(native_libs):
+    """A plan keeps a device pointer table per recent pointer list: gradients that alternate between
+    two allocations (what an executor that allocates them per iteration produces) cost two uploads
+    in all, a list seen before is found again after others were used, a fifth distinct list replaces
+    the least recently used one -- and every step reads the right table (checked against the oracle
+    with different gradient values in every allocation)."""
+    from raf_amd import kernels
+
+    sizes = [70001, 5, 1 << 16, 4096, 300_000]
+    hp = LansHParams()
+    _, w, m, v = lans_inputs(sizes, cfg=120)
+    grads = [lans_inputs(sizes, cfg=121 + k)[0] for k in range(5)]
+    tw, tm, tv = _to_dev(w), _to_dev(m), _to_dev(v)
+    tgs = [_to_dev(g) for g in grads]
+    plan = kernels.LansPlan(sizes, torch.float32, DEV)
+    order = [0, 1, 0, 1, 0, 1, 2, 0, 3, 4, 1, 1]
+    uploads = []
+    for i, k in enumerate(order):
+        plan.step(tgs[k], tw, tm, tv, i + 1, _khp(hp))
+        uploads.append(plan.table_uploads)
+    torch.cuda.synchronize()
+    plan.read_norms()
+    #            0  1  0  1  0  1  2  0  3  4  1 (evicted by 4: sent again)  1
+    assert uploads == [1, 2, 2, 2, 2, 2, 3, 3, 4, 5, 6, 6], uploads
+    ow, om, ov = w, m, v
+    for i, k in enumerate(order):
+        ow, om, ov, _ = lans_f64.lans_step(grads[k], ow, om, ov, i + 1, hp)
+    _assert_close([t.cpu().numpy() for t in tw], ow, 1e-4, "w")
+    _assert_close([t.cpu().numpy() for t in tv], ov, 1e-4, "v")
+    plan.close()
+
+
 def test_per_kernel_timing_slots(native_libs):
     """rafhip_lans_timing_*: five intervals per step, zero where the schedule launches nothing."""
     from raf_amd import kernels
