@@ -145,11 +145,27 @@ def workloads():
     }
 
 
-def gen_lans(sizes, g16, zero_state, dev, seed=2024):
+def gen_lans(sizes, g16, zero_state, dev, seed=2024, flat=False):
+    """Seeded synthetic tensors generated on the GPU.  `flat`: four flat buffers cut into views
+    that start on 512-byte boundaries (where torch's allocator would put separate tensors): a
+    handful of generator launches instead of two per tensor, for runs under a profiler."""
     import torch
 
     gen = torch.Generator(device=dev)
     gen.manual_seed(seed)
+    if flat:
+        starts, total = [], 0
+        for n in sizes:
+            starts.append(total)
+            total += -(-n // 128) * 128
+        cut = lambda buf: [buf[s:s + n] for s, n in zip(starts, sizes)]
+        gt = torch.randn(total, device=dev, generator=gen) * 1e-3
+        g = cut((gt * 1024.0).half() if g16 else gt)
+        w = cut(torch.randn(total, device=dev, generator=gen) * 0.02)
+        if zero_state:
+            return g, w, cut(torch.zeros(total, device=dev)), cut(torch.zeros(total, device=dev))
+        return (g, w, cut(torch.randn(total, device=dev, generator=gen) * 1e-4),
+                cut((torch.randn(total, device=dev, generator=gen) * 1e-6).abs()))
     g, w, m, v = [], [], [], []
     for n in sizes:
         gt = torch.randn(n, device=dev, generator=gen) * 1e-3
@@ -328,7 +344,7 @@ def bench_lans(name, wl, args, entry="c_abi", parity=True, cpu_baseline=True):
     dev = torch.device("cuda:0")
     sizes, g16 = wl["sizes"], wl["g16"]
     total = sum(sizes)
-    g, w, m, v = gen_lans(sizes, g16, wl["zero_state"], dev)
+    g, w, m, v = gen_lans(sizes, g16, wl["zero_state"], dev, flat=getattr(args, "flat_inputs", False))
     hp = kernels.make_hparams(grad_unscale=(1.0 / 1024 if g16 else 1.0))
     copy16 = bool(wl.get("copy16"))
     p16 = [torch.empty(n, dtype=torch.float16, device=dev) for n in sizes] if copy16 else None
@@ -921,6 +937,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline leg")
     ap.add_argument("--no-parity", action="store_true", help="skip the parity check after the timed region")
     ap.add_argument("--no-kernel-events", action="store_true", help="do not record per-kernel HIP events")
+    ap.add_argument("--flat-inputs", action="store_true",
+                    help="LANS workloads: generate the list as four flat buffers cut into views (a few "
+                         "generator launches instead of thousands; for runs under rocprofv3 --pmc)")
     ap.add_argument("--hip-graph", action="store_true",
                     help="LANS workloads: capture one step in a HIP graph and time its replays")
     args = ap.parse_args()

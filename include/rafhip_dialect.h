@@ -130,6 +130,14 @@ int rafhip_raf_defuse_tensor_make(const rafhip_tensor_desc* data, int32_t n_size
 int rafhip_raf_defuse_tensor_execute(rafhip_raf_env* env, const rafhip_tensor_desc* data,
                                      int32_t n_out, const rafhip_tensor_desc* outs, void* stream);
 
+/* OpEnv::RequestStream (include/raf/op.h:87).  The fuse_tensor and defuse_tensor OpEnvs request a
+ * copy stream the way the reference's do (src/op/dialect/cuda/memory.cc:34, :89).  By default this
+ * window leaves such requests unserved and the OpEnv launches on the `stream` argument.  With
+ * enable != 0 (per calling thread) the execute calls serve them from a pool of streams per
+ * (device, tag) and order that stream behind `stream` before Execute and `stream` behind it
+ * afterwards, so the results are still in `stream`'s order. */
+int rafhip_raf_serve_stream_requests(int32_t enable);
+
 /* What the op's declare function produced (call->out): number of output tensors (a tuple counts
  * its fields; -1 on NULL) and each one's dtype and shape, so that the caller can allocate them the
  * way an executor does (src/impl/interpreter.cc:397-426).  shape_out may be NULL to query ndim. */

@@ -163,6 +163,7 @@ DIALECT_SYMBOLS = {
                                               POINTER(c_int64), c_int32, POINTER(c_int64), POINTER(c_void_p)]),
     "rafhip_raf_defuse_tensor_execute": (c_int, [c_void_p, POINTER(TensorDesc), c_int32, POINTER(TensorDesc),
                                                  c_void_p]),
+    "rafhip_raf_serve_stream_requests": (c_int, [c_int32]),
     "rafhip_raf_env_num_outputs": (c_int32, [c_void_p]),
     "rafhip_raf_env_output": (c_int, [c_void_p, c_int32, POINTER(c_int32), POINTER(c_int32), POINTER(c_int32),
                                       POINTER(c_int64), c_int32]),

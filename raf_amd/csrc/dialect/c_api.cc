@@ -1,6 +1,9 @@
 // C entry points declared in rafhip_dialect.h: a minimal executor around the OpEnv mirror.
 #include <cstring>
+#include <map>
 #include <memory>
+#include <mutex>
+#include <tuple>
 #include <sstream>
 #include <string>
 
@@ -130,6 +133,67 @@ struct WorkspaceBinding {
     }
   }
   ~WorkspaceBinding() {
+    for (const auto& r : reqs) *r.dest = nullptr;
+  }
+};
+
+// Stream requests (OpEnv::RequestStream).  Off by default: the requests stay unserved (*dest is
+// null) and an OpEnv launches on the compute stream.  Switched on, the executor serves them from a
+// pool of streams per (device, tag), like Stream::Get in the reference (src/impl/interpreter.cc:384-389),
+// and -- since a caller of this window expects an operator's results in stream order -- makes the
+// requested stream wait for the compute stream before Execute and the compute stream wait for
+// the requested stream after it.
+thread_local bool g_serve_stream_requests = false;
+
+struct StreamPool {
+  std::mutex mu;
+  std::map<std::tuple<int, int, int, int>, void*> streams;  // (device type, device id, tag, index)
+  void* Get(const Device& dev, int tag, int index) {
+    std::lock_guard<std::mutex> lock(mu);
+    void*& s = streams[std::make_tuple((int)dev.device_type(), dev.device_id(), tag, index)];
+    if (!s) s = device_api::DeviceAPI::Get(dev.device_type())->CreateStream(dev);
+    return s;
+  }
+};
+StreamPool& Streams() {
+  static StreamPool* pool = new StreamPool();  // streams live as long as the process
+  return *pool;
+}
+
+struct StreamBinding {
+  const std::vector<StreamRequest>& reqs;
+  std::shared_ptr<device_api::DeviceAPI> api;
+  Device device;
+  void* compute = nullptr;
+  std::vector<void*> served;
+  StreamBinding(OpEnv* env, const Device& dev, void* compute_stream)
+      : reqs(env->stream_requests()), device(dev), compute(compute_stream) {
+    if (!g_serve_stream_requests || reqs.empty()) {
+      for (const auto& r : reqs) *r.dest = nullptr;
+      return;
+    }
+    api = device_api::DeviceAPI::Get(dev.device_type());
+    void* ev = api->CreateEvent(dev, 0);
+    api->EventRecordOnStream(ev, compute);
+    for (const auto& r : reqs) {
+      void* s = Streams().Get(r.device, r.tag_idx, r.stream_idx);
+      api->StreamWaitEvent(s, ev);
+      *r.dest = s;
+      served.push_back(s);
+    }
+    api->FreeEvent(dev, ev);
+  }
+  // Ordering the compute stream behind the served streams can fail; call it on the normal path.
+  void Finish() {
+    for (void* s : served) {
+      void* ev = api->CreateEvent(device, 0);
+      api->EventRecordOnStream(ev, s);
+      api->StreamWaitEvent(compute, ev);
+      api->FreeEvent(device, ev);
+    }
+    served.clear();
+  }
+  ~StreamBinding() {
     for (const auto& r : reqs) *r.dest = nullptr;
   }
 };
@@ -635,7 +699,9 @@ int rafhip_raf_fuse_tensor_execute(rafhip_raf_env* env, int32_t n, const rafhip_
     std::vector<value::Value> inputs = {value::MakeTuple(std::move(fields))};
     OpEnv::SetStreamForAllBackends(env->call->device, stream);
     WorkspaceBinding bind(env->env.get(), nullptr, 0);
+    StreamBinding streams(env->env.get(), env->call->device, stream);
     env->env->Execute(inputs, FromDesc(out, "out"));
+    streams.Finish();
   });
 }
 
@@ -666,8 +732,14 @@ int rafhip_raf_defuse_tensor_execute(rafhip_raf_env* env, const rafhip_tensor_de
     std::vector<value::Value> inputs = {FromDesc(data, "data")};
     OpEnv::SetStreamForAllBackends(env->call->device, stream);
     WorkspaceBinding bind(env->env.get(), nullptr, 0);
+    StreamBinding streams(env->env.get(), env->call->device, stream);
     env->env->Execute(inputs, value::MakeTuple(std::move(fields)));
+    streams.Finish();
   });
+}
+
+int rafhip_raf_serve_stream_requests(int32_t enable) {
+  return Guard([&] { g_serve_stream_requests = enable != 0; });
 }
 
 int32_t rafhip_raf_env_num_outputs(const rafhip_raf_env* env) {

@@ -443,8 +443,11 @@ class L2NormHipEnv : public OpEnv {
 
 // ------------------------------------------------------------------------- fuse / defuse tensor
 // Both hold a plan made from the tensors' byte sizes, which the reference's constructors record
-// too (memory.cc:37-43, :99-103).  The reference issues its copies on a dedicated copy stream
-// (RequestStream, memory.cc:32, :93); here the single launch goes to the current compute stream.
+// too (memory.cc:37-43, :99-103), and both request a copy stream with the reference's tags
+// (RequestStream, memory.cc:34, :89).  An executor that serves the request gets the single launch
+// on that stream (and owns the ordering against the compute stream, as in the reference); one
+// that leaves it unserved gets it on the current compute stream, which is the right place when
+// nothing else could run beside the copy.
 class FuseBase : public OpEnv {
  public:
   ~FuseBase() override {
@@ -453,8 +456,13 @@ class FuseBase : public OpEnv {
   std::string name() const override { return name_; }
 
  protected:
-  FuseBase(const char* op, const CallValues& cv) : op_(op), name_(TruncateName(GetUniqueName(op))) {
+  FuseBase(const char* op, const CallValues& cv, int stream_tag)
+      : op_(op), name_(TruncateName(GetUniqueName(op))) {
     if (cv->device.device_type() != DevType::kROCM()) error_msgs.push_back(op_ + ": device is not rocm");
+    RequestStream(&stream_, cv->device, stream_tag);
+  }
+  void* LaunchStream() const {
+    return stream_ ? stream_ : DeviceAPI::Get(DevType::kROCM())->GetStream();
   }
   void MakePlan(const std::vector<int64_t>& nbytes) {
     if (!error_msgs.empty()) return;
@@ -475,11 +483,13 @@ class FuseBase : public OpEnv {
   std::string op_, name_;
   rafhip_fuse_plan* plan_ = nullptr;
   size_t n_ = 0;
+  void* stream_ = nullptr;  // bound by the executor around Execute, or left null
 };
 
 class FuseTensorHipEnv : public FuseBase {
  public:
-  explicit FuseTensorHipEnv(const CallValues& cv) : FuseBase("raf.op.hip.fuse_tensor", cv) {
+  explicit FuseTensorHipEnv(const CallValues& cv)
+      : FuseBase("raf.op.hip.fuse_tensor", cv, stream_pool::kMemCpyCudaToCuda1) {
     const auto* args = cv->args_as<schema::FuseTensorArgs>();
     if (!args) {
       error_msgs.push_back(op_ + ": call does not carry FuseTensorArgs");
@@ -499,7 +509,7 @@ class FuseTensorHipEnv : public FuseBase {
   void Execute(const std::vector<Value>& inputs, Value output) override {
     RAF_CHECK(inputs.size() == 1, op_ + " takes (data)");
     std::vector<void*> ptrs = Pointers(AsTuple(inputs[0]));
-    void* stream = DeviceAPI::Get(DevType::kROCM())->GetStream();
+    void* stream = LaunchStream();
     int st = rafhip_fuse_tensors(plan_, ptrs.data(), AsTensor(output)->tensor.data, stream);
     if (st != RAFHIP_OK) throw Error(KernelError("rafhip_fuse_tensors", st));
   }
@@ -508,7 +518,8 @@ class FuseTensorHipEnv : public FuseBase {
 
 class DefuseTensorHipEnv : public FuseBase {
  public:
-  explicit DefuseTensorHipEnv(const CallValues& cv) : FuseBase("raf.op.hip.defuse_tensor", cv) {
+  explicit DefuseTensorHipEnv(const CallValues& cv)
+      : FuseBase("raf.op.hip.defuse_tensor", cv, stream_pool::kMemCpyCudaToCuda2) {
     const auto* args = cv->args_as<schema::DefuseTensorArgs>();
     if (!args) {
       error_msgs.push_back(op_ + ": call does not carry DefuseTensorArgs");
@@ -528,7 +539,7 @@ class DefuseTensorHipEnv : public FuseBase {
   void Execute(const std::vector<Value>& inputs, Value output) override {
     RAF_CHECK(inputs.size() == 1, op_ + " takes (data)");
     std::vector<void*> ptrs = Pointers(AsTuple(output));
-    void* stream = DeviceAPI::Get(DevType::kROCM())->GetStream();
+    void* stream = LaunchStream();
     int st = rafhip_defuse_tensor(plan_, AsTensor(inputs[0])->tensor.data, ptrs.data(), stream);
     if (st != RAFHIP_OK) throw Error(KernelError("rafhip_defuse_tensor", st));
   }

@@ -251,6 +251,27 @@ struct WorkspaceRequest {
   int64_t nbytes;
 };
 
+// include/raf/stream_pool.h:52-76: what a requested stream is for.  The copy tags are the ones
+// the fuse / defuse OpEnvs ask for (src/op/dialect/cuda/memory.cc:34, :89).
+namespace stream_pool {
+enum StreamTag : int {
+  kUnknown = 0,
+  kCudaCompute = 1,
+  kMemCpyCpuToCuda = 2,
+  kMemCpyCudaToCpu = 3,
+  kCudaCommunicate = 4,
+  kMemCpyCudaToCuda1 = 5,
+  kMemCpyCudaToCuda2 = 6,
+};
+}  // namespace stream_pool
+
+struct StreamRequest {  // requests::Requests::StreamRequest (src/requests.h)
+  void** dest;
+  Device device;
+  int tag_idx;
+  int stream_idx;
+};
+
 class OpEnv {
  public:
   OpEnv() = default;
@@ -266,6 +287,10 @@ class OpEnv {
   // Execute and may take it back afterwards.
   void RequestWorkspace(void** dest, const Device& device, int64_t nbytes);
   const std::vector<WorkspaceRequest>& workspace_requests() const { return workspace_; }
+  // Also recorded at construction; the executor points *dest at a stream of its pool for
+  // (device, tag_idx) before Execute (src/impl/interpreter.cc:384-389, src/impl/vm/vm.cc:1082-1091).
+  void RequestStream(void** dest, const Device& device, int tag_idx);
+  const std::vector<StreamRequest>& stream_requests() const { return stream_; }
 
   std::vector<int> arg_indices;  // schema fields handed to Execute(inputs, output) by the VM
 
@@ -273,6 +298,7 @@ class OpEnv {
 
  private:
   std::vector<WorkspaceRequest> workspace_;
+  std::vector<StreamRequest> stream_;
 };
 using OpEnvPtr = std::shared_ptr<OpEnv>;
 

@@ -262,6 +262,11 @@ void OpEnv::RequestWorkspace(void** dest, const Device& device, int64_t nbytes) 
   workspace_.push_back(WorkspaceRequest{dest, device, nbytes});
 }
 
+void OpEnv::RequestStream(void** dest, const Device& device, int tag_idx) {  // src/impl/op.cc:66-72
+  const int index = (int)stream_.size();
+  stream_.push_back(StreamRequest{dest, device, tag_idx, index});
+}
+
 void OpEnv::SetStreamForAllBackends(Device device, void* stream) {
   device_api::DeviceAPI::Get(device.device_type())->SetStream(device, stream);  // src/impl/op.cc:92-96
 }

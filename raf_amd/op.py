@@ -648,6 +648,14 @@ def set_lans_dynamic_scale(grad_unscale: torch.Tensor = None, found_inf: torch.T
     _lans_dynamic_scale = (grad_unscale, found_inf)
 
 
+def serve_stream_requests(enable: bool) -> None:
+    """Whether this thread's executor stand-in serves ``OpEnv::RequestStream`` (include/raf/op.h:87):
+    with it, ``fuse_tensor`` / ``defuse_tensor`` run on the copy stream they request, as the
+    reference's do (src/op/dialect/cuda/memory.cc:34, :89), ordered behind the current stream
+    before and in front of it after; without it (the default) they run on the current stream."""
+    check_raf(_lib.dialect().rafhip_raf_serve_stream_requests(int(bool(enable))))
+
+
 def get_lans_dynamic_scale():
     """The (grad_unscale, found_inf) tensors in force, either of them possibly None."""
     return _lans_dynamic_scale

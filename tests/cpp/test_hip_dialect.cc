@@ -154,6 +154,7 @@ int main() {
     EXPECT(value::AsTuple(lc->out)->fields[2] == l->tensor_list[2]);  // output aliases the inputs
     OpEnvPtr le((*OpEnvMaker::Get("raf.op.hip.lans"))(lc));
     EXPECT(le->HasError() && le->error_msgs[0].find("FP32") != std::string::npos);
+    EXPECT(le->stream_requests().empty());  // the optimizer steps run on the compute stream
     EXPECT((le->arg_indices == std::vector<int>{0, 1}));
   }
 
@@ -214,6 +215,11 @@ int main() {
     d->sizes = {15, 7, 1};
     OpEnvPtr de((*OpEnvMaker::Get("raf.op.hip.defuse_tensor"))(dc));
     EXPECT((de->arg_indices == std::vector<int>{0}));
+    // the copy streams the reference's fuse / defuse OpEnvs request (cuda/memory.cc:34, :89)
+    OpEnvPtr fe2((*OpEnvMaker::Get("raf.op.hip.fuse_tensor"))(fc));
+    EXPECT(fe2->stream_requests().size() == 1 && fe2->stream_requests()[0].tag_idx == stream_pool::kMemCpyCudaToCuda1);
+    EXPECT(de->stream_requests().size() == 1 && de->stream_requests()[0].tag_idx == stream_pool::kMemCpyCudaToCuda2 &&
+           de->stream_requests()[0].stream_idx == 0 && de->stream_requests()[0].dest != nullptr);
     auto cpu = std::make_shared<schema::L2NormArgs>();
     cpu->x = T({4}, DevType::kCPU());
     auto cc = MakeCall("raf.op.l2norm", cpu);

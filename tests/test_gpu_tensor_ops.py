@@ -258,3 +258,33 @@ def test_tensor_fusion_and_defusion(native_libs, shape, dtype):
         x_3 = op.defuse_tensor(x_2, sizes, tuple_shape, shape_indices)
     assert x_2.shape == (2 * size,) and x_2.dtype == dtype
     assert len(x_3) == 2 and all(y.shape == x.shape and torch.equal(y, x) for y in x_3)
+
+
+def test_fuse_and_defuse_on_a_requested_copy_stream(native_libs):
+    """With the executor serving OpEnv::RequestStream, fuse_tensor / defuse_tensor run on the copy
+    streams they request (the reference's tags, src/op/dialect/cuda/memory.cc:34, :89), ordered
+    against the current stream on both sides: producers enqueued before the op and consumers
+    enqueued after it, all on the current stream, see the right bytes."""
+    from raf_amd import op
+
+    parts = [torch.zeros(n, device=DEV) for n in (1 << 20, 70_001, 3, 1 << 22)]
+    host = None
+    op.serve_stream_requests(True)
+    try:
+        for rep in range(3):
+            for k, t in enumerate(parts):  # producers on the current stream, right before the op
+                t.fill_(float(10 * rep + k))
+            flat = op.fuse_tensor(parts)
+            total = flat.sum()  # a consumer on the current stream, right after the op
+            want = sum(float(10 * rep + k) * t.numel() for k, t in enumerate(parts))
+            assert float(total) == want
+            flat.mul_(2.0)
+            sizes, shapes, idx = tensor_ops.defuse_args([t.cpu().numpy() for t in parts])
+            back = op.defuse_tensor(flat, sizes, shapes, idx)
+            for k, b in enumerate(back):
+                assert torch.equal(b, parts[k] * 2.0)
+    finally:
+        op.serve_stream_requests(False)
+    # and without it the same results on the current stream
+    flat = op.fuse_tensor(parts)
+    assert torch.equal(flat, torch.cat([t.reshape(-1) for t in parts]))
