@@ -146,8 +146,8 @@ int32_t rafhip_lans_pass_a_unit_elements(int64_t numel);
  *              neighbouring cache-sized tensor groups, so that a group's second and third reads
  *              come from the 256 MB Infinity Cache instead of HBM.
  * A plan picks PIPELINED for lists of 64 Mi elements or more and PHASED below (short lists are
- * launch- and latency-bound); RAFHIP_LANS_SCHEDULE=phased|pipelined overrides that per process and
- * rafhip_lans_plan_set_schedule per plan.
+ * launch- and latency-bound); RAFHIP_LANS_SCHEDULE=phased|pipelined overrides that per process,
+ * rafhip_lans_plan_options.schedule and rafhip_lans_plan_set_schedule per plan.
  */
 typedef enum rafhip_lans_schedule {
   RAFHIP_LANS_PHASED = 0,
@@ -171,6 +171,39 @@ int rafhip_lans_pipeline_order(int32_t n_tensors, const int64_t* numel, int64_t 
 /* numel[i] >= 0 (zero-sized tensors are allowed and untouched); n_tensors >= 0. */
 int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t grad_dtype,
                             rafhip_lans_plan** out_plan);
+
+/*
+ * How a plan cuts and orders its work, for callers that want something else than the measured
+ * defaults (the tests force every code path onto small lists this way).  None of it changes a
+ * result.  Fill the struct with rafhip_lans_default_plan_options first; a field left at its
+ * default value keeps the library's choice.  What the environment sets (RAFHIP_LANS_SCHEDULE,
+ * RAFHIP_LANS_GROUP_ELEMS, RAFHIP_LANS_SPIN_LIMIT) stands between the two: it overrides the
+ * built-in defaults and is overridden by a field set here.
+ */
+typedef struct rafhip_lans_plan_options {
+  int32_t schedule;             /* -1: by list length; RAFHIP_LANS_PHASED / RAFHIP_LANS_PIPELINED        */
+  int32_t round_slices;         /* pipelined: slices per round in which passes B and C alternate; 0: 8  */
+  int64_t group_elements;       /* pipelined: elements per cache group; 0: 13,000,000                   */
+  int64_t stream_from_elements; /* pipelined: tensors from this size bypass the cache; 0: 22,369,621    */
+  int32_t stream_hold_items;    /* pipelined: cached items drawn after a streamed finish; -1: 4 x grid  */
+  int32_t blocks_per_cu;        /* pipelined: resident workgroups per CU; 0: 3, or 2 for long tensors   */
+  int32_t resident_mib;         /* phased: lists up to this size use temporal accesses; -1: 192         */
+  int32_t apply_slice_shift;    /* phased, streaming lists: log2 of the last pass's slice, 0 = whole
+                                   chunks; -1: 10                                                       */
+  int64_t spin_limit;           /* pipelined: polls a wait may take before the step is flagged invalid;
+                                   -1: 2^22 (0 makes every wait give up at once: the tests' way of
+                                   forcing the time-out path while every kernel still exits normally) */
+} rafhip_lans_plan_options;
+void rafhip_lans_default_plan_options(rafhip_lans_plan_options* options);
+/* options may be NULL (= rafhip_lans_plan_create). */
+int rafhip_lans_plan_create_with(int32_t n_tensors, const int64_t* numel, int32_t grad_dtype,
+                                 const rafhip_lans_plan_options* options,
+                                 rafhip_lans_plan** out_plan);
+/* rafhip_lans_pipeline_order with the cutting taken from `options` (group_elements,
+ * round_slices, stream_from_elements, stream_hold_items; NULL = defaults). */
+int rafhip_lans_pipeline_order_with(int32_t n_tensors, const int64_t* numel,
+                                    const rafhip_lans_plan_options* options, int32_t* triples_out,
+                                    int64_t capacity, int64_t* n_items_out);
 int rafhip_lans_plan_destroy(rafhip_lans_plan* plan);
 int rafhip_lans_plan_set_schedule(rafhip_lans_plan* plan, int32_t schedule);
 int32_t rafhip_lans_plan_schedule(const rafhip_lans_plan* plan); /* the schedule in force; -1 on NULL */

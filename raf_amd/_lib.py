@@ -60,6 +60,33 @@ class LansHParams(Structure):
     ]
 
 
+class LansPlanOptions(Structure):
+    """``rafhip_lans_plan_options``; ``defaults()`` gives the struct with every field at "the
+    library's choice"."""
+
+    _fields_ = [
+        ("schedule", c_int32),
+        ("round_slices", c_int32),
+        ("group_elements", c_int64),
+        ("stream_from_elements", c_int64),
+        ("stream_hold_items", c_int32),
+        ("blocks_per_cu", c_int32),
+        ("resident_mib", c_int32),
+        ("apply_slice_shift", c_int32),
+        ("spin_limit", c_int64),
+    ]
+
+    @classmethod
+    def defaults(cls, **fields):
+        o = cls()
+        optim().rafhip_lans_default_plan_options(ctypes.byref(o))
+        for name, value in fields.items():
+            if name not in dict(cls._fields_):
+                raise TypeError(f"no plan option {name!r}")
+            setattr(o, name, int(value))
+        return o
+
+
 # name -> (restype, argtypes); every symbol the header declares.
 OPTIM_SYMBOLS = {
     "rafhip_abi_version": (c_int, []),
@@ -77,6 +104,11 @@ OPTIM_SYMBOLS = {
     "rafhip_lans_query_layout": (c_int, [c_int32, POINTER(c_int64), POINTER(c_int64),
                                          POINTER(c_int64)]),
     "rafhip_lans_plan_create": (c_int, [c_int32, POINTER(c_int64), c_int32, POINTER(c_void_p)]),
+    "rafhip_lans_default_plan_options": (None, [POINTER(LansPlanOptions)]),
+    "rafhip_lans_plan_create_with": (c_int, [c_int32, POINTER(c_int64), c_int32, POINTER(LansPlanOptions),
+                                             POINTER(c_void_p)]),
+    "rafhip_lans_pipeline_order_with": (c_int, [c_int32, POINTER(c_int64), POINTER(LansPlanOptions),
+                                                POINTER(c_int32), c_int64, POINTER(c_int64)]),
     "rafhip_lans_plan_destroy": (c_int, [c_void_p]),
     "rafhip_lans_workspace_bytes": (c_int64, [c_void_p]),
     "rafhip_lans_plan_num_tensors": (c_int32, [c_void_p]),

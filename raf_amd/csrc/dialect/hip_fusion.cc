@@ -565,19 +565,23 @@ Expr FuseLansMixed(const Expr& root) {
     }
     if (!ok) continue;
     // what is taken from the op's result: only w, m, v may be (the fp32 gradients would be gone)
-    std::map<int, Expr> taken;  // field index -> the TupleGetItem
+    // A field may be projected by more than one TupleGetItem node; every one of them is replaced,
+    // or the old call would stay alive beside the new one and update the tensors twice.
+    std::map<int, std::vector<Expr>> taken;  // field index -> its TupleGetItem nodes
     bool only_projections = true;
     for (const ExprNode* user : uses.of(e.get())) {
       const auto* g = ir::AsTupleGetItem(by_ptr.at(user));
       only_projections = only_projections && g != nullptr && g->index >= (int)n && g->index < (int)(4 * n);
-      if (g) taken[g->index] = by_ptr.at(user);
+      if (g) taken[g->index].push_back(by_ptr.at(user));
     }
     if (!only_projections) continue;
-    // the half-precision tails, all or none
+    // the half-precision tails, all or none; a new weight that is projected twice has other users
+    // than its cast, so it has no tail
     std::vector<HalfTail> tails;
     for (size_t i = 0; i < n; ++i) {
       auto it = taken.find((int)(n + i));
-      HalfTail t = it == taken.end() ? HalfTail() : FindHalfTail(it->second, uses, by_ptr);
+      HalfTail t = it == taken.end() || it->second.size() != 1 ? HalfTail()
+                                                              : FindHalfTail(it->second[0], uses, by_ptr);
       if (!t.add || (!tails.empty() && t.bf16 != tails[0].bf16)) break;
       tails.push_back(t);
     }
@@ -596,7 +600,8 @@ Expr FuseLansMixed(const Expr& root) {
     std::vector<Expr> args(lans->args.begin(), lans->args.end());
     args[0] = ir::MakeTuple(fields);
     const Expr call = ir::MakeTupleCall(op, args, TypesOf(fields));
-    for (const auto& kv : taken) replace[kv.second.get()] = ir::MakeTupleGetItem(call, kv.first);
+    for (const auto& kv : taken)
+      for (const Expr& projection : kv.second) replace[projection.get()] = ir::MakeTupleGetItem(call, kv.first);
     if (mixed)
       for (size_t i = 0; i < n; ++i) replace[tails[i].add.get()] = ir::MakeTupleGetItem(call, (int)(4 * n + i));
   }

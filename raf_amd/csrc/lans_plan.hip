@@ -72,23 +72,8 @@ constexpr int64_t kResidentBytes = 192LL << 20;
 constexpr int64_t kLongTensorElems = 6 * 1000 * 1000;
 
 // Slices per round in which passes B and C alternate (measured on MI355X: 4 to 16 are within
-// 0.1 % of each other on the BERT-large list, 1 is 3 % slower).  RAFHIP_LANS_ROUND_SLICES overrides.
+// 0.1 % of each other on the BERT-large list, 1 is 3 % slower).
 constexpr int kDefaultRoundSlices = 8;
-int round_slices_setting() {
-  if (const char* e = std::getenv("RAFHIP_LANS_ROUND_SLICES")) {
-    const int v = std::atoi(e);
-    if (v >= 1 && v <= 4096) return v;
-  }
-  return kDefaultRoundSlices;
-}
-
-int env_count(const char* name, int fallback) {
-  if (const char* e = std::getenv(name)) {
-    const int v = std::atoi(e);
-    if (v >= 0) return v;
-  }
-  return fallback;
-}
 
 inline WorkItem make_item(int32_t tensor, uint32_t phase, int64_t chunk, uint32_t flags = 0) {
   return WorkItem{tensor, (phase << kPhaseShift) | flags | (uint32_t)chunk};
@@ -97,13 +82,6 @@ inline WorkItem make_item(int32_t tensor, uint32_t phase, int64_t chunk, uint32_
 // A tensor whose w, m, v alone exceed the 256 MB Infinity Cache cannot keep anything there between
 // its passes; handled like the others it would only flush the groups that can.
 constexpr int64_t kStreamedTensorFromElems = (256LL << 20) / 12;
-int64_t streamed_from_setting() {
-  if (const char* e = std::getenv("RAFHIP_LANS_STREAM_FROM_ELEMS")) {
-    const long long v = std::atoll(e);
-    if (v > 0) return v;
-  }
-  return kStreamedTensorFromElems;
-}
 
 // Resident workgroups of the persistent kernel on a 256-CU device, for the host-only queries.
 constexpr int kDefaultPipelineGrid = 256 * 3;
@@ -125,22 +103,29 @@ constexpr int kDefaultPipelineGrid = 256 * 3;
 //
 // Invariant the kernel's waits rely on, per tensor: pass-A units, then its finish-A item, then
 // pass-B chunks, then its finish-B item, then pass-C chunks.
-std::vector<WorkItem> build_pipeline(int32_t n, const int64_t* numel, int64_t group_elems,
+struct PipelineCut {
+  int64_t group_elems;
+  int64_t stream_from;  // tensors from this many elements on are streamed
+  int round_slices;
+  int hold_items;       // < 0: 4 x grid
+};
+
+std::vector<WorkItem> build_pipeline(int32_t n, const int64_t* numel, const PipelineCut& cut,
                                      int grid = kDefaultPipelineGrid) {
+  const int64_t group_elems = cut.group_elems;
   struct Group {
     std::vector<WorkItem> a, b, c;
   };
   std::vector<Group> groups;
   std::vector<WorkItem> streamed;  // every streamed tensor: A units, finish A, B chunks, finish B, C chunks
   std::vector<int64_t> streamed_bytes;  // what each of those items moves (for the proportional merge)
-  const bool stream_large = std::getenv("RAFHIP_LANS_NO_STREAMED_TENSORS") == nullptr;
-  const int64_t stream_from = streamed_from_setting();
+  const int64_t stream_from = cut.stream_from;
   std::vector<int32_t> cached_tensors;
   for (int32_t t = 0; t < n; ++t) {
     if (numel[t] == 0) continue;
     const int64_t nc = chunks_of(numel[t]);
     const int64_t ce = chunk_elems_for(numel[t]);
-    if (stream_large && numel[t] >= stream_from) {
+    if (numel[t] >= stream_from) {
       auto len_of = [&](int64_t idx, int64_t unit) { return std::min(unit, numel[t] - idx * unit); };
       for (int64_t u = 0; u < units_a_of(numel[t]); ++u) {
         streamed.push_back(make_item(t, kPhaseA, u, kStreamBit));
@@ -193,7 +178,7 @@ std::vector<WorkItem> build_pipeline(int32_t n, const int64_t* numel, int64_t gr
   // survive in the cache (3 % on the BERT-large list; a dependency never crosses: the C items of
   // a round belong to an earlier group than its B items).
   static const std::vector<WorkItem> none;
-  const size_t slices = (size_t)round_slices_setting();
+  const size_t slices = (size_t)cut.round_slices;
   for (int64_t r = 0; r < ng + 2; ++r) {
     const std::vector<WorkItem>& b = (r >= 1 && r - 1 < ng) ? groups[r - 1].b : none;
     const std::vector<WorkItem>& c = (r >= 2 && r - 2 < ng) ? groups[r - 2].c : none;
@@ -223,7 +208,7 @@ std::vector<WorkItem> build_pipeline(int32_t n, const int64_t* numel, int64_t gr
         default: return 0;
       }
     };
-    const int hold_items = env_count("RAFHIP_LANS_STREAM_HOLD_ITEMS", 4 * grid);
+    const int hold_items = cut.hold_items >= 0 ? cut.hold_items : 4 * grid;
     double total_c = 0, total_s = 0;
     for (const WorkItem& it : cached) total_c += (double)bytes_of(it);
     for (int64_t b : streamed_bytes) total_s += (double)b;
@@ -263,31 +248,52 @@ std::vector<WorkItem> build_pipeline(int32_t n, const int64_t* numel, int64_t gr
   return out;
 }
 
-int64_t group_elems_setting() {
+// The settings in force for a plan: the built-in defaults, overridden by the three user-facing
+// environment variables, overridden by what the caller set in rafhip_lans_plan_options.
+struct ResolvedOptions {
+  int schedule;  // -1: by list length
+  PipelineCut cut;
+  int blocks_per_cu;  // 0: by the list
+  int64_t resident_bytes;
+  int apply_slice_shift;
+  uint32_t spin_limit;
+};
+
+ResolvedOptions resolve_options(const rafhip_lans_plan_options* o) {
+  ResolvedOptions r;
+  r.schedule = -1;
+  r.cut = PipelineCut{kDefaultGroupElems, kStreamedTensorFromElems, kDefaultRoundSlices, -1};
+  r.blocks_per_cu = 0;
+  r.resident_bytes = kResidentBytes;
+  r.apply_slice_shift = 10;
+  // Polls a wait of the pipelined kernel may take before it gives up and raises the error word:
+  // with a sleep of a few hundred cycles per poll the default is seconds, far beyond any real
+  // dependency latency.
+  r.spin_limit = 1u << 22;
+  if (const char* e = std::getenv("RAFHIP_LANS_SCHEDULE")) {
+    if (!std::strcmp(e, "phased")) r.schedule = RAFHIP_LANS_PHASED;
+    if (!std::strcmp(e, "pipelined")) r.schedule = RAFHIP_LANS_PIPELINED;
+  }
   if (const char* e = std::getenv("RAFHIP_LANS_GROUP_ELEMS")) {
     const long long v = std::atoll(e);
-    if (v > 0) return v;
+    if (v > 0) r.cut.group_elems = v;
   }
-  return kDefaultGroupElems;
-}
-
-// Polls a wait of the pipelined kernel may take before it gives up and raises the error word:
-// with a sleep of a few hundred cycles per poll the default is seconds, far beyond any real
-// dependency latency.  RAFHIP_LANS_SPIN_LIMIT overrides it (tests force a time-out with 0).
-uint32_t spin_limit_setting() {
   if (const char* e = std::getenv("RAFHIP_LANS_SPIN_LIMIT")) {
     const long long v = std::atoll(e);
-    if (v >= 0 && v <= 0xFFFFFFFFll) return (uint32_t)v;
+    if (v >= 0 && v <= 0xFFFFFFFFll) r.spin_limit = (uint32_t)v;
   }
-  return 1u << 22;
-}
-
-int schedule_setting(int64_t total_elements) {
-  if (const char* e = std::getenv("RAFHIP_LANS_SCHEDULE")) {
-    if (!std::strcmp(e, "phased")) return RAFHIP_LANS_PHASED;
-    if (!std::strcmp(e, "pipelined")) return RAFHIP_LANS_PIPELINED;
-  }
-  return total_elements >= kPipelinedFromElems ? RAFHIP_LANS_PIPELINED : RAFHIP_LANS_PHASED;
+  if (!o) return r;
+  if (o->schedule == RAFHIP_LANS_PHASED || o->schedule == RAFHIP_LANS_PIPELINED) r.schedule = o->schedule;
+  if (o->group_elements > 0) r.cut.group_elems = o->group_elements;
+  if (o->round_slices > 0) r.cut.round_slices = o->round_slices < 4096 ? o->round_slices : 4096;
+  if (o->stream_from_elements > 0) r.cut.stream_from = o->stream_from_elements;
+  if (o->stream_hold_items >= 0) r.cut.hold_items = o->stream_hold_items;
+  if (o->blocks_per_cu > 0) r.blocks_per_cu = o->blocks_per_cu;
+  if (o->resident_mib >= 0) r.resident_bytes = (int64_t)o->resident_mib << 20;
+  if (o->apply_slice_shift == 0 || (o->apply_slice_shift >= 10 && o->apply_slice_shift < kChunkShift))
+    r.apply_slice_shift = o->apply_slice_shift;
+  if (o->spin_limit >= 0 && o->spin_limit <= 0xFFFFFFFFll) r.spin_limit = (uint32_t)o->spin_limit;
+  return r;
 }
 
 // The address of `scratch` on a device, resolved once per device with that device current.
@@ -446,19 +452,33 @@ int rafhip_lans_query_layout(int32_t n_tensors, const int64_t* numel, int64_t* n
   return RAFHIP_OK;
 }
 
-int rafhip_lans_pipeline_order(int32_t n_tensors, const int64_t* numel, int64_t group_elements,
-                               int32_t* triples_out, int64_t capacity, int64_t* n_items_out) {
+void rafhip_lans_default_plan_options(rafhip_lans_plan_options* o) {
+  if (!o) return;
+  o->schedule = -1;
+  o->round_slices = 0;
+  o->group_elements = 0;
+  o->stream_from_elements = 0;
+  o->stream_hold_items = -1;
+  o->blocks_per_cu = 0;
+  o->resident_mib = -1;
+  o->apply_slice_shift = -1;
+  o->spin_limit = -1;
+}
+
+int rafhip_lans_pipeline_order_with(int32_t n_tensors, const int64_t* numel,
+                                    const rafhip_lans_plan_options* options, int32_t* triples_out,
+                                    int64_t capacity, int64_t* n_items_out) {
   clear_error();
-  if (int st = validate_list("rafhip_lans_pipeline_order", n_tensors, numel)) return st;
-  if (!n_items_out) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_pipeline_order: n_items_out is NULL");
-  return guarded("rafhip_lans_pipeline_order", [&]() -> int {
-    const std::vector<WorkItem> items =
-        build_pipeline(n_tensors, numel, group_elements > 0 ? group_elements : kDefaultGroupElems);
+  const char* who = "rafhip_lans_pipeline_order";
+  if (int st = validate_list(who, n_tensors, numel)) return st;
+  if (!n_items_out) return fail(RAFHIP_ERR_INVALID_ARG, "%s: n_items_out is NULL", who);
+  return guarded(who, [&]() -> int {
+    const std::vector<WorkItem> items = build_pipeline(n_tensors, numel, resolve_options(options).cut);
     *n_items_out = (int64_t)items.size();
     if (triples_out) {
       if (capacity < (int64_t)items.size())
-        return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_pipeline_order: capacity %lld < %zu items",
-                    (long long)capacity, items.size());
+        return fail(RAFHIP_ERR_INVALID_ARG, "%s: capacity %lld < %zu items", who, (long long)capacity,
+                    items.size());
       for (size_t i = 0; i < items.size(); ++i) {
         const uint32_t cp = items[i].chunk_phase;
         triples_out[3 * i + 0] = (int32_t)(cp >> kPhaseShift) + ((cp & kStreamBit) ? 8 : 0);
@@ -470,8 +490,22 @@ int rafhip_lans_pipeline_order(int32_t n_tensors, const int64_t* numel, int64_t 
   });
 }
 
+int rafhip_lans_pipeline_order(int32_t n_tensors, const int64_t* numel, int64_t group_elements,
+                               int32_t* triples_out, int64_t capacity, int64_t* n_items_out) {
+  rafhip_lans_plan_options o;
+  rafhip_lans_default_plan_options(&o);
+  o.group_elements = group_elements > 0 ? group_elements : kDefaultGroupElems;
+  return rafhip_lans_pipeline_order_with(n_tensors, numel, &o, triples_out, capacity, n_items_out);
+}
+
 int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t grad_dtype,
                             rafhip_lans_plan** out_plan) {
+  return rafhip_lans_plan_create_with(n_tensors, numel, grad_dtype, nullptr, out_plan);
+}
+
+int rafhip_lans_plan_create_with(int32_t n_tensors, const int64_t* numel, int32_t grad_dtype,
+                                 const rafhip_lans_plan_options* options,
+                                 rafhip_lans_plan** out_plan) {
   clear_error();
   if (!out_plan) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_lans_plan_create: out_plan is NULL");
   *out_plan = nullptr;
@@ -495,15 +529,15 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
       longest = std::max(longest, chunks_of(numel[t]));
       total += numel[t];
     }
+    const ResolvedOptions opt = resolve_options(options);
     p->short_tensors_only = longest <= kInlineFinishChunks;
-    p->resident_bytes = (int64_t)env_count("RAFHIP_LANS_RESIDENT_MIB", (int)(kResidentBytes >> 20)) << 20;
-    p->apply_slice_shift = env_count("RAFHIP_LANS_APPLY_SLICE_SHIFT", 10);
-    if (p->apply_slice_shift != 0 && (p->apply_slice_shift < 10 || p->apply_slice_shift >= kChunkShift))
-      p->apply_slice_shift = 0;
+    p->resident_bytes = opt.resident_bytes;
+    p->apply_slice_shift = opt.apply_slice_shift;
     p->n_chunks = chunks;
     p->total_elements = total;
-    p->schedule = schedule_setting(total);
-    p->spin_limit = spin_limit_setting();
+    p->schedule = opt.schedule >= 0 ? opt.schedule
+                                    : (total >= kPipelinedFromElems ? RAFHIP_LANS_PIPELINED : RAFHIP_LANS_PHASED);
+    p->spin_limit = opt.spin_limit;
     p->ws = make_layout(n_tensors, chunks);
 
     if (hipGetDevice(&p->device) != hipSuccess) {
@@ -531,20 +565,17 @@ int rafhip_lans_plan_create(int32_t n_tensors, const int64_t* numel, int32_t gra
       // default three; a larger window of in-flight items measured slower on MI355X (it crowds the
       // Infinity Cache).  Lists whose bulk is in long tensors (GPT-2's 8-10 M element matrices)
       // measured 3 % faster with two, lists of shorter tensors (BERT: up to 4 M) 1-2 % slower.
-      // RAFHIP_LANS_BLOCKS_PER_CU overrides the choice downwards or up to the fit.
+      // rafhip_lans_plan_options.blocks_per_cu overrides the choice downwards or up to the fit.
       const int fit = pipelined_blocks_per_cu(grad_dtype);
       int64_t in_long_tensors = 0;
       for (int32_t t = 0; t < n_tensors; ++t)
         if (numel[t] >= kLongTensorElems) in_long_tensors += numel[t];
       const int wanted = 2 * in_long_tensors > total ? 2 : 3;
       int per_cu = fit > 0 ? (fit < wanted ? fit : wanted) : 2;
-      if (const char* e = std::getenv("RAFHIP_LANS_BLOCKS_PER_CU")) {
-        const int want = std::atoi(e);
-        if (want > 0) per_cu = (fit > 0 && want > fit) ? fit : want;
-      }
+      if (opt.blocks_per_cu > 0) per_cu = (fit > 0 && opt.blocks_per_cu > fit) ? fit : opt.blocks_per_cu;
       p->pipeline_grid = (unsigned)(p->n_cus * per_cu);
       const std::vector<WorkItem> pipeline =
-          build_pipeline(n_tensors, numel, group_elems_setting(), (int)p->pipeline_grid);
+          build_pipeline(n_tensors, numel, opt.cut, (int)p->pipeline_grid);
       p->n_pipeline_items = (uint32_t)pipeline.size();
       if (p->pipeline_grid > p->n_pipeline_items) p->pipeline_grid = p->n_pipeline_items;
 

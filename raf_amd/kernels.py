@@ -49,7 +49,10 @@ _DTYPE_CODE = {torch.float32: RAFHIP_F32, torch.float16: RAFHIP_F16, torch.bfloa
 class SgdPlan:
     """Owns a ``rafhip_sgd_plan``: momentum SGD over a whole parameter list, in place, one launch."""
 
-    def __init__(self, numels: Sequence[int], grad_dtype=torch.float32, device="cuda:0"):
+    def __init__(self, numels: Sequence[int], grad_dtype=torch.float32, device="cuda:0", **options):
+        """``options``: fields of ``rafhip_lans_plan_options`` (``schedule``, ``group_elements``,
+        ``round_slices``, ``blocks_per_cu``, ``stream_from_elements``, ``stream_hold_items``,
+        ``resident_mib``, ``apply_slice_shift``, ``spin_limit``); none changes a result."""
         self._h = c_void_p(None)
         self.lib = _lib.optim()
         self.device = torch.device(device)
@@ -202,22 +205,35 @@ def query_layout(numels: Sequence[int]):
     return chunks.value, ws.value
 
 
-def pipeline_order(numels: Sequence[int], group_elements: int = 0):
-    """[(pass, tensor, chunk)] in the order the pipelined schedule hands out work; host arithmetic."""
+def pipeline_order(numels: Sequence[int], group_elements: int = 0, **options):
+    """[(pass, tensor, chunk)] in the order the pipelined schedule hands out work; host arithmetic.
+    ``options``: fields of ``rafhip_lans_plan_options`` that cut the list (``round_slices``,
+    ``stream_from_elements``, ``stream_hold_items``)."""
     n = len(numels)
     arr = (c_int64 * max(n, 1))(*numels)
     count = c_int64(0)
     lib = _lib.optim()
-    check(lib.rafhip_lans_pipeline_order(n, arr, group_elements, None, 0, ctypes.byref(count)))
+    if not options:
+        order = lambda buf, cap: lib.rafhip_lans_pipeline_order(n, arr, group_elements, buf, cap, ctypes.byref(count))
+    else:
+        o = _lib.LansPlanOptions.defaults(**options)
+        if group_elements > 0:
+            o.group_elements = group_elements
+        order = lambda buf, cap: lib.rafhip_lans_pipeline_order_with(n, arr, ctypes.byref(o), buf, cap,
+                                                                     ctypes.byref(count))
+    check(order(None, 0))
     buf = (ctypes.c_int32 * max(3 * count.value, 1))()
-    check(lib.rafhip_lans_pipeline_order(n, arr, group_elements, buf, count.value, ctypes.byref(count)))
+    check(order(buf, count.value))
     return [(buf[3 * i], buf[3 * i + 1], buf[3 * i + 2]) for i in range(count.value)]
 
 
 class LansPlan:
     """Owns a ``rafhip_lans_plan`` and a workspace tensor sized for it."""
 
-    def __init__(self, numels: Sequence[int], grad_dtype=torch.float32, device="cuda:0"):
+    def __init__(self, numels: Sequence[int], grad_dtype=torch.float32, device="cuda:0", **options):
+        """``options``: fields of ``rafhip_lans_plan_options`` (``schedule``, ``group_elements``,
+        ``round_slices``, ``blocks_per_cu``, ``stream_from_elements``, ``stream_hold_items``,
+        ``resident_mib``, ``apply_slice_shift``, ``spin_limit``); none changes a result."""
         self._h = c_void_p(None)
         self.lib = _lib.optim()
         self.device = torch.device(device)
@@ -229,7 +245,11 @@ class LansPlan:
         self.grad_dtype = grad_dtype
         arr = (c_int64 * max(self.n, 1))(*self.numels)
         with torch.cuda.device(self.device):
-            check(self.lib.rafhip_lans_plan_create(self.n, arr, code, ctypes.byref(self._h)))
+            if options:
+                o = _lib.LansPlanOptions.defaults(**options)
+                check(self.lib.rafhip_lans_plan_create_with(self.n, arr, code, ctypes.byref(o), ctypes.byref(self._h)))
+            else:
+                check(self.lib.rafhip_lans_plan_create(self.n, arr, code, ctypes.byref(self._h)))
         self.workspace_bytes = self.lib.rafhip_lans_workspace_bytes(self._h)
         self.n_chunks = self.lib.rafhip_lans_plan_num_chunks(self._h)
         self.total_elements = self.lib.rafhip_lans_plan_total_elements(self._h)

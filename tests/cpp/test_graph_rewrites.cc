@@ -285,6 +285,35 @@ int main() {
            Contains(AsText(got), "raf.op.cast"));
   }
 
+  std::puts("LANS: a result field projected by two TupleGetItem nodes: both move to the new call");
+  {
+    Params q = MakeParams(shapes, 16, kDLFloat, kDLFloat);
+    Expr step = MakeVar("step", Ty({})), zero = MakeZeros(Ty({}, 16));
+    Expr traced = hip::TracedLansOptimizer(q.g, q.w, q.m, q.v, q.p, zero, step, hyper);
+    Expr lans_call;
+    for (const Expr& e : PostOrder(traced))
+      if (AsCall(e) && AsOp(AsCall(e)->op) && AsOp(AsCall(e)->op)->name == "raf.op.lans") lans_call = e;
+    // a second, separate projection of the first moment of parameter 0 and of the new weight of
+    // parameter 1 (which thereby has a user besides its cast: no 16-bit tails are folded in)
+    std::vector<Expr> fields = AsTupleNode(traced)->fields;
+    fields.push_back(MakeTupleGetItem(lans_call, (int)(2 * n)));
+    Expr twice_m = MakeTuple(fields);
+    Expr got = pass::FuseDialect(twice_m, DevType::kROCM());
+    std::string text = AsText(got);
+    EXPECT(Contains(text, "raf.op.hip.lans_mixed") && !Contains(text, "raf.op.lans(") && !Contains(text, "group_cast"));
+    fields.push_back(MakeTupleGetItem(lans_call, (int)(n + 1)));
+    Expr twice_w = MakeTuple(fields);
+    got = pass::FuseDialect(twice_w, DevType::kROCM());
+    text = AsText(got);
+    EXPECT(Contains(text, "raf.op.hip.lans(") && !Contains(text, "lans_mixed") && !Contains(text, "raf.op.lans(") &&
+           !Contains(text, "group_cast") && Contains(text, "raf.op.cast"));
+    // every call of the rewritten graph is reached through the ONE new call
+    size_t calls = 0;
+    for (const Expr& e : PostOrder(got))
+      if (AsCall(e) && AsOp(AsCall(e)->op) && AsOp(AsCall(e)->op)->name == "raf.op.hip.lans") ++calls;
+    EXPECT(calls == 1);
+  }
+
   std::puts("ALL OK");
   return 0;
 }

@@ -255,6 +255,12 @@ def test_default_schedule_follows_list_length(native_libs, monkeypatch):
     plan = kernels.LansPlan([1000, 5], torch.float32, DEV)
     assert plan.schedule == "pipelined"
     plan.close()
+    # a plan option beats the environment, which beats the built-in choice
+    plan = kernels.LansPlan([1000, 5], torch.float32, DEV, schedule=native_libs.RAFHIP_LANS_PHASED)
+    assert plan.schedule == "phased"
+    plan.close()
+    with pytest.raises(TypeError, match="no plan option"):
+        kernels.LansPlan([8], torch.float32, DEV, chunk=3)
 
 
 @pytest.mark.parametrize("group_elems", [None, 1 << 20])
@@ -308,11 +314,11 @@ def test_sliced_last_pass_of_streaming_lists_is_bitwise_equal(native_libs, monke
              (1 << 20) + 1029, 12345]
     g, w, m, v = lans_inputs(sizes, cfg=81, g16=True)
     hp = LansHParams(grad_unscale=1 / 1024)
-    monkeypatch.setenv("RAFHIP_LANS_RESIDENT_MIB", "0")
     results = {}
     for variant in ("pipelined", "0", "10", "11", "12"):
+        options = {"resident_mib": 0}  # treat even these short lists as far larger than the cache
         if variant != "pipelined":
-            monkeypatch.setenv("RAFHIP_LANS_APPLY_SLICE_SHIFT", variant)
+            options["apply_slice_shift"] = int(variant)
         tg, tw, tm, tv = _to_dev(g), _to_dev(w), _to_dev(m), _to_dev(v)
         # every third tensor starts 4 bytes off a 16-byte boundary
         backing = [torch.zeros(n + 1, device=DEV) for n in sizes]
@@ -321,7 +327,7 @@ def test_sliced_last_pass_of_streaming_lists_is_bitwise_equal(native_libs, monke
             off.copy_(tw[i])
             tw[i] = off
         tp = [torch.zeros(n, dtype=torch.float16, device=DEV) for n in sizes] if copy16 else None
-        plan = kernels.LansPlan(sizes, tg[0].dtype, DEV)
+        plan = kernels.LansPlan(sizes, tg[0].dtype, DEV, **options)
         plan.set_schedule("pipelined" if variant == "pipelined" else "phased")
         for step in (1, 2):
             plan.step(tg, tw, tm, tv, step, _khp(hp), p=tp)
@@ -357,16 +363,18 @@ def test_random_lists_groupings_and_slicings_agree_bitwise(native_libs, monkeypa
         hp_case = LansHParams(grad_unscale=(1 / 1024 if case % 2 else 1.0), mode=int(case % 3 == 0))
         outs = []
         for schedule in ("phased", "pipelined"):
+            options = {}
             if schedule == "pipelined":
-                monkeypatch.setenv("RAFHIP_LANS_GROUP_ELEMS", str(int(rng.choice([1, 50_000, 400_000, 3_000_000]))))
-                monkeypatch.setenv("RAFHIP_LANS_ROUND_SLICES", str(int(rng.choice([1, 2, 8, 64, 4096]))))
-                monkeypatch.setenv("RAFHIP_LANS_BLOCKS_PER_CU", str(int(rng.choice([1, 2, 3]))))
-                # tensors from this size on are treated as too large for the cache: their items are
-                # marked streaming and merged into the list of the cached groups
-                monkeypatch.setenv("RAFHIP_LANS_STREAM_FROM_ELEMS", str(int(rng.choice([50_000, 600_000, 10**9]))))
-                monkeypatch.setenv("RAFHIP_LANS_STREAM_HOLD_ITEMS", str(int(rng.choice([0, 7, 3072]))))
+                options = dict(
+                    group_elements=int(rng.choice([1, 50_000, 400_000, 3_000_000])),
+                    round_slices=int(rng.choice([1, 2, 8, 64, 4096])),
+                    blocks_per_cu=int(rng.choice([1, 2, 3])),
+                    # tensors from this size on are treated as too large for the cache: their items
+                    # are marked streaming and merged into the list of the cached groups
+                    stream_from_elements=int(rng.choice([50_000, 600_000, 10**9])),
+                    stream_hold_items=int(rng.choice([0, 7, 3072])))
             tg, tw, tm, tv = _to_dev(g), _to_dev(w), _to_dev(m), _to_dev(v)
-            plan = kernels.LansPlan(sizes, tg[0].dtype, DEV)
+            plan = kernels.LansPlan(sizes, tg[0].dtype, DEV, **options)
             plan.set_schedule(schedule)
             for step in (1, 2):
                 plan.step(tg, tw, tm, tv, step, _khp(hp_case))

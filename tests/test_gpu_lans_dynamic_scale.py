@@ -178,3 +178,41 @@ def test_two_models_of_one_architecture_share_an_op_env(native_libs):
             assert max_rel_err(tl[n + t].cpu().numpy(), ow[t]) <= 1e-5
             assert max_rel_err(tl[3 * n + t].cpu().numpy(), ov[t]) <= 1e-5
     op.clear_op_env_cache()
+
+
+def test_optimizer_class_does_not_count_a_skipped_step(native_libs):
+    """raf_amd.optim.LANS under dynamic loss scaling: a step that the kernels skipped because of an
+    overflow leaves w, m, v alone AND leaves the device-resident step counter where it was, so the
+    bias corrections of the next applied step are those of step 2, not 3 (the oracle's
+    lans_step_dynamic_scale with the count of applied steps)."""
+    from raf_amd import op, optim
+
+    sizes = [70_001, 9, 4096]
+    hp = LansHParams()
+    g, w, _, _ = lans_inputs(sizes, cfg=74)
+    params = [torch.nn.Parameter(t) for t in _to_dev(w)]
+    for p, gt in zip(params, _to_dev(g)):
+        p.grad = gt
+    inv_scale = torch.ones((), device=DEV)
+    found_inf = torch.zeros((), device=DEV)
+    op.clear_op_env_cache()
+    op.set_lans_dynamic_scale(inv_scale, found_inf)
+    try:
+        opt = optim.LANS(params)
+        zeros = [np.zeros_like(a) for a in w]
+        opt.step()                       # applied as step 1
+        ow, om, ov, _ = lans_f64.lans_step_dynamic_scale(g, w, zeros, zeros, 1, hp, 1.0, 0.0)
+        found_inf.fill_(1.0)
+        opt.step()                       # skipped: nothing moves, nothing is counted
+        found_inf.zero_()
+        opt.step()                       # applied as step 2
+        ow, om, ov, _ = lans_f64.lans_step_dynamic_scale(g, ow, om, ov, 2, hp, 1.0, 0.0)
+        torch.cuda.synchronize()
+        assert float(opt._step_dev) == 3.0 and opt._step == 4  # applied steps + 1; calls + 1
+        for t in range(len(sizes)):
+            assert max_rel_err(params[t].data.cpu().numpy(), ow[t]) <= 1e-5
+            assert max_rel_err(opt.params[t][2].cpu().numpy(), om[t]) <= 1e-5
+            assert max_rel_err(opt.params[t][3].cpu().numpy(), ov[t]) <= 1e-5
+    finally:
+        op.set_lans_dynamic_scale(None, None)
+        op.clear_op_env_cache()

@@ -275,7 +275,7 @@ def test_fuse_and_defuse_on_a_requested_copy_stream(native_libs):
             for k, t in enumerate(parts):  # producers on the current stream, right before the op
                 t.fill_(float(10 * rep + k))
             flat = op.fuse_tensor(parts)
-            total = flat.sum()  # a consumer on the current stream, right after the op
+            total = flat.double().sum()  # a consumer on the current stream, right after the op
             want = sum(float(10 * rep + k) * t.numel() for k, t in enumerate(parts))
             assert float(total) == want
             flat.mul_(2.0)

@@ -105,10 +105,10 @@ def test_order_invariants_on_random_lists(native_libs, monkeypatch):
                 sizes.append(int(rng.integers(22_400_000, 60_000_000)))  # streamed
         group = int(rng.choice([0, 1, 50_000, 3_000_000, 13_000_000, 10**12]))
         stream_from = int(rng.choice([(256 << 20) // 12, 30_000, 1_000_000, 10**12]))
-        monkeypatch.setenv("RAFHIP_LANS_STREAM_FROM_ELEMS", str(stream_from))
-        monkeypatch.setenv("RAFHIP_LANS_STREAM_HOLD_ITEMS", str(int(rng.choice([0, 3, 3072, 10**6]))))
+        hold = int(rng.choice([0, 3, 3072, 10**6]))
         try:
-            _check(kernels.pipeline_order(sizes, group), sizes, lib, stream_from)
+            _check(kernels.pipeline_order(sizes, group, stream_from_elements=stream_from, stream_hold_items=hold),
+                   sizes, lib, stream_from)
         except AssertionError as e:
             raise AssertionError(f"case {case}: sizes {sizes}, group {group}: {e}") from e
 
