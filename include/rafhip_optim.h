@@ -74,6 +74,19 @@ int rafhip_sgd_f32(const float* x, const float* dx, const float* v, float* v_out
                    int64_t n, double learning_rate, double mu, void* stream);
 
 /*
+ * The same step in the element type of x, which is how the reference writes the compute
+ * (tir.const(value, dtype=x0.dtype), python/raf/_tvm_op/sgd.py:18-19): dtype RAFHIP_F32 (the call
+ * above), RAFHIP_F64, RAFHIP_F16 or RAFHIP_BF16; x, dx, v and both outputs share it.  mu and
+ * learning_rate are rounded once to the element type; each of the four operations is rounded to
+ * the element type on its own -- for the 16-bit types by widening to fp32, operating there and
+ * rounding the result back, which is what a CPU without half arithmetic does (the reference's CPU
+ * target is bare `llvm`) and gives the correctly rounded 16-bit result.  No test of the reference
+ * pins the 16-bit or fp64 bits.
+ */
+int rafhip_sgd(const void* x, const void* dx, const void* v, void* v_out, void* x_out, int64_t n,
+               int32_t dtype, double learning_rate, double mu, void* stream);
+
+/*
  * Multi-tensor momentum SGD, IN PLACE on x and v, one launch for a whole parameter list.  Per
  * element exactly the four roundings above.  It replaces, per step, the op sequence the reference's
  * traced optimizer emits for EVERY parameter -- cast(dx, fp32), multiply, add(out=v), multiply,

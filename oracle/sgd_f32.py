@@ -49,6 +49,61 @@ def sgd_step(x0, dx, v0, learning_rate: float, mu: float):
     return v1, x1
 
 
+def sgd_step_typed(x0, dx, v0, learning_rate: float, mu: float, dtype: str):
+    """The same step in another element type, which is how the reference's compute is written
+    (``tir.const(value, dtype=x0.dtype)``, sgd.py:18-19): ``"float64"``, ``"float16"`` or
+    ``"bfloat16"`` (arrays of uint16 bit patterns).  The constants are rounded once from double to
+    the element type and each of the four operations is rounded to the element type on its own;
+    for the 16-bit types through fp32 (widen, operate, round back), as a CPU without half
+    arithmetic evaluates them -- with 24 >= 2p + 2 bits in between that equals the correctly
+    rounded 16-bit operation.  **Parity unpinned by the reference**: its tests run the op in fp32
+    only; pinned here against exact rational arithmetic (tests/test_oracle_sgd.py)."""
+    from oracle.halfs import bf16_bits_to_f32, f32_to_bf16_bits
+
+    if dtype == "float64":
+        x0, dx, v0 = (np.asarray(a, dtype=np.float64) for a in (x0, dx, v0))
+        with np.errstate(all="ignore"):
+            v1 = np.float64(mu) * v0 + dx
+            x1 = x0 - np.float64(learning_rate) * v1
+        return v1, x1
+    if dtype == "float16":
+        x0, dx, v0 = (np.asarray(a, dtype=np.float16) for a in (x0, dx, v0))
+        op = lambda f, a, b: f(a.astype(np.float32), b.astype(np.float32), dtype=np.float32).astype(np.float16)
+        lr, m = np.float16(learning_rate), np.float16(mu)  # double -> half, one rounding
+        with np.errstate(all="ignore"):
+            v1 = op(np.add, op(np.multiply, np.full_like(v0, m), v0), dx)
+            x1 = op(np.subtract, x0, op(np.multiply, np.full_like(v1, lr), v1))
+        return v1, x1
+    if dtype == "bfloat16":
+        x0, dx, v0 = (np.asarray(a, dtype=np.uint16) for a in (x0, dx, v0))
+        op = lambda f, a, b: f32_to_bf16_bits(f(bf16_bits_to_f32(a), bf16_bits_to_f32(b), dtype=np.float32))
+        lr, m = bf16_from_double(learning_rate), bf16_from_double(mu)
+        with np.errstate(all="ignore"):
+            v1 = op(np.add, op(np.multiply, np.full_like(v0, m), v0), dx)
+            x1 = op(np.subtract, x0, op(np.multiply, np.full_like(v1, lr), v1))
+        return v1, x1
+    raise TypeError(f"dtype {dtype!r}: expected 'float64', 'float16' or 'bfloat16'")
+
+
+def bf16_from_double(x: float) -> np.uint16:
+    """double -> bfloat16 bit pattern with ONE rounding to nearest even (going through fp32 first
+    could round twice): the two neighbouring bfloat16 values are compared exactly."""
+    from fractions import Fraction
+
+    from oracle.halfs import bf16_bits_to_f32
+
+    lo = int(np.asarray(np.float32(x)).view(np.uint32)) & 0xFFFF0000
+    # candidates around the fp32 neighbour: one step of the bfloat16 grid either side
+    best = None
+    for bits in (lo - 0x10000, lo, lo + 0x10000):
+        value = Fraction(float(bf16_bits_to_f32(np.uint16((bits >> 16) & 0xFFFF))))
+        err = abs(value - Fraction(x))
+        key = (err, (bits >> 16) & 1)  # nearest; ties to the even pattern
+        if best is None or key < best[0]:
+            best = (key, bits)
+    return np.uint16((best[1] >> 16) & 0xFFFF)
+
+
 def sgd_list_step(x_list, dx_list, v_list, learning_rate: float, mu: float, model_dtype=None):
     """What the reference's traced optimizer computes per parameter (python/raf/optim/
     sgd.py:187-215): ``dx`` widened to fp32 (``cast(dxi, "float32")``, exact), then

@@ -94,6 +94,8 @@ OPTIM_SYMBOLS = {
     "rafhip_device_count": (c_int, []),
     "rafhip_sgd_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_double,
                                c_double, c_void_p]),
+    "rafhip_sgd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_double,
+                           c_double, c_void_p]),
     "rafhip_lans_default_hparams": (None, [POINTER(LansHParams)]),
     "rafhip_lans_chunk_elements": (c_int32, [c_int64]),
     "rafhip_lans_pass_a_unit_elements": (c_int32, [c_int64]),

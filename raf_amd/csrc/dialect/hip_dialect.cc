@@ -81,8 +81,13 @@ class SgdHipEnv : public OpEnv, public HasLearningRate {
     const TensorView& x = args->x->tensor;
     if (cv->device.device_type() != DevType::kROCM())
       error_msgs.push_back("raf.op.hip.sgd: device is not rocm");
-    if (!IsF32(x.dtype) || !IsF32(args->dx->tensor.dtype) || !IsF32(args->v->tensor.dtype))
-      error_msgs.push_back("raf.op.hip.sgd: only float32 tensors are supported");
+    // The reference's compute is written in x's dtype (python/raf/_tvm_op/sgd.py:18-19): all three
+    // tensors share one floating-point type.
+    dtype_ = IsF32(x.dtype) ? RAFHIP_F32 : IsF16(x.dtype) ? RAFHIP_F16 : IsBF16(x.dtype) ? RAFHIP_BF16
+             : (x.dtype.code == kDLFloat && x.dtype.bits == 64) ? RAFHIP_F64 : -1;
+    auto same = [&](const DType& t) { return t.code == x.dtype.code && t.bits == x.dtype.bits; };
+    if (dtype_ < 0 || !same(args->dx->tensor.dtype) || !same(args->v->tensor.dtype))
+      error_msgs.push_back("raf.op.hip.sgd: x, dx and v must share one of float32, float64, float16, bfloat16");
     if (error_msgs.empty() && rafhip_device_count() <= 0)
       error_msgs.push_back("raf.op.hip.sgd: no HIP device is visible");
   }
@@ -108,10 +113,8 @@ class SgdHipEnv : public OpEnv, public HasLearningRate {
     RAF_CHECK(x.numel() == n && v.numel() == n && v1.numel() == n && x1.numel() == n,
               "raf.op.hip.sgd: tensor sizes differ");
     void* stream = DeviceAPI::Get(DevType::kROCM())->GetStream();
-    int st = rafhip_sgd_f32(static_cast<const float*>(x.data), static_cast<const float*>(dx.data),
-                            static_cast<const float*>(v.data), static_cast<float*>(v1.data),
-                            static_cast<float*>(x1.data), n, learning_rate_, mu_, stream);
-    if (st != RAFHIP_OK) throw Error(KernelError("rafhip_sgd_f32", st));
+    int st = rafhip_sgd(x.data, dx.data, v.data, v1.data, x1.data, n, dtype_, learning_rate_, mu_, stream);
+    if (st != RAFHIP_OK) throw Error(KernelError("rafhip_sgd", st));
   }
 
   void SetLearningRate(double learning_rate) override { learning_rate_ = learning_rate; }
@@ -122,6 +125,7 @@ class SgdHipEnv : public OpEnv, public HasLearningRate {
  private:
   double learning_rate_ = 0.0;
   double mu_ = 0.0;
+  int32_t dtype_ = RAFHIP_F32;
   std::string name_ = TruncateName(GetUniqueName("raf.op.hip.sgd"));
 };
 

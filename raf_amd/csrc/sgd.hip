@@ -19,8 +19,10 @@
 // parameter -- cast(dx), multiply, add(out=v), multiply, subtract(out=w), cast, add(out=p)
 // (python/raf/optim/sgd.py:187-215) -- and for the one-op-call-per-parameter loop of its imperative
 // optimizer (sgd.py:51-58).
+#include <cmath>
 #include <cstdint>
 #include <cstdlib>
+#include <cstring>
 #include <memory>
 #include <new>
 #include <vector>
@@ -94,6 +96,129 @@ __global__ __launch_bounds__(kSgdBlock) void sgd_scalar_kernel(
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ------------------------------------------------------------------ other element types
+// The reference's compute is written in the dtype of x0 (tir.const(value, dtype=x0.dtype),
+// python/raf/_tvm_op/sgd.py:18-19), so the op also exists for float64 and the 16-bit types.  Each
+// of the four operations is rounded to the element type on its own.  For binary16 and bfloat16
+// the operation is done the way a CPU without half arithmetic does it (the reference's CPU target
+// is bare `llvm`, include/raf/device.h:97-104): widen to fp32, operate there, round the result
+// back.  fp32 carries 24 >= 2p + 2 significant bits for both 16-bit formats (p = 11 and 8), so
+// the two roundings in a row give the correctly rounded 16-bit result: the same bits as native
+// half arithmetic would.
+template <typename T>
+struct SgdElem;
+template <>
+struct SgdElem<double> {
+  typedef double Store;
+  static constexpr int kWide = 2;  // elements per 16-byte access
+  static __device__ __forceinline__ double mul(double a, double b) { return a * b; }
+  static __device__ __forceinline__ double add(double a, double b) { return a + b; }
+  static __device__ __forceinline__ double sub(double a, double b) { return a - b; }
+  static double from_double(double x) { return x; }
+};
+template <>
+struct SgdElem<_Float16> {
+  typedef _Float16 Store;
+  static constexpr int kWide = 8;
+  static __device__ __forceinline__ _Float16 mul(_Float16 a, _Float16 b) { return (_Float16)((float)a * (float)b); }
+  static __device__ __forceinline__ _Float16 add(_Float16 a, _Float16 b) { return (_Float16)((float)a + (float)b); }
+  static __device__ __forceinline__ _Float16 sub(_Float16 a, _Float16 b) { return (_Float16)((float)a - (float)b); }
+  static _Float16 from_double(double x) { return (_Float16)x; }  // one rounding, like the constant's
+};
+template <>
+struct SgdElem<Bf16> {
+  typedef unsigned short Store;
+  static constexpr int kWide = 8;
+  static __device__ __forceinline__ unsigned short mul(unsigned short a, unsigned short b) {
+    return bf16_narrow(bf16_widen(a) * bf16_widen(b));
+  }
+  static __device__ __forceinline__ unsigned short add(unsigned short a, unsigned short b) {
+    return bf16_narrow(bf16_widen(a) + bf16_widen(b));
+  }
+  static __device__ __forceinline__ unsigned short sub(unsigned short a, unsigned short b) {
+    return bf16_narrow(bf16_widen(a) - bf16_widen(b));
+  }
+  // double -> bfloat16 with one rounding to nearest even (the value is finite and far from the
+  // range limits for any usable learning rate or momentum)
+  static unsigned short from_double(double x) {
+    const float f = (float)x;  // candidate; fix the double rounding by comparing neighbours
+    unsigned u;
+    std::memcpy(&u, &f, 4);
+    unsigned lo = u & 0xFFFF0000u, hi = lo + 0x10000u;
+    float flo, fhi;
+    std::memcpy(&flo, &lo, 4);
+    std::memcpy(&fhi, &hi, 4);
+    const double dlo = std::fabs(x - (double)flo), dhi = std::fabs((double)fhi - x);
+    const bool up = dhi < dlo || (dhi == dlo && ((lo >> 16) & 1u));
+    return (unsigned short)((up ? hi : lo) >> 16);
+  }
+};
+
+template <typename T>
+__device__ __forceinline__ void sgd_elem_t(typename SgdElem<T>::Store x0, typename SgdElem<T>::Store dx,
+                                           typename SgdElem<T>::Store v0, typename SgdElem<T>::Store lr,
+                                           typename SgdElem<T>::Store mu, typename SgdElem<T>::Store& v1,
+                                           typename SgdElem<T>::Store& x1) {
+  v1 = SgdElem<T>::add(SgdElem<T>::mul(mu, v0), dx);
+  x1 = SgdElem<T>::sub(x0, SgdElem<T>::mul(lr, v1));
+}
+
+// One 16-byte access per lane and array and trip; `vec` = every pointer is 16-byte aligned, else
+// element by element.
+template <typename T>
+__global__ __launch_bounds__(kSgdBlock) void sgd_typed_kernel(
+    const typename SgdElem<T>::Store* x, const typename SgdElem<T>::Store* dx,
+    const typename SgdElem<T>::Store* v, typename SgdElem<T>::Store* v_out,
+    typename SgdElem<T>::Store* x_out, int64_t n, typename SgdElem<T>::Store lr,
+    typename SgdElem<T>::Store mu, int vec) {
+  typedef typename SgdElem<T>::Store E;
+  constexpr int kW = SgdElem<T>::kWide;
+  typedef E Wide __attribute__((ext_vector_type(kW)));
+  const int64_t stride = (int64_t)gridDim.x * kSgdBlock;
+  const int64_t first = (int64_t)blockIdx.x * kSgdBlock + threadIdx.x;
+  int64_t done = 0;
+  if (vec) {
+    const int64_t nw = n / kW;
+    for (int64_t i = first; i < nw; i += stride) {
+      const Wide rx = __builtin_nontemporal_load(reinterpret_cast<const Wide*>(x) + i);
+      const Wide rd = __builtin_nontemporal_load(reinterpret_cast<const Wide*>(dx) + i);
+      const Wide rv = __builtin_nontemporal_load(reinterpret_cast<const Wide*>(v) + i);
+      Wide nv, nx;
+#pragma unroll
+      for (int j = 0; j < kW; ++j) {
+        E a, b;
+        sgd_elem_t<T>(rx[j], rd[j], rv[j], lr, mu, a, b);
+        nv[j] = a;
+        nx[j] = b;
+      }
+      __builtin_nontemporal_store(nv, reinterpret_cast<Wide*>(v_out) + i);
+      __builtin_nontemporal_store(nx, reinterpret_cast<Wide*>(x_out) + i);
+    }
+    done = nw * kW;
+  }
+  for (int64_t i = done + first; i < n; i += stride) {
+    E a, b;
+    sgd_elem_t<T>(x[i], dx[i], v[i], lr, mu, a, b);
+    v_out[i] = a;
+    x_out[i] = b;
+  }
+}
+
+template <typename T>
+void launch_sgd_typed(const void* x, const void* dx, const void* v, void* v_out, void* x_out, int64_t n,
+                      double learning_rate, double mu, hipStream_t s) {
+  typedef typename SgdElem<T>::Store E;
+  const bool vec = aligned16(x) && aligned16(dx) && aligned16(v) && aligned16(v_out) && aligned16(x_out);
+  const int64_t items = vec ? (n + SgdElem<T>::kWide - 1) / SgdElem<T>::kWide : n;
+  int64_t blocks = (items + kSgdBlock - 1) / kSgdBlock;
+  if (blocks > kMaxGridBlocks) blocks = kMaxGridBlocks;
+  // One rounding double -> element type, as tir.const(value, dtype) makes the constant.
+  hipLaunchKernelGGL(sgd_typed_kernel<T>, dim3((unsigned)blocks), dim3(kSgdBlock), 0, s,
+                     static_cast<const E*>(x), static_cast<const E*>(dx), static_cast<const E*>(v),
+                     static_cast<E*>(v_out), static_cast<E*>(x_out), n,
+                     SgdElem<T>::from_double(learning_rate), SgdElem<T>::from_double(mu), vec ? 1 : 0);
+}
 
 // ------------------------------------------------------------------ multi-tensor, in place
 // 1024 elements per work item: a workgroup makes one trip (one 16-byte access per lane and array)
@@ -250,6 +375,34 @@ extern "C" int rafhip_sgd_f32(const float* x, const float* dx, const float* v, f
                        v_out, x_out, done, n, lr32, mu32);
     RAFHIP_HIP_TRY(hipGetLastError());
   }
+  return RAFHIP_OK;
+}
+
+extern "C" int rafhip_sgd(const void* x, const void* dx, const void* v, void* v_out, void* x_out,
+                          int64_t n, int32_t dtype, double learning_rate, double mu, void* stream) {
+  using namespace rafhip;
+  if (dtype == RAFHIP_F32)
+    return rafhip_sgd_f32(static_cast<const float*>(x), static_cast<const float*>(dx),
+                          static_cast<const float*>(v), static_cast<float*>(v_out),
+                          static_cast<float*>(x_out), n, learning_rate, mu, stream);
+  clear_error();
+  if (dtype != RAFHIP_F64 && dtype != RAFHIP_F16 && dtype != RAFHIP_BF16)
+    return fail(RAFHIP_ERR_UNSUPPORTED, "rafhip_sgd: dtype %d", dtype);
+  if (n < 0) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_sgd: n = %lld < 0", (long long)n);
+  if (n == 0) return RAFHIP_OK;
+  if (!x || !dx || !v || !v_out || !x_out) return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_sgd: null tensor pointer");
+  const uintptr_t eb = dtype == RAFHIP_F64 ? 8 : 2;
+  for (const void* p : {x, dx, v, (const void*)v_out, (const void*)x_out})
+    if (reinterpret_cast<uintptr_t>(p) % eb != 0)
+      return fail(RAFHIP_ERR_INVALID_ARG, "rafhip_sgd: a tensor is not element-aligned");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == RAFHIP_F64)
+    launch_sgd_typed<double>(x, dx, v, v_out, x_out, n, learning_rate, mu, s);
+  else if (dtype == RAFHIP_F16)
+    launch_sgd_typed<_Float16>(x, dx, v, v_out, x_out, n, learning_rate, mu, s);
+  else
+    launch_sgd_typed<Bf16>(x, dx, v, v_out, x_out, n, learning_rate, mu, s);
+  RAFHIP_HIP_TRY(hipGetLastError());
   return RAFHIP_OK;
 }
 

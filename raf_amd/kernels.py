@@ -46,13 +46,27 @@ def sgd_f32(x: torch.Tensor, dx: torch.Tensor, v: torch.Tensor, learning_rate: f
 _DTYPE_CODE = {torch.float32: RAFHIP_F32, torch.float16: RAFHIP_F16, torch.bfloat16: RAFHIP_BF16}
 
 
+def sgd(x: torch.Tensor, dx: torch.Tensor, v: torch.Tensor, learning_rate: float, mu: float):
+    """``rafhip_sgd``: the step in the tensors' own element type (float32, float64, float16 or
+    bfloat16, the same for all three); returns new ``(v1, x1)``."""
+    code = {**_DTYPE_CODE, torch.float64: _lib.RAFHIP_F64}.get(x.dtype)
+    if code is None or dx.dtype != x.dtype or v.dtype != x.dtype:
+        raise TypeError("sgd: x, dx and v must share one of float32, float64, float16, bfloat16")
+    for t, name in ((x, "x"), (dx, "dx"), (v, "v")):
+        if not t.is_cuda or not t.is_contiguous():
+            raise TypeError(f"sgd: {name} must be a contiguous GPU tensor")
+    if not (x.shape == dx.shape == v.shape):
+        raise ValueError(f"sgd: shapes differ: x{tuple(x.shape)} dx{tuple(dx.shape)} v{tuple(v.shape)}")
+    v1, x1 = torch.empty_like(dx), torch.empty_like(dx)
+    check(_lib.optim().rafhip_sgd(x.data_ptr(), dx.data_ptr(), v.data_ptr(), v1.data_ptr(), x1.data_ptr(),
+                                  x.numel(), code, float(learning_rate), float(mu), _current_stream(x.device)))
+    return v1, x1
+
+
 class SgdPlan:
     """Owns a ``rafhip_sgd_plan``: momentum SGD over a whole parameter list, in place, one launch."""
 
-    def __init__(self, numels: Sequence[int], grad_dtype=torch.float32, device="cuda:0", **options):
-        """``options``: fields of ``rafhip_lans_plan_options`` (``schedule``, ``group_elements``,
-        ``round_slices``, ``blocks_per_cu``, ``stream_from_elements``, ``stream_hold_items``,
-        ``resident_mib``, ``apply_slice_shift``, ``spin_limit``); none changes a result."""
+    def __init__(self, numels: Sequence[int], grad_dtype=torch.float32, device="cuda:0"):
         self._h = c_void_p(None)
         self.lib = _lib.optim()
         self.device = torch.device(device)

@@ -48,9 +48,10 @@ def max_rel_err(got, want) -> float:
     return float(np.max(r))
 
 
-def round_to_f32(x: Fraction) -> Fraction:
-    """Exact round-to-nearest-even of a rational to the fp32 grid (normals and subnormals;
-    no overflow handling: callers stay far below FLT_MAX)."""
+def round_to_format(x: Fraction, mantissa_bits: int, emin: int) -> Fraction:
+    """Exact round-to-nearest-even of a rational to a binary floating-point grid with
+    `mantissa_bits` explicit fraction bits and least normal exponent `emin` (normals and
+    subnormals; no overflow handling: callers stay far below the format's maximum)."""
     if x == 0:
         return Fraction(0)
     sign = -1 if x < 0 else 1
@@ -60,10 +61,17 @@ def round_to_f32(x: Fraction) -> Fraction:
         e -= 1
     elif Fraction(2) ** (e + 1) <= a:
         e += 1
-    e = max(e, -126)
-    quantum = Fraction(2) ** (e - 23)
+    e = max(e, emin)
+    quantum = Fraction(2) ** (e - mantissa_bits)
     q = round(a / quantum)  # Fraction.__round__ rounds half to even
     return sign * q * quantum
+
+
+def round_to_f32(x: Fraction) -> Fraction:
+    return round_to_format(x, 23, -126)
+
+
+FORMATS = {"float16": (10, -14), "bfloat16": (7, -126), "float32": (23, -126), "float64": (52, -1022)}
 
 
 def f32_to_fraction(x) -> Fraction:

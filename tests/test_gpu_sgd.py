@@ -133,3 +133,36 @@ def test_reference_style_closed_form(native_libs, shape, seed):
     assert m_v1.shape == tuple(shape) and m_x1.shape == tuple(shape)
     _bits_equal(m_v1.reshape(-1), ov.reshape(-1))
     _bits_equal(m_x1.reshape(-1), ox.reshape(-1))
+
+
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "float64"])
+def test_sgd_in_other_element_types_is_bit_exact(native_libs, dtype):
+    """raf.op.sgd is written in the dtype of x (python/raf/_tvm_op/sgd.py:18-19): float64 and the
+    16-bit types, through the C ABI and through the operator front end, bit for bit against the
+    oracle (itself pinned by exact rational arithmetic; the reference's tests run fp32 only), on
+    sizes that exercise the 16-byte path, its tail and the unaligned path."""
+    from oracle.halfs import f32_to_bf16_bits
+    from raf_amd import kernels, op
+
+    rng = np.random.default_rng(11)
+    tdt = {"float16": torch.float16, "bfloat16": torch.bfloat16, "float64": torch.float64}[dtype]
+    for n, offset in ((100_003, 0), (8, 0), (5, 0), (70_001, 1), (1 << 20, 0)):
+        raw = [rng.normal(0, s, n + offset) for s in (0.02, 1e-3, 1e-3)]
+        raw[0][:4] = [6.1e-5, -5.96e-8, 1.0, 0.0]  # 16-bit subnormals among them
+        if dtype == "bfloat16":
+            host = [f32_to_bf16_bits(a.astype(np.float32)) for a in raw]
+            dev = [torch.from_numpy(a.view(np.int16).copy()).to(DEV).view(torch.bfloat16)[offset:] for a in host]
+            back = lambda t: t.view(torch.int16).cpu().numpy().view(np.uint16)
+        else:
+            npdt = np.float16 if dtype == "float16" else np.float64
+            host = [a.astype(npdt) for a in raw]
+            dev = [torch.from_numpy(a).to(DEV)[offset:] for a in host]
+            back = lambda t: t.cpu().numpy()
+        want_v, want_x = sgd_f32.sgd_step_typed(*[a[offset:] for a in host], 0.0123, 0.9, dtype)
+        for call in (kernels.sgd, op.sgd):
+            v1, x1 = call(*dev, 0.0123, 0.9)
+            assert v1.dtype == tdt and x1.dtype == tdt
+            assert np.array_equal(back(v1), want_v, equal_nan=False), (dtype, n, call.__module__, "v1")
+            assert np.array_equal(back(x1), want_x, equal_nan=False), (dtype, n, call.__module__, "x1")
+    with pytest.raises(TypeError):
+        kernels.sgd(torch.zeros(4, device=DEV), torch.zeros(4, device=DEV).half(), torch.zeros(4, device=DEV), 0.1, 0.9)

@@ -150,3 +150,67 @@ def test_list_step_is_the_op_per_parameter_with_exact_widening_and_rne_copies():
             assert np.array_equal(p.view(np.uint16), t)
     nx, nv, ps = sgd_f32.sgd_list_step(xs, d32, vs, 0.01, 0.9)
     assert ps is None and np.array_equal(nx[1], sgd_f32.sgd_step(xs[1], d32[1], vs[1], 0.01, 0.9)[1])
+
+
+# ------------------------------------------------------------------ other element types
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "float64"])
+def test_typed_step_against_exact_rationals(dtype):
+    """sgd_step_typed: constants rounded once from double, then four operations each rounded once
+    to the element type -- checked with exact rational arithmetic, on values that include
+    subnormals of the 16-bit formats and pairs whose sum falls between two grid points."""
+    from fractions import Fraction
+
+    from oracle.halfs import bf16_bits_to_f32, f32_to_bf16_bits
+    from tests.helpers import FORMATS, round_to_format
+
+    bits, emin = FORMATS[dtype]
+    rnd = lambda q: round_to_format(q, bits, emin)
+    rng = np.random.default_rng(77)
+    n = 400
+    raw = [rng.normal(0, s, n) for s in (0.02, 1e-3, 1e-3)]
+    raw[0][:8] = [6.1e-5, -5.96e-8, 3.0e-7, 1.0, -1.0, 0.333, 65000.0 if dtype == "float16" else 1e30, 0.0]
+    raw[2][:4] = [1.0009765625, 0.99951171875, 2.0**-14, -(2.0**-24)]
+    if dtype == "float64":
+        x, dx, v = (a.astype(np.float64) for a in raw)
+        value = lambda a: [Fraction(float(t)) for t in a]
+    elif dtype == "float16":
+        x, dx, v = (a.astype(np.float16) for a in raw)
+        value = lambda a: [Fraction(float(t)) for t in a]
+    else:
+        x, dx, v = (f32_to_bf16_bits(a.astype(np.float32)) for a in raw)
+        value = lambda a: [Fraction(float(t)) for t in bf16_bits_to_f32(a)]
+    lr, mu = 0.0123, 0.9
+    v1, x1 = sgd_f32.sgd_step_typed(x, dx, v, lr, mu, dtype)
+    lr_q, mu_q = rnd(Fraction(lr)), rnd(Fraction(mu))
+    fx, fd, fv, got_v, got_x = value(x), value(dx), value(v), value(v1), value(x1)
+    for i in range(n):
+        if i == 6:
+            continue  # the large entry: fine for the product, but keep the check away from overflow
+        want_v = rnd(rnd(mu_q * fv[i]) + fd[i])
+        want_x = rnd(fx[i] - rnd(lr_q * want_v))
+        assert got_v[i] == want_v, (dtype, i, "v1")
+        assert got_x[i] == want_x, (dtype, i, "x1")
+
+
+def test_typed_step_reduces_to_the_fp32_rule():
+    """The same construction in float32 must be sgd_step itself (a dropped rounding or a swapped
+    operand in the typed path would show here too)."""
+    rng = np.random.default_rng(5)
+    x, dx, v = (rng.normal(0, s, 1000).astype(np.float32) for s in (0.02, 1e-3, 1e-3))
+    v1, x1 = sgd_f32.sgd_step(x, dx, v, 0.01, 0.9)
+    w1, y1 = sgd_f32.sgd_step_typed(x, dx, v, float(np.float32(0.01)), float(np.float32(0.9)), "float64")
+    # float64 evaluation of the fp32 inputs agrees with the four-rounding fp32 result to the
+    # rounding errors of its operands (an ulp of |x0| ~ 0.02 is 1.9e-9, of |v| ~ 1e-3 1.2e-10)
+    assert np.max(np.abs(w1 - v1.astype(np.float64))) <= 6e-10
+    assert np.max(np.abs(y1 - x1.astype(np.float64))) <= 4e-9
+
+
+def test_bfloat16_constant_is_rounded_once():
+    """double -> bfloat16 directly; going through fp32 first would round 1 + 2^-8 + 2^-30 down
+    to a tie and then to even (1.0) instead of up."""
+    from oracle.halfs import bf16_bits_to_f32
+
+    tricky = 1.0 + 2.0**-8 + 2.0**-30
+    assert float(bf16_bits_to_f32(sgd_f32.bf16_from_double(tricky))) == 1.0 + 2.0**-7
+    assert float(bf16_bits_to_f32(sgd_f32.bf16_from_double(0.5))) == 0.5
+    assert float(bf16_bits_to_f32(sgd_f32.bf16_from_double(-3.0))) == -3.0
