@@ -84,6 +84,14 @@ typedef struct rafhip_raf_tuple rafhip_raf_tuple;
 int rafhip_raf_tuple_make(int32_t n, const rafhip_tensor_desc* fields, rafhip_raf_tuple** tuple_out);
 int rafhip_raf_tuple_replace(const rafhip_raf_tuple* base, int32_t first, int32_t count,
                              const rafhip_tensor_desc* fields, rafhip_raf_tuple** tuple_out);
+/* Rebinds fields [first, first + count) of a tuple to the storage `fields` name, in place, the way
+ * the reference's ndarray.update rebinds an array to another value (python/raf/_core/ndarray.py:
+ * 191-195): for a holder that owns its tuple alone and whose caller has let go of the tensors the
+ * range held.  Done (*done_out = 1) only if nothing else shares the tuple or a tensor value of the
+ * range and every field keeps its dtype, device and shape; otherwise nothing is changed
+ * (*done_out = 0) and the caller makes a new tuple with _replace. */
+int rafhip_raf_tuple_rebind(rafhip_raf_tuple* tuple, int32_t first, int32_t count,
+                            const rafhip_tensor_desc* fields, int32_t* done_out);
 int32_t rafhip_raf_tuple_size(const rafhip_raf_tuple* tuple); /* -1 on NULL */
 int rafhip_raf_tuple_destroy(rafhip_raf_tuple* tuple);
 /* rafhip_raf_lans_execute / rafhip_raf_sgd_multi_execute on a tuple made beforehand.  as_vm != 0

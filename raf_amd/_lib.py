@@ -179,6 +179,7 @@ DIALECT_SYMBOLS = {
                                         POINTER(TensorDesc), c_void_p, c_int64, c_void_p]),
     "rafhip_raf_tuple_make": (c_int, [c_int32, POINTER(TensorDesc), POINTER(c_void_p)]),
     "rafhip_raf_tuple_replace": (c_int, [c_void_p, c_int32, c_int32, POINTER(TensorDesc), POINTER(c_void_p)]),
+    "rafhip_raf_tuple_rebind": (c_int, [c_void_p, c_int32, c_int32, POINTER(TensorDesc), POINTER(c_int32)]),
     "rafhip_raf_tuple_size": (c_int32, [c_void_p]),
     "rafhip_raf_tuple_destroy": (c_int, [c_void_p]),
     "rafhip_raf_lans_execute_tuple": (c_int, [c_void_p, c_void_p, POINTER(TensorDesc), c_void_p, c_int64,

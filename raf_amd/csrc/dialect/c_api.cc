@@ -579,6 +579,36 @@ int rafhip_raf_tuple_replace(const rafhip_raf_tuple* base, int32_t first, int32_
   });
 }
 
+int rafhip_raf_tuple_rebind(rafhip_raf_tuple* tuple, int32_t first, int32_t count,
+                            const rafhip_tensor_desc* fields, int32_t* done_out) {
+  return Guard([&] {
+    if (!done_out) throw Error("rafhip_raf_tuple_rebind: done_out is NULL");
+    *done_out = 0;
+    if (!tuple) throw Error("rafhip_raf_tuple_rebind: tuple is NULL");
+    const int64_t n = (int64_t)tuple->value->fields.size();
+    if (first < 0 || count < 0 || (int64_t)first + count > n || (count > 0 && !fields))
+      throw Error("rafhip_raf_tuple_rebind: range [" + std::to_string(first) + ", " +
+                  std::to_string((int64_t)first + count) + ") does not fit a tuple of " + std::to_string(n));
+    if (tuple->value.use_count() != 1) return;
+    std::vector<value::Value>& held = tuple->value->fields;
+    for (int32_t i = 0; i < count; ++i) {
+      const value::Value& v = held[(size_t)first + (size_t)i];
+      const auto* t = dynamic_cast<const value::TensorValueObj*>(v.get());
+      const rafhip_tensor_desc& d = fields[i];
+      if (!t || v.use_count() != 1 || d.ndim < 0 || (size_t)d.ndim != t->tensor.shape.size() ||
+          (d.ndim > 0 && !d.shape) || d.dtype_code != t->tensor.dtype.code ||
+          d.dtype_bits != t->tensor.dtype.bits || d.device_type != (int)t->tensor.device.device_type() ||
+          d.device_id != t->tensor.device.device_id())
+        return;
+      for (int32_t k = 0; k < d.ndim; ++k)
+        if (d.shape[k] != t->tensor.shape[(size_t)k]) return;
+    }
+    for (int32_t i = 0; i < count; ++i)
+      static_cast<value::TensorValueObj*>(held[(size_t)first + (size_t)i].get())->tensor.data = fields[i].data;
+    *done_out = 1;
+  });
+}
+
 int32_t rafhip_raf_tuple_size(const rafhip_raf_tuple* tuple) {
   return tuple ? (int32_t)tuple->value->fields.size() : -1;
 }

@@ -17,6 +17,15 @@
 //   signature(descs_addr, n) -> bytes
 //       dtype, device and shape of every descriptor packed into one bytes object: what two
 //       lists must share to be served by one OpEnv
+//   rebind(tensors, first, end, descs_addr, ptrs_addr) -> bool
+//       brings descriptors and recorded pointers of a list described earlier up to date with
+//       `tensors`, of which [first, end) are other objects than the ones described: True, and the
+//       addresses of that range written, if those have the recorded dtype, device and shape and
+//       every tensor outside the range still lives at its recorded address; False, and nothing
+//       written, otherwise
+//
+//   grads(params) -> (list, missing)
+//       the `.grad` of every parameter (None where there is none) and how many are None
 //
 // torch is used for nothing but this object access; no kernels, no allocator, no dispatcher.
 #include <Python.h>
@@ -154,6 +163,66 @@ PyObject* signature_impl(PyObject* args) {
                                    (Py_ssize_t)(words.size() * sizeof(int64_t)));
 }
 
+PyObject* rebind_impl(PyObject* args) {
+  PyObject* list;
+  long long first, end;
+  unsigned long long descs_addr, ptrs_addr;
+  if (!PyArg_ParseTuple(args, "OLLKK", &list, &first, &end, &descs_addr, &ptrs_addr)) return nullptr;
+  if (!list_arg(list, "tensors")) return nullptr;
+  const Py_ssize_t n = PyList_GET_SIZE(list);
+  if (first < 0 || end < first || end > (long long)n) {
+    PyErr_SetString(PyExc_IndexError, "range outside the list");
+    return nullptr;
+  }
+  auto* descs = reinterpret_cast<rafhip_tensor_desc*>(descs_addr);
+  auto* ptrs = reinterpret_cast<uint64_t*>(ptrs_addr);
+  for (Py_ssize_t i = 0; i < n; ++i) {
+    const at::Tensor* t = tensor_at(list, i);
+    if (!t) return nullptr;
+    if (i < first || i >= end) {
+      if (reinterpret_cast<uint64_t>(t->data_ptr()) != ptrs[i]) Py_RETURN_FALSE;
+      continue;
+    }
+    const rafhip_tensor_desc& d = descs[i];
+    int32_t code = 0, bits = 0;
+    if (!t->is_contiguous() || !dtype_of(t->scalar_type(), &code, &bits) || code != d.dtype_code ||
+        bits != d.dtype_bits || (t->is_cuda() ? kDevRocm : kDevCpu) != d.device_type ||
+        (t->is_cuda() && t->device().has_index() ? t->device().index() : 0) != d.device_id)
+      Py_RETURN_FALSE;
+    const auto sizes = t->sizes();
+    if ((int32_t)sizes.size() != d.ndim) Py_RETURN_FALSE;
+    for (int32_t k = 0; k < d.ndim; ++k)
+      if (sizes[(size_t)k] != d.shape[k]) Py_RETURN_FALSE;
+  }
+  for (Py_ssize_t i = (Py_ssize_t)first; i < (Py_ssize_t)end; ++i) {
+    void* p = THPVariable_Unpack(PyList_GET_ITEM(list, i)).data_ptr();
+    descs[i].data = p;
+    ptrs[i] = reinterpret_cast<uint64_t>(p);
+  }
+  Py_RETURN_TRUE;
+}
+
+PyObject* grads_impl(PyObject* args) {
+  PyObject* list;
+  if (!PyArg_ParseTuple(args, "O", &list)) return nullptr;
+  if (!list_arg(list, "params")) return nullptr;
+  static PyObject* const name = PyUnicode_InternFromString("grad");
+  const Py_ssize_t n = PyList_GET_SIZE(list);
+  PyObject* out = PyList_New(n);
+  if (!out) return nullptr;
+  Py_ssize_t missing = 0;
+  for (Py_ssize_t i = 0; i < n; ++i) {
+    PyObject* g = PyObject_GetAttr(PyList_GET_ITEM(list, i), name);  // new reference
+    if (!g) {
+      Py_DECREF(out);
+      return nullptr;
+    }
+    missing += g == Py_None;
+    PyList_SET_ITEM(out, i, g);  // steals it
+  }
+  return Py_BuildValue("(Nn)", out, missing);
+}
+
 // No C++ exception may reach the interpreter: torch raises c10::Error for tensors without storage.
 template <PyObject* (*F)(PyObject*)>
 PyObject* guarded(PyObject*, PyObject* args) {
@@ -171,6 +240,8 @@ PyMethodDef kMethods[] = {
     {"describe", guarded<describe_impl>, METH_VARARGS, "fill descriptors, shapes and data pointers of a tensor list"},
     {"same_storage", guarded<same_storage_impl>, METH_VARARGS, "whether the tensors' data pointers equal the recorded ones"},
     {"diff_range", guarded<diff_range_impl>, METH_VARARGS, "index range outside which two lists hold the same objects"},
+    {"rebind", guarded<rebind_impl>, METH_VARARGS, "bring a described list up to date with tensors that replace a range of it"},
+    {"grads", guarded<grads_impl>, METH_VARARGS, "the .grad of every parameter and the number of missing ones"},
     {"signature", guarded<signature_impl>, METH_VARARGS, "dtype, device and shape of every descriptor as bytes"},
     {nullptr, nullptr, 0, nullptr}};
 

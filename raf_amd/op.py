@@ -150,6 +150,7 @@ class TensorList:
         self._tensors = list(tensors)
         self.track = bool(track)
         self.rebuilds = 0
+        self.rebinds = 0
         self._handle = c_void_p(None)
         self._build(_share)
 
@@ -218,6 +219,29 @@ class TensorList:
         merged = self._tensors[:first] + tensors + self._tensors[end:]
         return TensorList(merged, self.track, _share=(self, first, end))
 
+    def _rebind(self, tensors: list, first: int, end: int) -> bool:
+        """Takes over ``tensors``, which differ from this handle's in [first, end), in place: the
+        tuple's tensor values of that range are rebound to the new storage, the way the
+        reference's ``ndarray.update`` rebinds an array (python/raf/_core/ndarray.py:191-195).
+        Only for a handle that no caller holds.  False, with nothing changed, if a tensor of the
+        range differs in dtype, device or shape, a tensor outside it has moved, or something
+        still shares the tuple."""
+        if not _lib.glue().rebind(tensors, first, end, ctypes.addressof(self._descs), ctypes.addressof(self._ptrs)):
+            return False
+        done = ctypes.c_int32(0)
+        fields = ctypes.cast(ctypes.addressof(self._descs) + ctypes.sizeof(TensorDesc) * first,
+                             ctypes.POINTER(TensorDesc))
+        check_raf(_lib.dialect().rafhip_raf_tuple_rebind(self._handle, first, end - first, fields,
+                                                         ctypes.byref(done)))
+        if not done.value:  # the descriptors already name the new storage: make the tuple anew from them
+            h = c_void_p(None)
+            check_raf(_lib.dialect().rafhip_raf_tuple_make(len(tensors), self._descs, ctypes.byref(h)))
+            old, self._handle = self._handle, h
+            _lib.dialect().rafhip_raf_tuple_destroy(old)
+        self._tensors = list(tensors)
+        self.rebinds += 1
+        return True
+
     def __len__(self):
         return len(self._tensors)
 
@@ -258,9 +282,22 @@ def _tensor_list(tensors) -> TensorList:
                 _recent_lists.remove(h)
                 _recent_lists.appendleft(h)
             return h.refresh()
-        if nearest is None or end - first < nearest[2] - nearest[1]:
+        if 2 * (end - first) <= len(lst) and (nearest is None or end - first < nearest[2] - nearest[1]):
             nearest = (h, first, end)
-    if nearest is not None and 2 * (nearest[2] - nearest[1]) <= len(lst) and nearest[0].current():
+    if nearest is not None and len(_recent_lists) == _recent_lists.maxlen:
+        # Every step brings tensors never seen before (gradients allocated per iteration): rather
+        # than make handle after handle, the one used longest ago takes the new tensors over.
+        # Callers that alternate between a few lists never get here: theirs are all found above.
+        for h in reversed(_recent_lists):
+            if len(h) != len(lst):
+                continue
+            first, end = glue.diff_range(lst, h._tensors)
+            if 2 * (end - first) <= len(lst) and h._rebind(lst, first, end):
+                _recent_lists.remove(h)
+                _recent_lists.appendleft(h)
+                return h
+            break
+    if nearest is not None and nearest[0].current():
         h = nearest[0].replaced(nearest[1], lst[nearest[1]:nearest[2]])
     else:
         h = TensorList(lst)

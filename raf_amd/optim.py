@@ -7,6 +7,7 @@ from __future__ import annotations
 
 import torch
 
+from . import _lib
 from . import op as _op
 
 
@@ -27,6 +28,7 @@ class SGD:
             raise ValueError("Invalid momentum value: {}".format(momentum))
         self.params = []
         self._lists = None  # the weight and velocity lists of all parameters, made on first use
+        self._xs = None  # the parameters themselves as a list, made on first use
         self._model = None  # (data pointers, aliases of the half-precision parameters' data)
         self._lr = learning_rate
         self._momentum = momentum
@@ -43,9 +45,12 @@ class SGD:
 
     def step(self):
         """Update the parameters with gradients."""
-        live = [(x, w, v) for x, w, v in self.params if x.grad is not None]
-        if not live:
+        if self._xs is None:
+            self._xs = [x for x, _, _ in self.params]
+        grads, missing = _lib.glue().grads(self._xs)  # one pass at C speed
+        if missing == len(grads):
             return
+        live = self.params if not missing else [t for t, g in zip(self.params, grads) if g is not None]
         if not self.multi_tensor:
             for x0, _, v0 in live:
                 v1, x1 = _op.sgd(x0.data, x0.grad, v0, self._lr, self._momentum)
@@ -54,15 +59,15 @@ class SGD:
                 x0.data.copy_(x1)
                 v0.copy_(v1)
             return
-        if len(live) == len(self.params):
-            # every parameter has a gradient: the weight and velocity lists made once, and one
-            # attribute read per parameter
+        if not missing:
+            # every parameter has a gradient: the weight and velocity lists made once
             if self._lists is None:
                 self._lists = ([w for _, w, _ in self.params], [v for _, _, v in self.params])
             ws, vs = self._lists
         else:
             ws, vs = [w for _, w, _ in live], [v for _, _, v in live]
-        tensor_list = ws + [x.grad for x, _, _ in live] + vs
+            grads = [g for g in grads if g is not None]
+        tensor_list = ws + grads + vs
         if self.mixed:
             _op.sgd_multi_mixed(tensor_list + self._model_data(live), self._lr, self._momentum)
         else:
@@ -104,6 +109,7 @@ class LANS:
         # would block on the previous step's kernels.
         self._step_dev = None
         self._lists = None  # the w, m, v lists of all parameters, made on first use
+        self._xs = None  # the parameters themselves as a list, made on first use
         self._model = None  # (data pointers, aliases of the half-precision parameters' data)
         params = list(params)
         halves = {x.dtype for x in params if isinstance(x, torch.Tensor)} & {torch.float16, torch.bfloat16}
@@ -119,8 +125,10 @@ class LANS:
     def step(self):
         """Update the parameters with gradients."""
         params = self.params
-        grads = [x.grad for x, _, _, _ in params]
-        if any(g is None for g in grads):  # the reference skips parameters without a gradient (lans.py:81-83)
+        if self._xs is None:
+            self._xs = [t[0] for t in params]
+        grads, missing = _lib.glue().grads(self._xs)  # one pass at C speed
+        if missing:  # the reference skips parameters without a gradient (lans.py:81-83)
             live = [i for i, g in enumerate(grads) if g is not None]
             g_list = [grads[i] for i in live]
             x_list = [params[i][1] for i in live]

@@ -144,3 +144,35 @@ def test_sgd_multi_with_a_handle_and_fresh_gradient_objects(native_libs):
         assert np.array_equal(tx[t].cpu().numpy(), ox[t]) and np.array_equal(tv[t].cpu().numpy(), ov[t])
     assert len([k for k in op._env_cache if k[0] == "sgd_multi"]) == 1
     op.clear_op_env_cache()
+
+
+def test_gradients_allocated_anew_every_step(native_libs):
+    """torch's default: `.grad` tensors are new objects at new addresses every iteration.  The
+    front end has a handful of handles for recent lists; once they are taken the oldest is rebound
+    to the new gradients in place.  Twelve steps with different gradient values at every step
+    against the oracle, one OpEnv throughout."""
+    from raf_amd import op
+
+    hp = LansHParams()
+    g0, w, m, v = lans_inputs(SIZES, cfg=131)
+    n = len(SIZES)
+    op.clear_op_env_cache()
+    tw, tm, tv = _dev(w), _dev(m), _dev(v)
+    step = torch.zeros((), device=DEV)
+    ow, om, ov = w, m, v
+    held = []  # keeps every step's gradients alive, so that every step's are at addresses of their own
+    steps = op._recent_lists.maxlen + 4
+    for s in range(1, steps + 1):
+        g = [(a * np.float32(1.0 + 0.125 * s)).astype(np.float32) for a in g0]
+        tg = _dev(g)
+        held.append(tg)
+        step.fill_(float(s))
+        op.lans(tg + tw + tm + tv, step, *_args(hp))
+        ow, om, ov, _ = lans_f64.lans_step(g, ow, om, ov, s, hp)
+    torch.cuda.synchronize()
+    assert len({t.data_ptr() for tg in held for t in tg if t.numel()}) == steps * sum(1 for k in SIZES if k)
+    assert len([k for k in op._env_cache if k[0] == "lans"]) == 1
+    assert len(op._recent_lists) == op._recent_lists.maxlen
+    assert sum(h.rebinds for h in op._recent_lists) == 4
+    _check(tg + tw + tm + tv, n, ow, om, ov, tol=2e-5)
+    op.clear_op_env_cache()

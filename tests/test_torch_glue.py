@@ -120,3 +120,108 @@ def test_tensor_list_handle_on_the_cpu(native_libs):
     assert h2 is not h and h2[5] is ts[5]
     assert op._tensor_list(ts) is h
     op.clear_op_env_cache()
+
+
+def test_rebind_writes_only_what_fits(native_libs):
+    """`rebind` brings a described list up to date with other tensors in a range: the addresses
+    of the range are written if dtype, device and shape agree and the rest has not moved; nothing
+    at all is written otherwise."""
+    glue = native_libs.glue()
+    ts = [torch.zeros(2, 3), torch.zeros(7), torch.zeros(4, dtype=torch.float16), torch.zeros(())]
+    descs, ptrs, _shapes, _ = _describe(glue, ts)
+    addr = lambda: (ctypes.addressof(descs), ctypes.addressof(ptrs))
+    new = [torch.ones(2, 3), torch.ones(7)]
+    assert glue.rebind(new + ts[2:], 0, 2, *addr()) is True
+    assert [ptrs[i] for i in range(4)] == [t.data_ptr() for t in new + ts[2:]]
+    assert descs[0].data == new[0].data_ptr() and descs[1].data == new[1].data_ptr()
+    assert descs[2].data == ts[2].data_ptr() and descs[0].ndim == 2 and descs[0].shape[1] == 3
+    before = [ptrs[i] for i in range(4)]
+    for bad in ([torch.ones(3, 2), torch.ones(7)],                       # another shape
+                [torch.ones(2, 3), torch.ones(7, dtype=torch.float64)],  # another dtype
+                [torch.ones(2, 3), torch.ones(7, 1)],                    # another rank
+                [torch.ones(3, 2).t(), torch.ones(7)]):                  # not contiguous
+        assert glue.rebind(bad + ts[2:], 0, 2, *addr()) is False
+        assert [ptrs[i] for i in range(4)] == before and descs[0].data == before[0]
+    # a tensor outside the range that has moved since: refused as a whole
+    moved = ts[3]
+    moved.data = torch.ones(())
+    assert glue.rebind([torch.ones(2, 3), torch.ones(7)] + ts[2:], 0, 2, *addr()) is False
+    assert [ptrs[i] for i in range(4)] == before
+    with pytest.raises(IndexError):
+        glue.rebind(new + ts[2:], 3, 5, *addr())
+    with pytest.raises(TypeError):
+        glue.rebind(new + [None, None], 0, 2, *addr())
+
+
+def test_lists_with_new_tensors_every_call_reuse_the_oldest_handle(native_libs):
+    """Gradients allocated anew at every step: once the front end's few recent handles are all
+    taken, the one used longest ago takes the new tensors over in place instead of a handle being
+    made per step; lists that come back are still found, and a list that does not fit (another
+    shape in the range) gets a handle of its own."""
+    from raf_amd import op
+
+    op.clear_op_env_cache()
+    state = [torch.zeros(3, 5) for _ in range(9)]
+    keep, handles = [], []
+    cap = op._recent_lists.maxlen
+    for step in range(cap + 4):
+        g = [torch.zeros(3, 5) for _ in range(3)]
+        keep.append(g)
+        h = op._tensor_list(g + state)
+        assert h[0] is g[0] and h[3] is state[0] and h._ptrs[2] == g[2].data_ptr() and h.current()
+        assert native_libs.dialect().rafhip_raf_tuple_size(h._handle) == 12
+        handles.append(h)
+    assert len(set(map(id, handles[:cap]))) == cap            # a handle each while there is room
+    assert all(any(h is e for e in handles[:cap]) for h in handles[cap:])  # then reuse
+    assert handles[cap] is handles[0] and handles[cap].rebinds == 1
+    assert len(op._recent_lists) == cap
+    # the most recent lists are still found as they are
+    assert op._tensor_list(keep[-1] + state) is handles[-1]
+    assert op._tensor_list(keep[-2] + state) is handles[-2]
+    # a range that does not fit the old descriptors: a handle made from scratch, nothing rebound
+    rebinds = sum(h.rebinds for h in op._recent_lists)
+    odd = op._tensor_list([torch.zeros(5, 3) for _ in range(3)] + state)
+    assert odd.rebinds == 0 and sum(h.rebinds for h in op._recent_lists if h is not odd) <= rebinds
+    assert odd[0].shape == (5, 3) and odd.signature != handles[-1].signature
+    op.clear_op_env_cache()
+
+
+def test_tuple_rebind_refuses_a_shared_tuple(native_libs):
+    """The C window rebinds in place only what nothing else shares: a tuple whose fields another
+    tuple shares (made from it by _replace) is left as it is."""
+    from raf_amd import op
+    from raf_amd._lib import TensorDesc, check_raf
+
+    lib = native_libs.dialect()
+    ts = [torch.zeros(4) for _ in range(6)]
+    a = op.TensorList(ts)
+    b = a.replaced(0, [torch.zeros(4), torch.zeros(4)])   # shares fields 2..5 with a
+    keep: list = []
+    fresh = [torch.ones(4), torch.ones(4)]
+    descs = (TensorDesc * 2)(*[op._desc(t, keep) for t in fresh])
+    done = ctypes.c_int32(-1)
+    check_raf(lib.rafhip_raf_tuple_rebind(a._handle, 4, 2, descs, ctypes.byref(done)))
+    assert done.value == 0                                 # fields 4, 5 are b's too
+    check_raf(lib.rafhip_raf_tuple_rebind(a._handle, 0, 2, descs, ctypes.byref(done)))
+    assert done.value == 1                                 # fields 0, 1 are a's alone
+    wrong = (TensorDesc * 2)(*[op._desc(t, keep) for t in (torch.ones(4, 1), torch.ones(4))])
+    check_raf(lib.rafhip_raf_tuple_rebind(a._handle, 0, 2, wrong, ctypes.byref(done)))
+    assert done.value == 0
+    assert lib.rafhip_raf_tuple_rebind(a._handle, 5, 2, descs, ctypes.byref(done)) != 0  # out of range
+    del b
+
+
+def test_grads_reads_every_parameters_gradient(native_libs):
+    glue = native_libs.glue()
+    ps = [torch.nn.Parameter(torch.zeros(3)) for _ in range(4)]
+    assert glue.grads(ps) == ([None] * 4, 4)
+    ps[1].grad = torch.ones(3)
+    ps[3].grad = torch.full((3,), 2.0)
+    got, missing = glue.grads(ps)
+    assert missing == 2 and got[0] is None and got[2] is None
+    assert got[1] is ps[1].grad and got[3] is ps[3].grad
+    assert glue.grads([]) == ([], 0)
+    with pytest.raises(AttributeError):
+        glue.grads([object()])
+    with pytest.raises(TypeError):
+        glue.grads(tuple(ps))
