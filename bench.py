@@ -789,7 +789,8 @@ def bench_traced_lans(name, wl, args):
 
 
 def _short_traffic_source(source: str) -> str:
-    """One token for the line the driver keeps; the full sentence is in profiles/ and DESIGN.md."""
+    """One token instead of the sentence, to keep the JSON line short: the summary's path, "stale"
+    (measured on other kernel sources) or "unmeasured"."""
     if "other kernel sources" in source:
         return "stale"
     if source.startswith("profiles/"):
