@@ -3,10 +3,9 @@
 
 #include <cstdio>
 #include <cstdlib>
-#include <list>
 #include <map>
 #include <mutex>
-#include <unordered_map>
+#include <vector>
 
 namespace raf {
 namespace memory_pool {
@@ -142,61 +141,115 @@ class NoPool final : public MemoryPool {
 };
 
 // ---------------------------------------------------------------------------- page_unit_pool
-// Requests are rounded up to 4 KiB pages and chunks are kept, grouped by size, after their users
-// let go; a request takes an idle chunk of its size if there is one.  When the device runs out of
-// memory, or the pool outgrows RAF_MEMORY_POOL_SIZE_LIMIT, idle chunks are released and the
-// allocation is tried once more (page_unit_pool.cc:64-231).
+// The reference's caching strategy (page_unit_pool.cc:64-231): requests are rounded up to 4 KiB
+// pages, a block whose users have let go is kept for the next request of its size, and when the
+// device runs out of memory, or the pool outgrows RAF_MEMORY_POOL_SIZE_LIMIT, the idle blocks
+// go back to the device and the allocation is tried once more.
+//
+// Bookkeeping here: a block handed out is a `Lease` whose destructor returns the block to a
+// per-size free list, so taking and returning a block are O(1) and the pool never scans for
+// blocks that have become idle.  The free lists live in a `Ledger` that the leases share with
+// the pool: a lease that outlives its pool (RemovePool while tensors are alive) finds the ledger
+// closed and hands its block straight back to the device.
 class PageUnitPool final : public MemoryPool {
+  struct Ledger {
+    std::mutex mu;
+    std::shared_ptr<DeviceAPI> api;
+    std::map<int64_t, std::vector<void*>> idle;  // page-rounded size -> blocks nobody holds
+    int64_t idle_bytes = 0;
+    int64_t leased_bytes = 0;
+    bool closed = false;
+
+    // Returns every idle block to the device; the number of bytes that freed.
+    int64_t DrainLocked() {
+      const int64_t freed = idle_bytes;
+      for (auto& bucket : idle)
+        for (void* block : bucket.second) Release([&] { api->FreeMemory(block); });
+      idle.clear();
+      idle_bytes = 0;
+      return freed;
+    }
+  };
+
+  class Lease final : public Memory {
+   public:
+    Lease(void* ptr, int64_t nbytes, const Device& dev, std::shared_ptr<Ledger> ledger)
+        : nbytes_(nbytes), ledger_(std::move(ledger)) {
+      data = ptr;
+      device = dev;
+    }
+    ~Lease() override {
+      if (data == nullptr) return;
+      std::lock_guard<std::mutex> lock(ledger_->mu);
+      ledger_->leased_bytes -= nbytes_;
+      if (ledger_->closed) {
+        Release([&] { ledger_->api->FreeMemory(data); });
+        return;
+      }
+      ledger_->idle[nbytes_].push_back(data);
+      ledger_->idle_bytes += nbytes_;
+    }
+
+   private:
+    int64_t nbytes_;
+    std::shared_ptr<Ledger> ledger_;
+  };
+
  public:
   PageUnitPool(const Device& dev, int64_t limit)
-      : device_(dev), max_pool_size_(limit), api_(DeviceAPI::Get(dev.device_type())) {
-    if (IsGpu(dev.device_type())) api_->SetDevice(dev.device_id());
+      : device_(dev), size_limit_(limit), ledger_(std::make_shared<Ledger>()) {
+    ledger_->api = DeviceAPI::Get(dev.device_type());
+    if (IsGpu(dev.device_type())) ledger_->api->SetDevice(dev.device_id());
+  }
+  ~PageUnitPool() override {
+    std::lock_guard<std::mutex> lock(ledger_->mu);
+    ledger_->closed = true;
+    ledger_->DrainLocked();
   }
   std::string GetName() override { return "page_unit_pool"; }
-  int64_t GetAllocBytes(int64_t nbytes) override {
-    return (nbytes + kPage - 1) / kPage * kPage;
-  }
+  int64_t GetAllocBytes(int64_t nbytes) override { return (nbytes + kPage - 1) / kPage * kPage; }
 
   std::shared_ptr<Memory> Alloc(int64_t nbytes, int64_t alignment) override {
     RAF_CHECK(nbytes >= 0, "negative allocation size");
     nbytes = GetAllocBytes(nbytes);
-    if (nbytes == 0) return std::make_shared<NonOwnedMemory>(nullptr, device_, api_);
-    std::lock_guard<std::mutex> lock(mu_);
-    auto& chunks = pool_[nbytes];
-    for (const auto& c : chunks)  // the pool's own reference is the only one: the chunk is idle
-      if (c.use_count() == 1 && reinterpret_cast<uintptr_t>(c->data) % (uintptr_t)alignment == 0) return c;
-    void* ptr = TryDevice(nbytes, alignment);
-    if (ptr == nullptr || (max_pool_size_ > 0 && pool_bytes_ >= max_pool_size_)) {
-      const int64_t freed = FreeIdleChunks();
-      if (ptr == nullptr && freed > 0) ptr = TryDevice(nbytes, alignment);
+    if (nbytes == 0) return std::make_shared<Lease>(nullptr, 0, device_, ledger_);
+    std::lock_guard<std::mutex> lock(ledger_->mu);
+    void* block = TakeIdleLocked(nbytes, alignment);
+    if (block == nullptr) {
+      block = TryDevice(nbytes, alignment);
+      const bool over_limit =
+          size_limit_ > 0 && ledger_->idle_bytes + ledger_->leased_bytes + (block ? nbytes : 0) > size_limit_;
+      if (block == nullptr || over_limit) {
+        const int64_t freed = ledger_->DrainLocked();
+        if (block == nullptr && freed > 0) block = TryDevice(nbytes, alignment);
+      }
+      if (block == nullptr) {
+        // the reference's message (page_unit_pool.cc:112-117): its tests match on it
+        throw Error("Out-Of-Memory. Tried to allocate " + std::to_string(BytesToMegaBytes((float)nbytes)) +
+                    " MBs; Already allocated " +
+                    std::to_string(BytesToMegaBytes((float)(ledger_->idle_bytes + ledger_->leased_bytes))) +
+                    " MBs and used " + std::to_string(BytesToMegaBytes((float)ledger_->leased_bytes)) + " MBs");
+      }
     }
-    if (ptr == nullptr) {
-      auto sz = SizesLocked();
-      throw Error("Out-Of-Memory. Tried to allocate " + std::to_string(BytesToMegaBytes((float)nbytes)) +
-                  " MBs; Already allocated " + std::to_string(sz.second) + " MBs and used " +
-                  std::to_string(sz.first) + " MBs");
-    }
-    pool_bytes_ += nbytes;
-    auto mem = std::make_shared<NonOwnedMemory>(ptr, device_, api_);
-    pool_[nbytes].push_back(mem);
-    return mem;
+    ledger_->leased_bytes += nbytes;
+    return std::make_shared<Lease>(block, nbytes, device_, ledger_);
   }
   std::shared_ptr<Memory> AllocAsync(int64_t, void*, int64_t) override {
-    throw Error("Please use NoPool to use AllocAsync.");
+    throw Error("Please use NoPool to use AllocAsync.");  // page_unit_pool.cc:127
   }
   std::vector<std::shared_ptr<Memory>> AllocBatch(const std::vector<int64_t>& nbytes,
                                                   int64_t alignment) override {
-    std::vector<std::shared_ptr<Memory>> ret;
-    ret.reserve(nbytes.size());
-    for (int64_t b : nbytes) ret.push_back(Alloc(b, alignment));
-    return ret;
+    std::vector<std::shared_ptr<Memory>> blocks(nbytes.size());
+    for (size_t i = 0; i < nbytes.size(); ++i) blocks[i] = Alloc(nbytes[i], alignment);
+    return blocks;
   }
   std::pair<float, float> GetPoolSize() override {
-    auto dev = api_->GetPoolSize();  // a device-side pool's own numbers win if it has any
+    auto dev = ledger_->api->GetPoolSize();  // a device-side pool's own numbers win if it has any
     if (dev.first != 0 || dev.second != 0)
       return {BytesToMegaBytes((float)dev.first), BytesToMegaBytes((float)dev.second)};
-    std::lock_guard<std::mutex> lock(mu_);
-    return SizesLocked();
+    std::lock_guard<std::mutex> lock(ledger_->mu);
+    return {BytesToMegaBytes((float)ledger_->leased_bytes),
+            BytesToMegaBytes((float)(ledger_->leased_bytes + ledger_->idle_bytes))};
   }
   static MemoryPool* make(const Device& dev) {
     int64_t limit = 0;
@@ -207,41 +260,32 @@ class PageUnitPool final : public MemoryPool {
  private:
   static constexpr int64_t kPage = 4096;
 
+  // The most recently returned idle block of this size that satisfies the alignment, if any.
+  void* TakeIdleLocked(int64_t nbytes, int64_t alignment) {
+    auto bucket = ledger_->idle.find(nbytes);
+    if (bucket == ledger_->idle.end()) return nullptr;
+    std::vector<void*>& blocks = bucket->second;
+    for (size_t i = blocks.size(); i-- > 0;) {
+      if (reinterpret_cast<uintptr_t>(blocks[i]) % (uintptr_t)alignment != 0) continue;
+      void* block = blocks[i];
+      blocks.erase(blocks.begin() + (std::ptrdiff_t)i);
+      if (blocks.empty()) ledger_->idle.erase(bucket);
+      ledger_->idle_bytes -= nbytes;
+      return block;
+    }
+    return nullptr;
+  }
   void* TryDevice(int64_t nbytes, int64_t alignment) {
     try {
-      return api_->AllocMemory(nbytes, alignment);
+      return ledger_->api->AllocMemory(nbytes, alignment);
     } catch (const std::exception&) {
       return nullptr;
     }
   }
-  int64_t FreeIdleChunks() {
-    int64_t freed = 0;
-    pool_bytes_ = 0;
-    for (auto& kv : pool_) {
-      const size_t before = kv.second.size();
-      kv.second.remove_if([](const std::shared_ptr<Memory>& m) { return m.use_count() == 1; });
-      freed += kv.first * (int64_t)(before - kv.second.size());
-      pool_bytes_ += kv.first * (int64_t)kv.second.size();
-    }
-    return freed;
-  }
-  std::pair<float, float> SizesLocked() {
-    float used = 0.f, total = 0.f;
-    for (auto& kv : pool_) {
-      size_t busy = 0;
-      for (const auto& c : kv.second) busy += c.use_count() > 1 ? 1 : 0;
-      used += BytesToMegaBytes((float)(kv.first * (int64_t)busy));
-      total += BytesToMegaBytes((float)(kv.first * (int64_t)kv.second.size()));
-    }
-    return {used, total};
-  }
 
   Device device_;
-  int64_t pool_bytes_ = 0;
-  int64_t max_pool_size_ = 0;  // 0 = no limit
-  std::shared_ptr<DeviceAPI> api_;
-  std::mutex mu_;
-  std::unordered_map<int64_t, std::list<std::shared_ptr<Memory>>> pool_;
+  int64_t size_limit_ = 0;  // bytes the pool may hold, idle and leased together; 0 = no limit
+  std::shared_ptr<Ledger> ledger_;
 };
 
 const bool kNoPoolRegistered = MemoryPool::RegisterMaker("no_pool", NoPool::make);

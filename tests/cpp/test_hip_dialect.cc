@@ -331,6 +331,25 @@ int main() {
     memory_pool::ResetPool(cpu);
     EXPECT(Memory::GetPool(cpu)->GetName() == "no_pool");
     EXPECT(Raises([&] { memory_pool::InitPool(cpu, "nope"); }).find("raf.memory_pool._make.nope") != std::string::npos);
+    // a size limit: what the pool holds, idle and in use together, may not outgrow it; the idle
+    // blocks go back to the device when a new block would
+    setenv("RAF_MEMORY_POOL_SIZE_LIMIT", "20000", 1);
+    memory_pool::InitPool(cpu, "page_unit_pool");
+    unsetenv("RAF_MEMORY_POOL_SIZE_LIMIT");
+    {
+      auto a = Memory::Alloc(cpu, 8192);
+      a.reset();
+      auto held = Memory::GetPoolSize(cpu);
+      EXPECT(held.first == 0.f && held.second == 8192.f / 1048576.f);  // kept for the next request
+      auto b = Memory::Alloc(cpu, 12288);  // 8192 idle + 12288 > 20000: the idle block is released
+      held = Memory::GetPoolSize(cpu);
+      EXPECT(held.first == 12288.f / 1048576.f && held.second == held.first);
+      auto c = Memory::Alloc(cpu, 4096);   // within the limit again: nothing to release, nothing refused
+      held = Memory::GetPoolSize(cpu);
+      EXPECT(held.second == 16384.f / 1048576.f);
+      memory_pool::RemovePool(cpu);        // b and c outlive their pool and free themselves
+      std::memset(b->data, 1, 12288);
+    }
     memory_pool::InitPool(cpu, "page_unit_pool");
     if (DeviceAPI_count_is_zero())  // the rocm pool makes its device current: a raf::Error without a GPU
       EXPECT(Raises([] { Memory::GetPool(Device(DevType::kROCM(), 0)); }).find("hipSetDevice") != std::string::npos);
