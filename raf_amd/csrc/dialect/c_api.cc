@@ -155,6 +155,17 @@ struct StreamPool {
     return s;
   }
 };
+// The two events that order a served stream against the compute stream, made once per thread and
+// device (an event may be recorded again as soon as the wait on its previous record has been
+// enqueued; two threads must not share one).  They live as long as the process.
+std::pair<void*, void*> OrderingEvents(const Device& dev, device_api::DeviceAPI* api) {
+  thread_local std::map<std::pair<int, int>, std::pair<void*, void*>> events;
+  auto& ev = events[{(int)dev.device_type(), dev.device_id()}];
+  constexpr uint32_t kNoTiming = 0x2;  // hipEventDisableTiming: ordering only
+  if (!ev.first) ev.first = api->CreateEvent(dev, kNoTiming);
+  if (!ev.second) ev.second = api->CreateEvent(dev, kNoTiming);
+  return ev;
+}
 StreamPool& Streams() {
   static StreamPool* pool = new StreamPool();  // streams live as long as the process
   return *pool;
@@ -165,6 +176,7 @@ struct StreamBinding {
   std::shared_ptr<device_api::DeviceAPI> api;
   Device device;
   void* compute = nullptr;
+  void* after = nullptr;
   std::vector<void*> served;
   StreamBinding(OpEnv* env, const Device& dev, void* compute_stream)
       : reqs(env->stream_requests()), device(dev), compute(compute_stream) {
@@ -173,23 +185,21 @@ struct StreamBinding {
       return;
     }
     api = device_api::DeviceAPI::Get(dev.device_type());
-    void* ev = api->CreateEvent(dev, 0);
-    api->EventRecordOnStream(ev, compute);
+    const auto events = OrderingEvents(dev, api.get());
+    after = events.second;
+    api->EventRecordOnStream(events.first, compute);
     for (const auto& r : reqs) {
       void* s = Streams().Get(r.device, r.tag_idx, r.stream_idx);
-      api->StreamWaitEvent(s, ev);
+      api->StreamWaitEvent(s, events.first);
       *r.dest = s;
       served.push_back(s);
     }
-    api->FreeEvent(dev, ev);
   }
   // Ordering the compute stream behind the served streams can fail; call it on the normal path.
   void Finish() {
     for (void* s : served) {
-      void* ev = api->CreateEvent(device, 0);
-      api->EventRecordOnStream(ev, s);
-      api->StreamWaitEvent(compute, ev);
-      api->FreeEvent(device, ev);
+      api->EventRecordOnStream(after, s);
+      api->StreamWaitEvent(compute, after);
     }
     served.clear();
   }
