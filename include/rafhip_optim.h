@@ -233,7 +233,13 @@ int64_t rafhip_lans_plan_total_elements(const rafhip_lans_plan* plan);
  * recently used through pinned staging memory of its own, without waiting for the device.  An
  * executor whose gradients alternate between two allocations (the reference's VM allocates them
  * per iteration, src/impl/vm/vm.cc:1099-1105) therefore stops uploading after two steps.  This
- * counts the uploads made so far (-1 on NULL). */
+ * counts the uploads made so far (-1 on NULL).
+ * A step made while its stream is being captured into a HIP graph leaves nodes that read one of
+ * the tables at every replay; that table is held from then on and never given to other pointers,
+ * so replays keep updating the tensors they were captured with.  A plan can thus serve up to
+ * RAFHIP_TABLE_SLOTS captured pointer sets; once all tables are held, a step with pointers that
+ * match none of them returns RAFHIP_ERR_UNSUPPORTED (use another plan).  The same holds for the
+ * tables of the multi-tensor SGD and fuse / defuse plans. */
 #define RAFHIP_TABLE_SLOTS 4
 int64_t rafhip_lans_plan_table_uploads(const rafhip_lans_plan* plan);
 

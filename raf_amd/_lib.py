@@ -30,6 +30,7 @@ RAFHIP_F64 = 3
 
 RAFHIP_LANS_PHASED = 0
 RAFHIP_LANS_PIPELINED = 1
+RAFHIP_TABLE_SLOTS = 4  # device pointer tables per plan
 RAFHIP_LANS_STATIC_SCRATCH_BYTES = 8 * 1024 * 1024
 
 

@@ -11,6 +11,12 @@
 // waits only for the upload that used the same slot kSlots uploads ago, i.e. in practice never
 // (it can run kSlots - 1 steps ahead of the device even when the pointers change at every call).
 //
+// Stream capture: a call made while its stream is being captured into a graph leaves kernel nodes
+// that read a slot's device table (and, if the records were new, a copy node that reads the slot's
+// staging buffer) at every replay.  Such a slot is held from then on: it is never chosen for other
+// records, so a graph keeps finding the pointers it was captured with for as long as the plan
+// lives.  When every slot is held a call with yet other records is refused.
+//
 // Rec must be trivially copyable with every byte initialised (records are compared with memcmp).
 #pragma once
 #include <hip/hip_runtime.h>
@@ -19,6 +25,8 @@
 #include <cstring>
 #include <type_traits>
 #include <vector>
+
+#include "status.h"
 
 namespace rafhip {
 
@@ -71,6 +79,7 @@ class RecordTables {
     staging_ = nullptr;
     device_ = nullptr;
     current_ = -1;
+    refused_ = false;
     used_once_ = false;
     last_stream_ = nullptr;
     clock_ = 0;
@@ -94,14 +103,17 @@ class RecordTables {
       current_ = hit;
       return use(slots_[hit], s, table_out);
     }
-    int victim = 0;
+    int victim = -1;
     for (int k = 0; k < kSlots; ++k) {
+      if (slots_[k].held) continue;
       if (!slots_[k].valid) {
         victim = k;
         break;
       }
-      if (slots_[k].last_use < slots_[victim].last_use) victim = k;
+      if (victim < 0 || slots_[k].last_use < slots_[victim].last_use) victim = k;
     }
+    refused_ = victim < 0;
+    if (refused_) return hipErrorNotSupported;
     Slot& sl = slots_[victim];
     if (sl.valid) {
       // The slot's previous upload may still be reading its staging buffer.
@@ -113,7 +125,9 @@ class RecordTables {
     if (e != hipSuccess) return e;
     std::memcpy(sl.staging, recs.data(), bytes);
     e = hipMemcpyAsync(sl.device, sl.staging, bytes, hipMemcpyHostToDevice, s);
-    if (e == hipSuccess) e = hipEventRecord(sl.staging_free, s);
+    // Under capture the copy is a graph node, not an upload in flight: there is nothing to wait
+    // for, and the slot (held now) is not written again.
+    if (e == hipSuccess && !sl.held) e = hipEventRecord(sl.staging_free, s);
     if (e != hipSuccess) return e;
     sl.sent.swap(recs);
     sl.valid = true;
@@ -133,6 +147,8 @@ class RecordTables {
 
   // Uploads made so far (what a caller with steady pointers expects to stop growing).
   int64_t uploads() const { return uploads_; }
+  // Whether the last sync() failed because every slot is held by a captured graph.
+  bool refused() const { return refused_; }
 
  private:
   struct Slot {
@@ -141,6 +157,7 @@ class RecordTables {
     hipEvent_t staging_free = nullptr;   // recorded after the slot's last upload was enqueued
     std::vector<Rec> sent;               // what the device table holds
     bool valid = false;
+    bool held = false;                   // read by a captured graph: keeps its records for good
     uint64_t last_use = 0;
   };
 
@@ -149,24 +166,34 @@ class RecordTables {
   // the uploads, and behind the kernels that read a table or wrote the caller's workspace.  The
   // calls of one plan thus form a single line however the caller moves between streams (one step
   // at a time per plan is the contract; this makes it hold on the device too).  A stream under
-  // graph capture is left alone (events of other streams cannot be recorded into it): capture
-  // after a warm-up call on that stream has completed.
+  // graph capture is left alone (events of other streams cannot be recorded into it; the graph's
+  // launches are ordered by whoever replays it) and the slot it reads becomes a held one.
   hipError_t use(Slot& sl, hipStream_t s, const Rec** table_out) {
     sl.last_use = ++clock_;
     *table_out = sl.device;
+    if (capturing(s)) {
+      sl.held = true;
+      return hipSuccess;
+    }
     if (!used_once_) {
       used_once_ = true;
       last_stream_ = s;
       return hipSuccess;
     }
     if (s == last_stream_) return hipSuccess;
-    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(s, &capturing) != hipSuccess) (void)hipGetLastError();
-    if (capturing != hipStreamCaptureStatusNone) return hipSuccess;
     hipError_t e = order_behind(last_stream_, s);
     if (e != hipSuccess) return e;
     last_stream_ = s;
     return hipSuccess;
+  }
+
+  static bool capturing(hipStream_t s) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &status) != hipSuccess) {
+      (void)hipGetLastError();  // e.g. the legacy default stream while another stream captures
+      return false;
+    }
+    return status != hipStreamCaptureStatusNone;
   }
 
   // Everything enqueued on `before` so far happens before what is enqueued on `s` from now on.
@@ -187,9 +214,24 @@ class RecordTables {
   hipStream_t last_stream_ = nullptr;  // the stream of the plan's last call
   bool used_once_ = false;
   int current_ = -1;               // the slot of the last sync()
+  bool refused_ = false;
   uint64_t clock_ = 0;
   int64_t uploads_ = 0;
 };
+
+// sync() for the entry points: a HIP failure or a refusal becomes a status code with a message.
+template <typename Rec>
+int sync_tables(const char* who, RecordTables<Rec>& tables, std::vector<Rec>& recs, hipStream_t s,
+                const Rec** table_out) {
+  const hipError_t e = tables.sync(recs, s, table_out);
+  if (e == hipSuccess) return RAFHIP_OK;
+  if (tables.refused())
+    return fail(RAFHIP_ERR_UNSUPPORTED,
+                "%s: all %d pointer tables of the plan are held by captured graphs; these pointers are "
+                "new to it (use another plan for them)",
+                who, RecordTables<Rec>::kSlots);
+  return fail(RAFHIP_ERR_HIP, "%s: sending the pointer table failed: %s", who, hipGetErrorString(e));
+}
 
 // HIP refuses a launch of 2^32 threads or more; with the 256-thread workgroups used throughout
 // that is a grid of 2^24.  One-workgroup-per-item launches are capped here and stride over the rest.

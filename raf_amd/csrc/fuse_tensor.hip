@@ -157,7 +157,7 @@ int run(rafhip_fuse_plan* plan, const char* what, void* const* parts, void* flat
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
     const Segment* table = nullptr;
-    RAFHIP_HIP_TRY(plan->tables.sync(segs, s, &table));
+    if (int st = sync_tables(what, plan->tables, segs, s, &table)) return st;
     // One workgroup per item; the kernel strides over what a launch cannot hold.
     const unsigned grid = (unsigned)(plan->n_items < kMaxGridBlocks ? plan->n_items : kMaxGridBlocks);
     auto go = [&](auto kernel) {

@@ -847,7 +847,7 @@ int lans_step_impl(rafhip_lans_plan* plan, const void* const* g, float* const* w
     if (int st = build_records(who, plan, g, w, m, v, p, p_dtype, plan->recs)) return st;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const TensorRec* table = nullptr;
-    RAFHIP_HIP_TRY(plan->tensors.sync(plan->recs, s, &table));
+    if (int st = sync_tables(who, plan->tensors, plan->recs, s, &table)) return st;
     plan->bound_on_device = false;  // whatever was bound, the table used last now follows this call
     return launch_step(who, plan, table, p_dtype, step_dev, step_host, hp, workspace, workspace_bytes, s);
   });
@@ -891,7 +891,7 @@ int rafhip_lans_step_bound(rafhip_lans_plan* plan, const float* step_dev, int32_
       RAFHIP_HIP_TRY(plan->tensors.follow(s, &table));  // nothing to build, compare or send
     } else {
       plan->recs = plan->bound;  // same size: a copy, no allocation
-      RAFHIP_HIP_TRY(plan->tensors.sync(plan->recs, s, &table));
+      if (int st = sync_tables(who, plan->tensors, plan->recs, s, &table)) return st;
       plan->bound_on_device = true;
     }
     return launch_step(who, plan, table, plan->bound_p_dtype, step_dev, step_host, hp, workspace,

@@ -517,7 +517,7 @@ extern "C" int rafhip_sgd_multi_step(rafhip_sgd_plan* plan, float* const* x, con
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
     const SgdRec* table = nullptr;
-    RAFHIP_HIP_TRY(plan->tables.sync(recs, s, &table));
+    if (int st = sync_tables("rafhip_sgd_multi_step", plan->tables, recs, s, &table)) return st;
     // One rounding double -> fp32, as for the single-tensor op.
     const float lr32 = static_cast<float>(learning_rate);
     const float mu32 = static_cast<float>(mu);

@@ -57,6 +57,8 @@ def test_status_and_dtype_codes_match_the_header(native_libs):
     assert len([k for k in codes if k.startswith("RAFHIP_ERR_")]) == 6
     for name, value in codes.items():
         assert getattr(native_libs, name) == int(value), name
+    slots = re.search(r"#define\s+RAFHIP_TABLE_SLOTS\s+(\d+)", text)
+    assert slots and native_libs.RAFHIP_TABLE_SLOTS == int(slots.group(1))
 
 
 def test_abi_version_and_struct_layout(native_libs):

@@ -437,6 +437,84 @@ def test_step_can_be_captured_in_a_hip_graph(native_libs, schedule):
     plan.close()
 
 
+def test_a_captured_step_keeps_its_pointer_table(native_libs):
+    """A graph replays kernels that read one of the plan's device tables.  The table a step was
+    captured with is held: eager steps with five other gradient lists afterwards (more than the
+    plan has tables) must not overwrite it, so a replay still updates the captured tensors with the
+    captured gradients; a capture whose pointers are new to the plan (no warm-up with them) sends
+    them inside the graph and is held likewise; and once every table is held by a graph, pointers
+    the plan has never seen are refused instead of evicting one."""
+    from raf_amd import kernels
+    from raf_amd._lib import RAFHIP_TABLE_SLOTS
+
+    sizes = [70001, 5, 8192, 300000, 1]
+    hp = LansHParams()
+    g, w, m, v = lans_inputs(sizes, cfg=87)
+    others = [lans_inputs(sizes, cfg=88 + k)[0] for k in range(RAFHIP_TABLE_SLOTS + 1)]
+    tg, tw, tm, tv = _to_dev(g), _to_dev(w), _to_dev(m), _to_dev(v)
+    tothers = [_to_dev(o) for o in others]
+    plan = kernels.LansPlan(sizes, torch.float32, DEV)
+    step = torch.full((), 1.0, device=DEV)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        plan.step(tg, tw, tm, tv, step, _khp(hp))  # warm-up: the table goes out, the workspace exists
+        step.add_(1.0)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        plan.step(tg, tw, tm, tv, step, _khp(hp))
+        step.add_(1.0)
+    torch.cuda.synchronize()
+    ow, om, ov, _ = lans_f64.lans_step(g, w, m, v, 1, hp)      # the warm-up; a capture runs nothing
+    n_steps = 1
+    uploads = plan.table_uploads
+    for k, other in enumerate(tothers):                       # five other lists: every free table is reused
+        plan.step(other, tw, tm, tv, step, _khp(hp))
+        step.add_(1.0)
+        n_steps += 1
+        ow, om, ov, _ = lans_f64.lans_step(others[k], ow, om, ov, n_steps, hp)
+    assert plan.table_uploads == uploads + len(tothers)
+    torch.cuda.synchronize()
+    for _ in range(2):
+        graph.replay()                                         # still the first gradient list
+        n_steps += 1
+        ow, om, ov, _ = lans_f64.lans_step(g, ow, om, ov, n_steps, hp)
+    torch.cuda.synchronize()
+    plan.read_norms()
+    _assert_close([t.cpu().numpy() for t in tw], ow, 1e-4, "w")
+    _assert_close([t.cpu().numpy() for t in tv], ov, 1e-4, "v")
+
+    # captures with pointers the plan has not seen: sent inside the graph, held, replayable
+    graphs = [graph]
+    for k in range(RAFHIP_TABLE_SLOTS - 1):
+        fresh = [t.clone() for t in tothers[k]]
+        tothers.append(fresh)  # keep alive
+        gk = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gk):
+            plan.step(fresh, tw, tm, tv, step, _khp(hp))
+            step.add_(1.0)
+        graphs.append((gk, k))
+    torch.cuda.synchronize()
+    for gk, k in graphs[1:]:
+        gk.replay()
+        n_steps += 1
+        ow, om, ov, _ = lans_f64.lans_step(others[k], ow, om, ov, n_steps, hp)
+    torch.cuda.synchronize()
+    _assert_close([t.cpu().numpy() for t in tw], ow, 1e-4, "w")
+    # every table is held now: a list the plan does not know is refused, a held one still runs
+    with pytest.raises(RuntimeError, match="held by captured graphs"):
+        plan.step(tothers[RAFHIP_TABLE_SLOTS], tw, tm, tv, step, _khp(hp))
+    plan.step(tg, tw, tm, tv, step, _khp(hp))
+    n_steps += 1
+    ow, om, ov, _ = lans_f64.lans_step(g, ow, om, ov, n_steps, hp)
+    torch.cuda.synchronize()
+    _assert_close([t.cpu().numpy() for t in tw], ow, 1e-4, "w")
+    _assert_close([t.cpu().numpy() for t in tm], om, 1e-4, "m")
+    plan.close()
+
+
 def test_same_tensors_on_another_stream(native_libs):
     """The pointer table is uploaded on the first call's stream; a second call with the same tensors
     on another stream must still see it (the library orders the new stream behind the upload)."""
