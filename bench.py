@@ -11,15 +11,24 @@ Inputs are synthetic (seeded, generated on the GPU) and resident in HBM before t
 Prints ONE JSON line.  Its top-level fields are the headline workload's; `value` is algorithmic
 bytes per step (the three-pass model: 46 B per element with fp16 gradients, 52 B with fp32) divided
 by the wall time per step.  With the default `--workload all` the line also carries
-  "configs"  every benchmark configuration (SGD on one tensor; LANS on the BERT-base, BERT-large,
-             2000-small-tensor and GPT-2-1.5B lists): step time, the dominant kernel's time from
-             HIP events, and its fraction of the 8 TB/s peak by the algorithmic and by the
-             compulsory bytes; for BERT-large and the small-tensor list also the step time through
-             the operator front end (`raf_amd.op.lans`: dialect dispatch -> OpEnv -> Execute);
-  "parity"   a check of the very buffers that were timed, after the timed region, against the CPU
-             oracle: SGD bit for bit, LANS w, m, v of whole tensors of the timed list by the strict
-             per-element relative error, the count of elements over the tolerance, and the error
-             relative to max(|reference|, |old weight|).
+  "configs"    every benchmark configuration (SGD on one tensor; LANS on the BERT-base, BERT-large,
+               2000-small-tensor and GPT-2-1.5B lists): step time, the dominant kernel and its time
+               from HIP events, its fraction of the 8 TB/s peak by the algorithmic (`frac`) and by
+               the compulsory bytes (`frac_c`), the bytes per launch rocprofv3 measured (`traffic`);
+  "entries"    for BERT-large and the small-tensor list, ms per step through each way into the
+               step: the C ABI, the operator front end (`raf_amd.op.lans`: dialect dispatch ->
+               OpEnv -> Execute) with a list handle, a plain list, new gradient objects every step,
+               and the VM's calling pattern (a new tuple every step, gradients at alternating
+               addresses), each with its difference to the C ABI in per cent;
+  "neighbours" multi-tensor SGD, the traced optimizers after the dialect's graph rewrites, the
+               mixed-precision step, l2norm, fuse and defuse: ms per step and fraction of the peak;
+  "yardsticks" GB/s of plain torch streaming kernels on the same GPU in the same process (write,
+               read+write, copy beyond the Infinity Cache; read+write and write inside it, with
+               zeros and with other values), beside which the fractions above can be read;
+  "parity"     a check of the very buffers that were timed, after the timed region, against the
+               CPU oracle: SGD bit for bit, LANS w, m, v of whole tensors of the timed list by the
+               strict per-element relative error (`max_rel`), the count of elements over the
+               tolerance (`over_tol`) and of elements not bit-equal (`ne`).
 """
 from __future__ import annotations
 
@@ -142,6 +151,7 @@ def workloads():
         # a plain device-to-device copy of known size: the yardstick that rocprofv3's FETCH_SIZE /
         # WRITE_SIZE counters are scaled by when HBM traffic is measured
         "copy_1gib": dict(kind="copy", nbytes=1 << 30),
+        "stream_yardsticks": dict(kind="yardsticks"),
     }
 
 
@@ -723,6 +733,48 @@ def bench_copy(name, wl, args):
             "roofline": roofline_obj(name, "torch copy", moved, dev_ms)}
 
 
+def stream_yardsticks(steps=30, warmup=5):
+    """What plain streaming kernels of the framework underneath (torch's element-wise kernels and
+    its device-to-device copy, not this library's code) reach on the same GPU in the same process:
+    GB/s by the bytes each one reads plus writes.  They are the rates the memory system gives a
+    read-only, a write-only and a read-and-write stream, beyond the Infinity Cache (1 GiB per
+    array) and inside it (180 MiB in all, the footprint of the 2000-tensor list), and they show
+    that a cache-resident stream of zeros is written faster than one of other values."""
+    import torch
+
+    dev = torch.device("cuda:0")
+
+    def rate(fn, nbytes):
+        for _ in range(warmup):
+            fn()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        start.record()
+        for _ in range(steps):
+            fn()
+        stop.record()
+        torch.cuda.synchronize()
+        return round(nbytes * steps / (start.elapsed_time(stop) * 1e-3) / 1e9)
+
+    out = {}
+    n = (1 << 30) // 4
+    src, dst = torch.randn(n, device=dev), torch.empty(n, device=dev)
+    out["torch_sum_1gib"] = rate(lambda: torch.sum(src), 4 * n)         # torch's own reduction: reads only
+    out["write_1gib"] = rate(lambda: dst.fill_(1.2345), 4 * n)
+    out["read_write_1gib"] = rate(lambda: torch.mul(src, 1.5, out=dst), 8 * n)
+    out["copy_1gib"] = rate(lambda: dst.copy_(src), 8 * n)
+    del src, dst
+    n = (90 << 20) // 4                                                   # 90 MiB + 90 MiB: cache-resident
+    src, dst = torch.randn(n, device=dev), torch.empty(n, device=dev)
+    zeros = torch.zeros(n, device=dev)
+    out["cached_read_write"] = rate(lambda: torch.mul(src, 1.5, out=dst), 8 * n)
+    out["cached_read_write_zeros"] = rate(lambda: torch.mul(zeros, 1.5, out=dst), 8 * n)
+    out["cached_write"] = rate(lambda: dst.fill_(1.2345), 4 * n)
+    out["cached_write_zeros"] = rate(lambda: dst.fill_(0.0), 4 * n)
+    out["unit"] = "GB/s"
+    return out
+
+
 def bench_traced_sgd(name, wl, args):
     """One step = the optimizer part of the reference's traced SGD optimizer over the whole model
     (per parameter: add(multiply(momentum, v), dx, out=v), subtract(w, multiply(lr, new_v), out=w)),
@@ -914,6 +966,8 @@ def run_suite(table, args):
         neighbours[name] = {"ms": line["ms_per_step"], "frac": line["roofline"]["frac"]}
         release()
     out["neighbours"] = neighbours
+    out["yardsticks"] = stream_yardsticks()
+    release()
     parity["ok"] = all(p is None or p.get("ok", False) for p in parity.values())
     out["parity"] = parity
     return out
@@ -967,6 +1021,8 @@ def main():
             out = bench_lans(args.workload, wl, args, entry=args.entry, parity=not args.no_parity)
         elif wl["kind"] == "sgd":
             out = bench_sgd(args.workload, wl, args, parity=not args.no_parity)
+        elif wl["kind"] == "yardsticks":
+            out = {"workload": args.workload, **stream_yardsticks(args.steps, args.warmup)}
         else:
             fn = {"copy": bench_copy, "l2norm": bench_l2norm, "fuse": bench_fuse, "sgd_multi": bench_sgd_multi,
                   "traced_sgd": bench_traced_sgd, "traced_lans": bench_traced_lans}[wl["kind"]]
