@@ -24,6 +24,9 @@
 //       every tensor outside the range still lives at its recorded address; False, and nothing
 //       written, otherwise
 //
+//   unreferenced(tensors, first, end) -> bool
+//       whether the list holds the only Python reference to every object in [first, end): nobody
+//       can pass those objects again
 //   grads(params) -> (list, missing)
 //       the `.grad` of every parameter (None where there is none) and how many are None
 //
@@ -202,6 +205,20 @@ PyObject* rebind_impl(PyObject* args) {
   Py_RETURN_TRUE;
 }
 
+PyObject* unreferenced_impl(PyObject* args) {
+  PyObject* list;
+  long long first, end;
+  if (!PyArg_ParseTuple(args, "OLL", &list, &first, &end)) return nullptr;
+  if (!list_arg(list, "tensors")) return nullptr;
+  if (first < 0 || end < first || end > (long long)PyList_GET_SIZE(list)) {
+    PyErr_SetString(PyExc_IndexError, "range outside the list");
+    return nullptr;
+  }
+  for (Py_ssize_t i = (Py_ssize_t)first; i < (Py_ssize_t)end; ++i)
+    if (Py_REFCNT(PyList_GET_ITEM(list, i)) != 1) Py_RETURN_FALSE;
+  Py_RETURN_TRUE;
+}
+
 PyObject* grads_impl(PyObject* args) {
   PyObject* list;
   if (!PyArg_ParseTuple(args, "O", &list)) return nullptr;
@@ -241,6 +258,7 @@ PyMethodDef kMethods[] = {
     {"same_storage", guarded<same_storage_impl>, METH_VARARGS, "whether the tensors' data pointers equal the recorded ones"},
     {"diff_range", guarded<diff_range_impl>, METH_VARARGS, "index range outside which two lists hold the same objects"},
     {"rebind", guarded<rebind_impl>, METH_VARARGS, "bring a described list up to date with tensors that replace a range of it"},
+    {"unreferenced", guarded<unreferenced_impl>, METH_VARARGS, "whether the list holds the only reference to a range of its objects"},
     {"grads", guarded<grads_impl>, METH_VARARGS, "the .grad of every parameter and the number of missing ones"},
     {"signature", guarded<signature_impl>, METH_VARARGS, "dtype, device and shape of every descriptor as bytes"},
     {nullptr, nullptr, 0, nullptr}};

@@ -151,6 +151,7 @@ class TensorList:
         self.track = bool(track)
         self.rebuilds = 0
         self.rebinds = 0
+        self._volatile = None  # the (first, end) stretch whose tensors are new at every call, once known
         self._handle = c_void_p(None)
         self._build(_share)
 
@@ -242,6 +243,15 @@ class TensorList:
         self.rebinds += 1
         return True
 
+    def _release_volatile(self) -> None:
+        """After a call: lets go of the tensors in the stretch that is new at every call (the
+        gradients of the step just enqueued).  Holding them until the next call would keep a whole
+        generation of gradients allocated through the next forward and backward pass; the kernels
+        already enqueued are ordered in front of any reuse of that memory by the stream."""
+        if self._volatile is not None:
+            first, end = self._volatile
+            self._tensors[first:end] = [None] * (end - first)
+
     def __len__(self):
         return len(self._tensors)
 
@@ -266,8 +276,12 @@ def _tensor_list(tensors) -> TensorList:
     """The handle behind a ``tensor_list`` argument.  A ``TensorList`` is used as it is (checked
     against its tensors unless it was made with ``track=False``).  A plain sequence is looked up
     among the handles made for recent calls by the identity of its elements -- a training loop
-    passes the same tensor objects every step -- and when only a stretch of it differs (fresh
-    gradient tensors, say) the new handle shares the rest with the old one."""
+    passes the same tensor objects every step.  When only a stretch of it differs from a recent
+    list, what happens depends on whether the old tensors of that stretch can come back: if
+    nothing but the handle refers to them any more (gradients that autograd allocates per
+    iteration), the handle takes the new ones over in place and stops holding on to that stretch
+    between calls; if the caller still has them (it alternates between lists), a new handle shares
+    the rest with the old one, and once there are eight the oldest is taken over."""
     if isinstance(tensors, TensorList):
         return tensors.refresh() if tensors.track else tensors
     lst = tensors if type(tensors) is list else list(tensors)
@@ -284,20 +298,38 @@ def _tensor_list(tensors) -> TensorList:
             return h.refresh()
         if 2 * (end - first) <= len(lst) and (nearest is None or end - first < nearest[2] - nearest[1]):
             nearest = (h, first, end)
-    if nearest is not None and len(_recent_lists) == _recent_lists.maxlen:
-        # Every step brings tensors never seen before (gradients allocated per iteration): rather
-        # than make handle after handle, the one used longest ago takes the new tensors over.
-        # Callers that alternate between a few lists never get here: theirs are all found above.
-        for h in reversed(_recent_lists):
-            if len(h) != len(lst):
-                continue
-            first, end = glue.diff_range(lst, h._tensors)
-            if 2 * (end - first) <= len(lst) and h._rebind(lst, first, end):
-                _recent_lists.remove(h)
-                _recent_lists.appendleft(h)
+
+    def take_over(h, first, end):
+        if not h._rebind(lst, first, end):
+            return False
+        if h is not _recent_lists[0]:
+            _recent_lists.remove(h)
+            _recent_lists.appendleft(h)
+        return True
+
+    if nearest is not None:
+        h, first, end = nearest
+        # Tensors that are new at every call (gradients allocated per iteration, torch's default):
+        # when nothing but the handle still refers to the ones it holds in the stretch, nobody can
+        # pass them again, so the handle takes the new ones over in place -- and from then on lets
+        # go of that stretch after every call instead of keeping a generation of gradients alive.
+        if h._volatile is not None or glue.unreferenced(h._tensors, first, end):
+            if take_over(h, first, end):
+                lo, hi = h._volatile or (first, end)
+                h._volatile = (min(lo, first), max(hi, end))
                 return h
-            break
-    if nearest is not None and nearest[0].current():
+        elif len(_recent_lists) == _recent_lists.maxlen:
+            # The caller keeps the old tensors (it may alternate between a few lists, which are all
+            # found above) but brings new ones again and again: rather than make handle after
+            # handle, the one used longest ago takes the new tensors over.
+            for old in reversed(_recent_lists):
+                if len(old) != len(lst) or old._volatile is not None:
+                    continue
+                first2, end2 = glue.diff_range(lst, old._tensors)
+                if 2 * (end2 - first2) <= len(lst) and take_over(old, first2, end2):
+                    return old
+                break
+    if nearest is not None and nearest[0]._volatile is None and nearest[0].current():
         h = nearest[0].replaced(nearest[1], lst[nearest[1]:nearest[2]])
     else:
         h = TensorList(lst)
@@ -515,6 +547,7 @@ def _sgd_multi(mixed, tensor_list, learning_rate, mu):
     if n:
         env.set_learning_rate(float(learning_rate))
     check_raf(lib.rafhip_raf_sgd_multi_execute_tuple(env.handle, tl._handle, _stream(tl[0]) if n else None, _as_vm))
+    tl._release_volatile()
     return tensor_list
 
 
@@ -564,6 +597,7 @@ def _lans(op_name, tensor_list, step, learning_rate, beta1, beta2, eps, bias_cor
     ws = _workspace(env, tl[0], stream) if env.workspace_bytes > 0 else None
     check_raf(lib.rafhip_raf_lans_execute_tuple(env.handle, tl._handle, dstep, ws.data if ws else None,
                                                 env.workspace_bytes, stream, _as_vm))
+    tl._release_volatile()
     return tensor_list
 
 

@@ -176,3 +176,42 @@ def test_gradients_allocated_anew_every_step(native_libs):
     assert sum(h.rebinds for h in op._recent_lists) == 4
     _check(tg + tw + tm + tv, n, ow, om, ov, tol=2e-5)
     op.clear_op_env_cache()
+
+
+def test_gradients_that_die_with_their_step_are_not_kept_alive(native_libs):
+    """The same, with the caller dropping each step's gradients after the call (what autograd with
+    `zero_grad(set_to_none=True)` amounts to): one handle takes every step's gradients over in
+    place and holds none of them once the call has returned; results against the oracle."""
+    import gc
+    import weakref
+
+    from raf_amd import op
+
+    hp = LansHParams()
+    g0, w, m, v = lans_inputs(SIZES, cfg=132)
+    n = len(SIZES)
+    op.clear_op_env_cache()
+    tw, tm, tv = _dev(w), _dev(m), _dev(v)
+    step = torch.zeros((), device=DEV)
+    ow, om, ov = w, m, v
+    for s in range(1, 7):
+        g = [(a * np.float32(1.0 + 0.25 * s)).astype(np.float32) for a in g0]
+        tg = _dev(g)
+        alive = weakref.ref(tg[0])
+        step.fill_(float(s))
+        op.lans(tg + tw + tm + tv, step, *_args(hp))
+        del tg
+        gc.collect()
+        if s == 1:
+            first_step = alive   # not known to be short-lived yet: kept until the next call shows it
+        else:
+            assert alive() is None, "the front end still holds the gradients of a finished call"
+            assert first_step() is None
+        ow, om, ov, _ = lans_f64.lans_step(g, ow, om, ov, s, hp)
+    torch.cuda.synchronize()
+    assert len(op._recent_lists) == 1 and op._recent_lists[0].rebinds == 5
+    assert len([k for k in op._env_cache if k[0] == "lans"]) == 1
+    for t in range(n):
+        assert max_rel_err(tw[t].cpu().numpy(), ow[t]) <= 2e-5
+        assert max_rel_err(tv[t].cpu().numpy(), ov[t]) <= 2e-5
+    op.clear_op_env_cache()

@@ -225,3 +225,44 @@ def test_grads_reads_every_parameters_gradient(native_libs):
         glue.grads([object()])
     with pytest.raises(TypeError):
         glue.grads(tuple(ps))
+
+
+def test_a_stretch_that_is_new_at_every_call_is_not_kept_alive(native_libs):
+    """Gradients that nobody holds after a step (autograd allocates new ones per iteration): one
+    handle serves every step, takes the new tensors over in place, and lets go of that stretch
+    after each call, so no generation of gradients outlives its step because of the front end."""
+    import gc
+    import weakref
+
+    from raf_amd import op
+
+    glue = native_libs.glue()
+    a = [torch.zeros(3), torch.zeros(3)]
+    assert glue.unreferenced([torch.zeros(3), a[0]], 0, 1) is True    # only the list holds item 0
+    assert glue.unreferenced([torch.zeros(3), a[0]], 0, 2) is False   # `a` holds item 1 as well
+    with pytest.raises(IndexError):
+        glue.unreferenced(a, 1, 3)
+
+    op.clear_op_env_cache()
+    state = [torch.zeros(3, 5) for _ in range(9)]
+    first = op._tensor_list([torch.zeros(3, 5) for _ in range(3)] + state)
+    first._release_volatile()                      # nothing is known to be volatile yet: a no-op
+    assert first[0] is not None and first._volatile is None
+    seen = []
+    for step in range(5):
+        g = [torch.full((3, 5), float(step)) for _ in range(3)]
+        seen.append(weakref.ref(g[0]))
+        h = op._tensor_list(g + state)
+        assert h is first and h._volatile == (0, 3) and h.rebinds == step + 1
+        assert h[0] is g[0] and h._ptrs[1] == g[1].data_ptr() and h._descs[2].data == g[2].data_ptr()
+        h._release_volatile()                      # what op.lans / op.sgd_multi do after Execute
+        assert h[0] is None and h[3] is state[0]
+        del g
+        gc.collect()
+        assert seen[-1]() is None                  # the step's gradients are gone with the step
+    assert len(op._recent_lists) == 1
+    # the persistent tensors are still tracked: a moved one makes the next call build a new handle
+    state[4].data = torch.ones(3, 5)
+    h2 = op._tensor_list([torch.zeros(3, 5) for _ in range(3)] + state)
+    assert h2 is not first and h2.current() and h2._ptrs[3 + 4] == state[4].data_ptr()
+    op.clear_op_env_cache()
