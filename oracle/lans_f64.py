@@ -121,7 +121,8 @@ def lans_directions(g, w, m, v, sc: LansScalars, hp: LansHParams, repeat: int = 
     """Stage 1 for one tensor; float64 in, float64 out.
     Returns (m1, v1, u_m, u_g, grad_norm).  ``repeat``: see lans_tensor_step."""
     gn = l2norm(g) * math.sqrt(repeat)
-    sg = g / (gn + sc.eps) if (hp.normalize_grad and gn != 0.0) else g
+    with np.errstate(invalid="ignore"):  # an overflowed gradient gives inf / inf = NaN, as on the device
+        sg = g / (gn + sc.eps) if (hp.normalize_grad and gn != 0.0) else g
     wp = w if sc.wd != 0.0 else np.zeros_like(w)
     if int(hp.mode) == 0:
         sg = sg + sc.wd * wp
