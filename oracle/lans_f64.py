@@ -129,13 +129,14 @@ def lans_directions(g, w, m, v, sc: LansScalars, hp: LansHParams, repeat: int = 
     m1 = m * sc.beta1 + sc.beta3 * sg
     v1 = v * sc.beta2 + sc.one_minus_beta2 * sg * sg
     den = np.sqrt(v1 / sc.bc2) + sc.eps
-    if int(hp.mode) == 0:
-        u_m = (m1 / sc.bc1) / den
-        u_g = sg / den
-    else:
-        sp = sc.wd * wp
-        u_m = (m1 / sc.bc1) / den + sp
-        u_g = sg / den + sp
+    with np.errstate(invalid="ignore", divide="ignore"):  # 0 / 0 (eps = 0) propagates NaN, as the rule says
+        if int(hp.mode) == 0:
+            u_m = (m1 / sc.bc1) / den
+            u_g = sg / den
+        else:
+            sp = sc.wd * wp
+            u_m = (m1 / sc.bc1) / den + sp
+            u_g = sg / den + sp
     return m1, v1, u_m, u_g, gn
 
 
